@@ -1,0 +1,255 @@
+"""Pins for the CPU oracle (oracle/sampling_oracle.c).
+
+The reference ships no golden vectors for this path (its scripts under DCNv4_op/scripts only
+compare two GPU ops live), so the oracle is pinned by what the mathematics fixes:
+  * agreement in fp64 with an independent torch grid_sample formulation, over strides,
+    dilations, paddings, offset_scale, remove_center, non-square kernels and images;
+  * closed forms (box sum, integer shifts, single-tap attention, uniform attention);
+  * exact zeros outside the image, linearity, padded-tail invariants;
+  * central finite differences of the oracle's own forward for every gradient, and torch
+    autograd through the grid_sample formulation.
+Each check is chosen so that a swapped x/y, a wrong tap order, a dropped offset_scale factor or
+a wrong sign in a bilinear derivative fails it.
+"""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import torch_core
+from tests.inputs import make_dcnv4_inputs, make_fda_inputs
+
+DCN_CASES = [
+    # B, H, W, G, D, kh, kw, sh, sw, ph, pw, dh, dw, remove_center, offset_scale, offset_range
+    (2, 7, 9, 2, 4, 3, 3, 1, 1, 1, 1, 1, 1, 0, 1.0, 2.0),
+    (1, 8, 6, 3, 2, 3, 3, 2, 2, 1, 1, 1, 1, 0, 0.5, 3.0),
+    (2, 9, 10, 2, 3, 3, 3, 1, 1, 2, 2, 2, 2, 0, 2.0, 1.5),
+    (1, 6, 7, 4, 2, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1.3, 2.5),
+    (1, 7, 8, 2, 2, 3, 3, 1, 2, 0, 1, 1, 1, 1, 1.0, 4.0),
+    (1, 9, 8, 1, 5, 1, 3, 1, 1, 0, 1, 1, 1, 0, 0.7, 2.0),   # kh != kw, pad_h != pad_w
+    (1, 10, 9, 2, 2, 3, 1, 2, 1, 2, 0, 2, 1, 0, 1.0, 2.0),  # kh != kw the other way, mixed stride/dilation
+    (1, 5, 5, 7, 1, 3, 3, 1, 1, 1, 1, 1, 1, 0, 1.0, 8.0),   # offsets mostly far outside
+]
+
+
+def _dcn_args(case):
+    B, H, W, G, D, kh, kw, sh, sw, ph, pw, dh, dw, rc, scale, rng = case
+    return (kh, kw, sh, sw, ph, pw, dh, dw, G, D, scale, rc)
+
+
+@pytest.mark.parametrize("case", DCN_CASES)
+@pytest.mark.parametrize("softmax", [False, True])
+def test_dcnv4_c_oracle_matches_grid_sample_formulation(oracle, case, softmax):
+    B, H, W, G, D, kh, kw, sh, sw, ph, pw, dh, dw, rc, scale, rng = case
+    value, om, go = make_dcnv4_inputs(B, H, W, G, D, kh, kw, sh, sw, ph, pw, dh, dw, rc, rng,
+                                      seed=11, dtype=torch.float64)
+    args = _dcn_args(case)
+    v = value.clone().requires_grad_(True)
+    o = om.clone().requires_grad_(True)
+    ref = torch_core.dcnv4_core_torch(v, o, *args, softmax=softmax)
+    ref.backward(go)
+    out = oracle.dcnv4_forward(value.numpy(), om.numpy(), *args, softmax=softmax)
+    gv, gom = oracle.dcnv4_backward(value.numpy(), om.numpy(), go.numpy(), *args, softmax=softmax)
+    np.testing.assert_allclose(out, ref.detach().numpy(), rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(gv, v.grad.numpy(), rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(gom, o.grad.numpy(), rtol=1e-10, atol=1e-11)
+    used = G * 3 * (kh * kw - rc)
+    assert np.all(gom[..., used:] == 0.0)          # padded tail keeps exact zeros
+
+
+def test_dcnv4_zero_offsets_unit_mask_is_box_sum(oracle):
+    B, H, W, G, D = 2, 9, 11, 3, 4
+    value, om, _ = make_dcnv4_inputs(B, H, W, G, D, seed=3, dtype=torch.float64)
+    K = 9
+    om.zero_()
+    body = om[..., : G * K * 3].reshape(B, H, W, G, K * 3)
+    body[..., 2 * K:] = 1.0
+    out = oracle.dcnv4_forward(value.numpy(), om.numpy(), 3, 3, 1, 1, 1, 1, 1, 1, G, D, 1.0)
+    box = F.avg_pool2d(value.permute(0, 3, 1, 2), 3, 1, 1, count_include_pad=True) * 9
+    np.testing.assert_allclose(out, box.permute(0, 2, 3, 1).numpy(), rtol=1e-12, atol=1e-12)
+
+
+def test_dcnv4_integer_offsets_are_shifted_copies_in_x_major_tap_order(oracle):
+    # one-hot mask on tap k with an integer offset (ox, oy) must copy value[y+ty+oy, x+tx+ox]
+    # where tap k = (tx index outer, ty index inner): a y-major order or swapped x/y fails.
+    B, H, W, G, D, K = 1, 8, 10, 1, 3, 9
+    value, om, _ = make_dcnv4_inputs(B, H, W, G, D, seed=5, dtype=torch.float64)
+    for k, (ox, oy) in [(1, (2, -1)), (3, (0, 0)), (5, (-2, 1)), (8, (1, 3))]:
+        om.zero_()
+        om[..., 2 * k] = ox
+        om[..., 2 * k + 1] = oy
+        om[..., 2 * K + k] = 1.0
+        out = oracle.dcnv4_forward(value.numpy(), om.numpy(), 3, 3, 1, 1, 1, 1, 1, 1, G, D, 1.0)
+        tx, ty = k // 3 - 1, k % 3 - 1
+        expect = np.zeros_like(out)
+        for y in range(H):
+            for x in range(W):
+                yy, xx = y + ty + oy, x + tx + ox
+                if 0 <= yy < H and 0 <= xx < W:
+                    expect[0, y, x] = value[0, yy, xx].numpy()
+        np.testing.assert_array_equal(out, expect)
+
+
+def test_dcnv4_offset_scale_multiplies_tap_and_offset(oracle):
+    # offset_scale 2 with a one-hot mask on the (+1,+1) tap and offset (0.5, 0) samples 3 px right
+    B, H, W, G, D, K = 1, 8, 8, 1, 2, 9
+    value, om, _ = make_dcnv4_inputs(B, H, W, G, D, seed=6, dtype=torch.float64)
+    om.zero_()
+    k = 8
+    om[..., 2 * k] = 0.5
+    om[..., 2 * K + k] = 1.0
+    out = oracle.dcnv4_forward(value.numpy(), om.numpy(), 3, 3, 1, 1, 1, 1, 1, 1, G, D, 2.0)
+    np.testing.assert_array_equal(out[0, 2, 1], value[0, 4, 4].numpy())   # x: 1 + 2*(1+0.5), y: 2 + 2*1
+
+
+def test_dcnv4_out_of_range_taps_give_exact_zeros(oracle):
+    B, H, W, G, D, K = 1, 5, 6, 2, 4, 9
+    value, om, go = make_dcnv4_inputs(B, H, W, G, D, seed=7, dtype=torch.float64)
+    body = om[..., : G * K * 3].reshape(B, H, W, G, K * 3)
+    body[..., : 2 * K] = 100.0
+    om[..., : G * K * 3] = body.reshape(B, H, W, -1)
+    args = (3, 3, 1, 1, 1, 1, 1, 1, G, D, 1.0, 0)
+    assert np.all(oracle.dcnv4_forward(value.numpy(), om.numpy(), *args) == 0.0)
+    gv, gom = oracle.dcnv4_backward(value.numpy(), om.numpy(), go.numpy(), *args)
+    assert np.all(gv == 0.0) and np.all(gom == 0.0)
+
+
+def test_dcnv4_is_linear_in_value_and_mask(oracle):
+    B, H, W, G, D, K = 1, 6, 7, 2, 3, 9
+    args = (3, 3, 1, 1, 1, 1, 1, 1, G, D, 1.0, 0)
+    v1, om, _ = make_dcnv4_inputs(B, H, W, G, D, seed=8, dtype=torch.float64)
+    v2, om2, _ = make_dcnv4_inputs(B, H, W, G, D, seed=9, dtype=torch.float64)
+    f = lambda v, o: oracle.dcnv4_forward(v.numpy(), o.numpy(), *args)
+    np.testing.assert_allclose(f(2.0 * v1 - 3.0 * v2, om), 2.0 * f(v1, om) - 3.0 * f(v2, om), rtol=1e-12, atol=1e-12)
+    oma, omb = om.clone(), om.clone()      # same offsets, different masks
+    ma = oma[..., : G * K * 3].reshape(B, H, W, G, K * 3)
+    mb = om2[..., : G * K * 3].reshape(B, H, W, G, K * 3)
+    mixed = ma.clone()
+    mixed[..., 2 * K:] = ma[..., 2 * K:] + mb[..., 2 * K:]
+    only_b = ma.clone()
+    only_b[..., 2 * K:] = mb[..., 2 * K:]
+    omb[..., : G * K * 3] = only_b.reshape(B, H, W, -1)
+    omm = om.clone()
+    omm[..., : G * K * 3] = mixed.reshape(B, H, W, -1)
+    np.testing.assert_allclose(f(v1, omm), f(v1, oma) + f(v1, omb), rtol=1e-12, atol=1e-12)
+
+
+def _central_differences(fn, x, go, idx, eps=1e-6):
+    out = []
+    flat = x.reshape(-1)
+    for i in idx:
+        old = flat[i]
+        flat[i] = old + eps
+        hi = fn()
+        flat[i] = old - eps
+        lo = fn()
+        flat[i] = old
+        out.append(float(((hi - lo) * go).sum() / (2 * eps)))
+    return np.array(out)
+
+
+@pytest.mark.parametrize("softmax", [False, True])
+def test_dcnv4_backward_matches_finite_differences(oracle, softmax):
+    B, H, W, G, D = 1, 5, 6, 2, 3
+    args = (3, 3, 1, 1, 1, 1, 1, 1, G, D, 1.7, 0)
+    value, om, go = make_dcnv4_inputs(B, H, W, G, D, offset_range=1.5, seed=21, dtype=torch.float64)
+    v, o, g = value.numpy().copy(), om.numpy().copy(), go.numpy()
+    gv, gom = oracle.dcnv4_backward(v, o, g, *args, softmax=softmax)
+    rng = np.random.default_rng(0)
+    fwd = lambda: oracle.dcnv4_forward(v, o, *args, softmax=softmax)
+    iv = rng.choice(v.size, 40, replace=False)
+    np.testing.assert_allclose(gv.reshape(-1)[iv], _central_differences(fwd, v, g, iv), rtol=1e-6, atol=1e-7)
+    used = np.arange(o.size).reshape(o.shape)[..., : G * 27].reshape(-1)
+    io = rng.choice(used, 80, replace=False)
+    np.testing.assert_allclose(gom.reshape(-1)[io], _central_differences(fwd, o, g, io), rtol=1e-5, atol=1e-6)
+
+
+def test_dcnv4_grad_mask_is_inner_product_with_each_tap_sample(oracle):
+    # grad_mask[k] = <grad_out, sample_k>; sample_k is the forward with a one-hot mask on k
+    B, H, W, G, D, K = 1, 4, 5, 1, 3, 9
+    args = (3, 3, 1, 1, 1, 1, 1, 1, G, D, 1.0, 0)
+    value, om, go = make_dcnv4_inputs(B, H, W, G, D, seed=22, dtype=torch.float64)
+    _, gom = oracle.dcnv4_backward(value.numpy(), om.numpy(), go.numpy(), *args)
+    for k in range(K):
+        one = om.clone()
+        one[..., 2 * K: 3 * K] = 0.0
+        one[..., 2 * K + k] = 1.0
+        sample = oracle.dcnv4_forward(value.numpy(), one.numpy(), *args)
+        np.testing.assert_allclose(gom[..., 2 * K + k], (sample * go.numpy()).sum(-1), rtol=1e-12, atol=1e-12)
+
+
+FDA_CASES = [
+    # B, shapes, G, D, K, Q, loc range
+    (2, [(6, 5), (3, 4)], 2, 4, 4, 7, (0.0, 1.0)),
+    (1, [(5, 7)], 3, 2, 8, 9, (-0.2, 1.2)),
+    (1, [(8, 8), (4, 4), (2, 2), (1, 1)], 2, 3, 4, None, (0.0, 1.0)),
+    (1, [(4, 6), (3, 3), (2, 5), (2, 2), (1, 3)], 1, 5, 4, 6, (-0.5, 1.5)),
+]
+
+
+@pytest.mark.parametrize("case", FDA_CASES)
+def test_fda_c_oracle_matches_grid_sample_formulation(oracle, case):
+    B, shapes, G, D, K, Q, (lo, hi) = case
+    value, shp, start, sla, go = make_fda_inputs(B, shapes, G, D, K, Q, seed=31, dtype=torch.float64,
+                                                 loc_lo=lo, loc_hi=hi)
+    v = value.clone().requires_grad_(True)
+    s = sla.clone().requires_grad_(True)
+    ref = torch_core.msda_core_torch(v, shapes, start.tolist(), s, K)
+    ref.backward(go)
+    out = oracle.flash_deform_attn_forward(value.numpy(), shp.numpy(), start.numpy(), sla.numpy(), K)
+    gv, gs = oracle.flash_deform_attn_backward(value.numpy(), shp.numpy(), start.numpy(), sla.numpy(),
+                                               go.numpy(), K)
+    np.testing.assert_allclose(out, ref.detach().numpy(), rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(gv, v.grad.numpy(), rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(gs, s.grad.numpy(), rtol=1e-10, atol=1e-11)
+
+
+def test_fda_pixel_centre_locations_with_uniform_logits_average_the_pixels(oracle):
+    # location ((x+0.5)/W, (y+0.5)/H) hits pixel (y,x) exactly; equal logits => plain mean of taps
+    H, W, G, D, K = 4, 5, 2, 3, 4
+    value, shp, start, sla, _ = make_fda_inputs(1, [(H, W)], G, D, K, Q=3, seed=32, dtype=torch.float64)
+    pix = [(0, 0), (3, 4), (2, 1), (1, 3)]
+    for k, (y, x) in enumerate(pix):
+        sla[..., 2 * k] = (x + 0.5) / W
+        sla[..., 2 * k + 1] = (y + 0.5) / H
+    sla[..., 2 * K:] = 0.25
+    out = oracle.flash_deform_attn_forward(value.numpy(), shp.numpy(), start.numpy(), sla.numpy(), K)
+    expect = sum(value[0, y * W + x] for y, x in pix) / 4          # (G, D)
+    np.testing.assert_allclose(out[0, 0], expect.reshape(-1).numpy(), rtol=1e-12, atol=1e-12)
+
+
+def test_fda_level_start_index_selects_the_level(oracle):
+    # a dominant logit on a tap of level 1 must read from value[start_1 + ...]
+    shapes, G, D, K = [(3, 3), (2, 2)], 1, 2, 4
+    value, shp, start, sla, _ = make_fda_inputs(1, shapes, G, D, K, Q=1, seed=33, dtype=torch.float64)
+    sla[..., 2 * 2 * K:] = -1e3
+    t = 1 * K + 2
+    sla[..., 2 * 2 * K + t] = 0.0
+    sla[..., 2 * t] = 1.5 / 2
+    sla[..., 2 * t + 1] = 0.5 / 2
+    out = oracle.flash_deform_attn_forward(value.numpy(), shp.numpy(), start.numpy(), sla.numpy(), K)
+    np.testing.assert_allclose(out[0, 0], value[0, 9 + 0 * 2 + 1, 0].numpy(), rtol=1e-12)
+
+
+def test_fda_backward_matches_finite_differences(oracle):
+    shapes, G, D, K = [(5, 4), (3, 2)], 2, 3, 4
+    value, shp, start, sla, go = make_fda_inputs(1, shapes, G, D, K, Q=5, seed=34, dtype=torch.float64,
+                                                 loc_lo=-0.1, loc_hi=1.1)
+    v, s, g = value.numpy().copy(), sla.numpy().copy(), go.numpy()
+    gv, gs = oracle.flash_deform_attn_backward(v, shp.numpy(), start.numpy(), s, g, K)
+    fwd = lambda: oracle.flash_deform_attn_forward(v, shp.numpy(), start.numpy(), s, K)
+    rng = np.random.default_rng(1)
+    iv = rng.choice(v.size, 40, replace=False)
+    np.testing.assert_allclose(gv.reshape(-1)[iv], _central_differences(fwd, v, g, iv), rtol=1e-6, atol=1e-7)
+    io = rng.choice(s.size, 80, replace=False)
+    np.testing.assert_allclose(gs.reshape(-1)[io], _central_differences(fwd, s, g, io), rtol=1e-5, atol=1e-6)
+
+
+def test_fda_logit_gradients_sum_to_zero_and_vanish_for_out_of_range_locations(oracle):
+    shapes, G, D, K = [(4, 4), (2, 2)], 2, 2, 4
+    value, shp, start, sla, go = make_fda_inputs(1, shapes, G, D, K, Q=6, seed=35, dtype=torch.float64)
+    _, gs = oracle.flash_deform_attn_backward(value.numpy(), shp.numpy(), start.numpy(), sla.numpy(), go.numpy(), K)
+    np.testing.assert_allclose(gs[..., 16:].sum(-1), 0.0, atol=1e-12)     # softmax Jacobian has zero row sums
+    sla[..., :16] = 7.0
+    gv, gs = oracle.flash_deform_attn_backward(value.numpy(), shp.numpy(), start.numpy(), sla.numpy(), go.numpy(), K)
+    assert np.all(gv == 0.0) and np.all(gs == 0.0)
