@@ -1,0 +1,214 @@
+#!/usr/bin/env python3
+"""Benchmark of the DCNv4 / flash-deformable-attention hot path on one MI355X.
+
+One "step" is one pass of the hot path over one batch of synthetic input: DCNv4 forward +
+backward at the four FlashInternImage-T stage shapes (batch 64, 3x3, group width 16), once
+with fp16 and once with fp32 tensors (16 operator calls).  The headline value is the
+algorithmic-byte throughput of that step: every tensor counted once in its I/O dtype,
+  forward  s*B*Q*(2C + P_pad)      backward  s*B*Q*(3C + 2*P_pad)
+divided by the step time, inputs resident in HBM.  Per-operator timings (HIP events on the
+stream the kernels run on) for these shapes, the dense-prediction shapes and the
+Deformable-DETR attention shape are reported under "detail"; "roofline" describes the operator
+that takes the largest share of the step; "cpu_baseline" times the pure-PyTorch grid_sample
+formulation of the same operator (oracle/torch_core.py) on the host cores on a reduced batch.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W]
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0           # MI355X HBM3E, published
+GEOM = (3, 3, 1, 1, 1, 1, 1, 1)  # kh kw sh sw ph pw dh dw
+
+# (name, B, H, W, C, G)
+CFG2 = [("T-stage1", 64, 56, 56, 64, 4), ("T-stage2", 64, 28, 28, 128, 8),
+        ("T-stage3", 64, 14, 14, 256, 16), ("T-stage4", 64, 7, 7, 512, 32)]
+CFG3 = [("L-dense1", 2, 256, 256, 160, 10), ("L-dense2", 2, 128, 128, 320, 20),
+        ("L-dense3", 2, 64, 64, 640, 40), ("L-dense4", 2, 32, 32, 1280, 80)]
+CFG4_SHAPES = [(128, 128), (64, 64), (32, 32), (16, 16)]
+
+
+def p_pad(G, K=9):
+    return int(math.ceil(G * K * 3 / 8) * 8)
+
+
+def dcn_bytes(s, B, H, W, C, G):
+    q = B * H * W
+    return s * q * (2 * C + p_pad(G)), s * q * (3 * C + 2 * p_pad(G))
+
+
+def fda_bytes(s, B, N, Q, G, D, L, K):
+    v, sla, out = B * N * G * D, B * Q * G * L * K * 3, B * Q * G * D
+    return s * (v + sla + out), s * (2 * v + 2 * sla + out)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--op-iters", type=int, default=100, help="timed launches per operator in the detail table")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-detail", action="store_true", help="skip per-operator timings other than the step's own")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this operator has no cross-GPU communication and every box here "
+                 "has a single MI355X; run with --gpus 1 (data-parallel scaling is a batch split, see DESIGN.md).")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an MI355X (torch.cuda.is_available() is False)")
+    from dcnv4_amd import ext
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    torch.manual_seed(0)
+
+    def dcn_inputs(B, H, W, C, G, dtype, off_range):
+        K = 9
+        value = torch.randn(B, H, W, C, device=dev, dtype=torch.float32)
+        om = torch.zeros(B, H, W, p_pad(G), device=dev, dtype=torch.float32)
+        body = torch.cat([(torch.rand(B, H, W, G, 2 * K, device=dev) * 2 - 1) * off_range,
+                          torch.randn(B, H, W, G, K, device=dev)], -1).reshape(B, H, W, G * K * 3)
+        om[..., : G * K * 3] = body
+        go = torch.randn(B, H, W, C, device=dev)
+        return value.to(dtype), om.to(dtype), go.to(dtype)
+
+    def dcn_fwd(t, G, C):
+        return ext.dcnv4_forward(t[0], t[1], *GEOM, G, C // G, 1.0, 64, 0, 0, 0, False)
+
+    def dcn_bwd(t, G, C):
+        return ext.dcnv4_backward(t[0], t[1], *GEOM, G, C // G, 1.0, 64, t[2], 0, 0, 0, False)
+
+    def time_op(fn, iters, warm=20):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters      # ms per call
+
+    # ------------------------------------------------------------------ the step (configs[1])
+    work = []
+    for dtype, s in ((torch.float16, 2), (torch.float32, 4)):
+        for name, B, H, W, C, G in CFG2:
+            work.append((name, dtype, s, (B, H, W, C, G), dcn_inputs(B, H, W, C, G, dtype, 3.0)))
+
+    def step():
+        for _, _, _, (B, H, W, C, G), t in work:
+            dcn_fwd(t, G, C)
+            dcn_bwd(t, G, C)
+
+    step_bytes = sum(sum(dcn_bytes(s, *shape)) for _, _, s, shape, _ in work)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ------------------------------------------------------------------ per-operator detail
+    detail = []
+
+    def add(op, name, dtype, ms, nbytes):
+        gbps = nbytes / (ms * 1e-3) / 1e9
+        detail.append({"op": op, "shape": name, "dtype": str(dtype).replace("torch.", ""), "ms": round(ms, 5),
+                       "MB": round(nbytes / 1e6, 2), "GBps": round(gbps, 1), "pct_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2)})
+
+    for name, dtype, s, shape, t in work:
+        B, H, W, C, G = shape
+        fb, bb = dcn_bytes(s, *shape)
+        add("dcnv4_fwd", name, dtype, time_op(lambda: dcn_fwd(t, G, C), args.op_iters), fb)
+        add("dcnv4_bwd", name, dtype, time_op(lambda: dcn_bwd(t, G, C), args.op_iters), bb)
+    step_ops = list(detail)
+
+    if not args.no_detail:
+        for name, B, H, W, C, G in CFG3:
+            t = dcn_inputs(B, H, W, C, G, torch.float16, 4.0)
+            fb, bb = dcn_bytes(2, B, H, W, C, G)
+            add("dcnv4_fwd", name, torch.float16, time_op(lambda: dcn_fwd(t, G, C), args.op_iters), fb)
+            add("dcnv4_bwd", name, torch.float16, time_op(lambda: dcn_bwd(t, G, C), args.op_iters), bb)
+            del t
+        B, G, D, L, K = 4, 8, 32, 4, 4
+        N = sum(h * w for h, w in CFG4_SHAPES)
+        shapes = torch.tensor(CFG4_SHAPES, dtype=torch.int64, device=dev)
+        sizes = [h * w for h, w in CFG4_SHAPES]
+        starts = torch.tensor([sum(sizes[:i]) for i in range(L)], dtype=torch.int64, device=dev)
+        for dtype, s in ((torch.float16, 2), (torch.float32, 4)):
+            v = torch.randn(B, N, G, D, device=dev).to(dtype)
+            sla = torch.cat([torch.rand(B, N, G, L * K * 2, device=dev), torch.randn(B, N, G, L * K, device=dev)], -1).to(dtype)
+            go = torch.randn(B, N, G * D, device=dev).to(dtype)
+            fb, bb = fda_bytes(s, B, N, N, G, D, L, K)
+            add("flash_deform_attn_fwd", "DETR-enc 4lvl Q=21760", dtype,
+                time_op(lambda: ext.flash_deform_attn_forward(v, shapes, starts, sla, 64, K, 0, 0), args.op_iters), fb)
+            add("flash_deform_attn_bwd", "DETR-enc 4lvl Q=21760", dtype,
+                time_op(lambda: ext.flash_deform_attn_backward(v, shapes, starts, sla, go, 64, K, 0, 0), args.op_iters), bb)
+            del v, sla, go
+
+    # ------------------------------------------------------------------ roofline of the dominant operator
+    dom = max(step_ops, key=lambda d: d["ms"])
+    dom_bytes = dom["MB"] * 1e6
+    roofline = {
+        "bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+        "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+        "kernel": f'{dom["op"]} {dom["shape"]} {dom["dtype"]}', "ms": dom["ms"],
+        "algorithmic_bytes": int(dom_bytes),
+        "note": "HIP events around whole operator calls (for backward: clear + scatter kernel + cast)",
+    }
+
+    # ------------------------------------------------------------------ CPU baseline (rank 0, bounded sample)
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import torch_core
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+        torch.set_num_threads(cores)
+        Bc = 8
+        cpu_bytes, cpu_time = 0, 0.0
+        for name, B, H, W, C, G in CFG2:
+            v, om, go = (x.cpu().float()[:Bc].contiguous() for x in dcn_inputs(Bc, H, W, C, G, torch.float32, 3.0))
+            v.requires_grad_(True)
+            om.requires_grad_(True)
+
+            def run():
+                out = torch_core.dcnv4_core_torch(v, om, *GEOM, G, C // G, 1.0)
+                out.backward(go)
+                v.grad = om.grad = None
+            run()
+            reps = 3
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                run()
+            cpu_time += (time.perf_counter() - t0) / reps
+            cpu_bytes += sum(dcn_bytes(4, Bc, H, W, C, G))
+        cpu = {"value": round(cpu_bytes / cpu_time / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+               "sample": f"DCNv4 fwd+bwd, four FlashInternImage-T stage shapes at batch {Bc} (of 64), fp32, "
+                         f"torch grid_sample formulation + autograd, {cpu_time * 1e3:.0f} ms per pass"}
+
+    line = {
+        "metric": "DCNv4 fwd+bwd achieved HBM GB/s (algorithmic bytes / time)", "value": round(value, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "DCNv4 forward+backward, FlashInternImage-T stages (56x56 C64 G4, 28x28 C128 G8, "
+                               "14x14 C256 G16, 7x7 C512 G32), batch 64, 3x3 s1 p1, fp16 and fp32 tensors, fp32 arithmetic",
+                   "step_algorithmic_MB": round(step_bytes / 1e6, 1), "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2)},
+        "roofline": roofline, "cpu_baseline": cpu, "detail": detail,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

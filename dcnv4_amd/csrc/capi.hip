@@ -1,0 +1,411 @@
+// C-ABI entry points of libdcnv4_gfx950.so (declared in include/dcnv4_gfx950.h): argument
+// checks, launch geometry for wave64, batch chunking for 32-bit buffer addressing, and the
+// small utility kernels (clear, fp32 -> half cast) around the sampling kernels.
+// Host-side counterpart of the reference's DCNv4_op/src/cuda/dcnv4_cuda.cu:26-175 and
+// DCNv4_op/src/cuda/flash_deform_attn_cuda.cu:26-163, minus tensor allocation, which the
+// caller owns.
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+
+#include "../../include/dcnv4_gfx950.h"
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace dcn {
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int elem_bytes(int dtype) {
+  switch (dtype) {
+    case DCNV4_DTYPE_F32: return 4;
+    case DCNV4_DTYPE_F16:
+    case DCNV4_DTYPE_BF16: return 2;
+  }
+  return 0;
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int ceil_log2(int v) {
+  int l = 0;
+  while ((1 << l) < v) ++l;
+  return l;
+}
+
+// Channels per lane: the widest power-of-two vector (<= 16 bytes) that divides D, unless a
+// valid d_stride hint asks for a narrower one.  Reference table: dcnv4_im2col_cuda.cuh:342-415.
+int choose_lanes(int D, int s, int d_stride, LaneMap *lm) {
+  if (d_stride != 0 && d_stride != 1 && d_stride != 2 && d_stride != 4 && d_stride != 8 && d_stride != 16)
+    return fail(DCNV4_ERR_INVALID_ARGUMENT, "invalid d_stride %d", d_stride);
+  int cpt = 1;
+  while (cpt * 2 * s <= 16 && D % (cpt * 2) == 0) cpt *= 2;
+  if (d_stride > 0 && d_stride < cpt && D % d_stride == 0) cpt = d_stride;
+  lm->cpt = cpt;
+  lm->tpg = D / cpt;
+  lm->tpgp_log2 = ceil_log2(lm->tpg);
+  return DCNV4_OK;
+}
+
+// ---------------------------------------------------------------- utility kernels
+__global__ void __launch_bounds__(256) clear_kernel(uint32_t *dst, size_t n16, size_t n_words) {
+  // n16 aligned 16-byte groups, then the (< 4) trailing 32-bit words
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (size_t i = tid; i < n16; i += stride) reinterpret_cast<u32x4 *>(dst)[i] = u32x4{0, 0, 0, 0};
+  for (size_t i = n16 * 4 + tid; i < n_words; i += stride) dst[i] = 0u;
+}
+
+template <typename Tag>
+__global__ void __launch_bounds__(256) narrow_kernel(const float *src, void *dst, size_t n8, size_t n) {
+  // n8 groups of 8 elements, then a scalar tail
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (size_t i = tid; i < n8; i += stride) {
+    const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src) + 2 * i);
+    const f32x4 b = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src) + 2 * i + 1);
+    const float f[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    reinterpret_cast<u32x4 *>(dst)[i] = Pack<Tag, 8>::encode(f);
+  }
+  for (size_t i = n8 * 8 + tid; i < n; i += stride) {
+    const float f[1] = {src[i]};
+    reinterpret_cast<uint16_t *>(dst)[i] = Pack<Tag, 1>::encode(f);
+  }
+}
+
+int grid_for(size_t work_items) {
+  const size_t blocks = (work_items + 255) / 256;
+  return (int)std::min<size_t>(std::max<size_t>(blocks, 1), 256 * 32);
+}
+
+// Clears n_words 32-bit words at a 16-byte aligned address with a kernel rather than a memset
+// node, so the call stays safe under HIP-graph capture.
+hipError_t clear_async(void *dst, size_t n_words, hipStream_t stream) {
+  if (n_words == 0) return hipSuccess;
+  const size_t n16 = n_words / 4;
+  hipLaunchKernelGGL(clear_kernel, dim3(grid_for(std::max<size_t>(n16, 1))), dim3(256), 0, stream,
+                     reinterpret_cast<uint32_t *>(dst), n16, n_words);
+  return hipGetLastError();
+}
+
+hipError_t narrow_async(int dtype, const float *src, void *dst, size_t n, hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  const size_t n8 = n / 8;
+  const dim3 grid(grid_for(std::max<size_t>(n8, 1))), block(256);
+  if (dtype == DCNV4_DTYPE_F16) hipLaunchKernelGGL(narrow_kernel<F16>, grid, block, 0, stream, src, dst, n8, n);
+  else hipLaunchKernelGGL(narrow_kernel<BF16>, grid, block, 0, stream, src, dst, n8, n);
+  return hipGetLastError();
+}
+
+size_t round16(size_t v) { return (v + 15) & ~size_t(15); }
+
+// ---------------------------------------------------------------- DCNv4
+struct DcnProblem {
+  DcnLaunch launch;      // geometry common to every chunk
+  int batch, Ho, Wo, s;
+  size_t img_elems, img_out_elems, img_om_elems;
+};
+
+int out_extent(int in, int pad, int dil, int k, int stride) {     // dcnv4_cuda.cu:48-52
+  return (in + 2 * pad - (dil * (k - 1) + 1)) / stride + 1;
+}
+
+int dcn_prepare(DcnProblem *pr, bool backward, int dtype, int batch, int H, int W, int G, int D, int kh,
+                int kw, int sh, int sw, int ph, int pw, int dh, int dw, float offset_scale, int im2col_step,
+                int remove_center, int P_pad, int softmax, int d_stride, int block_thread) {
+  const int s = elem_bytes(dtype);
+  if (s == 0) return fail(DCNV4_ERR_RUNTIME, "unsupported dtype code %d (fp32, fp16, bf16 only)", dtype);
+  if (batch <= 0 || H <= 0 || W <= 0 || G <= 0 || D <= 0)
+    return fail(DCNV4_ERR_RUNTIME, "empty or negative tensor extent (batch %d, H %d, W %d, group %d, group_channels %d)",
+                batch, H, W, G, D);
+  if (kh <= 0 || kw <= 0 || sh <= 0 || sw <= 0 || dh <= 0 || dw <= 0 || ph < 0 || pw < 0)
+    return fail(DCNV4_ERR_INVALID_ARGUMENT, "invalid kernel shape");
+  remove_center = remove_center ? 1 : 0;
+  if (remove_center && (kh % 2 == 0 || kw % 2 == 0))
+    return fail(DCNV4_ERR_INVALID_ARGUMENT, "remove_center needs an odd kernel, got %dx%d", kh, kw);
+  const int Kp = kh * kw - remove_center;
+  if (Kp < 1 || Kp > kMaxTaps) return fail(DCNV4_ERR_INVALID_ARGUMENT, "invalid kernel shape: %d taps (1..%d)", Kp, kMaxTaps);
+  if (im2col_step <= 0) return fail(DCNV4_ERR_RUNTIME, "im2col_step must be positive");
+  const int step = std::min(batch, im2col_step);
+  if (batch % step != 0) return fail(DCNV4_ERR_RUNTIME, "batch(%d) must divide im2col_step(%d)", batch, step);
+  const int Ho = out_extent(H, ph, dh, kh, sh), Wo = out_extent(W, pw, dw, kw, sw);
+  if (Ho <= 0 || Wo <= 0) return fail(DCNV4_ERR_RUNTIME, "kernel does not fit the padded input (output %dx%d)", Ho, Wo);
+  if (P_pad < G * Kp * 3)
+    return fail(DCNV4_ERR_RUNTIME, "offset_mask last dim %d is smaller than group*K*3 = %d", P_pad, G * Kp * 3);
+
+  DcnLaunch &L = pr->launch;
+  L = DcnLaunch{};
+  if (int rc = choose_lanes(D, s, d_stride, &L.lanes)) return rc;
+  const int width = 1 << L.lanes.tpgp_log2;
+  if (backward && width > kWave)
+    return fail(DCNV4_ERR_INVALID_ARGUMENT, "backward needs group_channels/%d <= 64 lanes per group, got %d",
+                L.lanes.cpt, L.lanes.tpg);
+  L.Q = Ho * Wo; L.Wo = Wo; L.H = H; L.W = W; L.G = G; L.D = D;
+  L.kh = kh; L.kw = kw; L.sh = sh; L.sw = sw; L.ph = ph; L.pw = pw; L.dh = dh; L.dw = dw;
+  L.Kp = Kp; L.P_pad = P_pad; L.remove_center = remove_center; L.softmax = softmax ? 1 : 0;
+  L.offset_scale = offset_scale;
+
+  const int lanes_per_pix = G * width;
+  const int want = block_thread > 0 ? block_thread : kBlockThreads;
+  int npix = std::max(1, want / lanes_per_pix);
+  const size_t lds_per_pix = (size_t)P_pad * sizeof(float) * (backward ? 2 : 1);
+  while (npix > 1 && npix * lds_per_pix > kMaxDynamicLds) --npix;
+  if (npix * lds_per_pix > kMaxDynamicLds)
+    return fail(DCNV4_ERR_RUNTIME, "offset_mask row of %d elements does not fit in LDS", P_pad);
+  L.npix_block = npix;
+
+  pr->batch = batch; pr->Ho = Ho; pr->Wo = Wo; pr->s = s;
+  pr->img_elems = (size_t)H * W * G * D;
+  pr->img_out_elems = (size_t)Ho * Wo * G * D;
+  pr->img_om_elems = (size_t)Ho * Wo * P_pad;
+  if ((uint64_t)pr->img_elems * (backward ? 4 : s) > kMaxSpanBytes)
+    return fail(DCNV4_ERR_RUNTIME, "one image of %zu elements exceeds the 2 GiB addressing span of a launch", pr->img_elems);
+  return DCNV4_OK;
+}
+
+int images_per_launch(const DcnProblem &pr, bool backward) {
+  const uint64_t per_img = (uint64_t)pr.img_elems * (backward ? 4 : pr.s);
+  uint64_t n = std::max<uint64_t>(1, kMaxSpanBytes / per_img);
+  n = std::min<uint64_t>(n, 0x7fffffffull / (uint64_t)pr.launch.Q);   // n_pix stays an int
+  return (int)std::min<uint64_t>(n, (uint64_t)pr.batch);
+}
+
+// ---------------------------------------------------------------- flash deformable attention
+struct FdaProblem {
+  FdaLaunch launch;
+  int batch, s;
+  size_t img_elems, img_row_elems, img_out_elems;
+};
+
+int fda_prepare(FdaProblem *pr, bool backward, int dtype, int batch, int N, int G, int D, int L, int Q, int K,
+                int im2col_step, int d_stride, int block_thread) {
+  const int s = elem_bytes(dtype);
+  if (s == 0) return fail(DCNV4_ERR_RUNTIME, "unsupported dtype code %d (fp32, fp16, bf16 only)", dtype);
+  if (batch <= 0 || N <= 0 || G <= 0 || D <= 0 || Q <= 0)
+    return fail(DCNV4_ERR_RUNTIME, "empty or negative tensor extent (batch %d, spatial %d, heads %d, channels %d, queries %d)",
+                batch, N, G, D, Q);
+  if (L < 1 || L > kMaxLevels) return fail(DCNV4_ERR_INVALID_ARGUMENT, "invalid number of scales: %d (1..%d)", L, kMaxLevels);
+  if (K < 1 || L * K > kMaxTaps)
+    return fail(DCNV4_ERR_INVALID_ARGUMENT, "invalid number of points: K=%d with %d levels (L*K <= %d)", K, L, kMaxTaps);
+  if (im2col_step <= 0) return fail(DCNV4_ERR_RUNTIME, "im2col_step must be positive");
+  const int step = std::min(batch, im2col_step);
+  if (batch % step != 0) return fail(DCNV4_ERR_RUNTIME, "batch(%d) must divide im2col_step(%d)", batch, step);
+
+  FdaLaunch &F = pr->launch;
+  F = FdaLaunch{};
+  if (int rc = choose_lanes(D, s, d_stride, &F.lanes)) return rc;
+  const int width = 1 << F.lanes.tpgp_log2;
+  if (backward && width > kWave)
+    return fail(DCNV4_ERR_INVALID_ARGUMENT, "backward needs head_channels/%d <= 64 lanes per head, got %d",
+                F.lanes.cpt, F.lanes.tpg);
+  F.Q = Q; F.N = N; F.G = G; F.D = D; F.L = L; F.K = K;
+  const int lanes_per_row = G * width;
+  const int want = block_thread > 0 ? block_thread : kBlockThreads;
+  int nq = std::max(1, want / lanes_per_row);
+  const size_t lds_per_row = (size_t)G * 3 * L * K * sizeof(float) * (backward ? 2 : 1);
+  while (nq > 1 && nq * lds_per_row > kMaxDynamicLds) --nq;
+  if (nq * lds_per_row > kMaxDynamicLds)
+    return fail(DCNV4_ERR_RUNTIME, "sampling_loc_attn row of %d x %d elements does not fit in LDS", G, 3 * L * K);
+  F.nq_block = nq;
+
+  pr->batch = batch; pr->s = s;
+  pr->img_elems = (size_t)N * G * D;
+  pr->img_row_elems = (size_t)Q * G * 3 * L * K;
+  pr->img_out_elems = (size_t)Q * G * D;
+  if ((uint64_t)pr->img_elems * (backward ? 4 : s) > kMaxSpanBytes)
+    return fail(DCNV4_ERR_RUNTIME, "one value image of %zu elements exceeds the 2 GiB addressing span of a launch", pr->img_elems);
+  return DCNV4_OK;
+}
+
+int images_per_launch(const FdaProblem &pr, bool backward) {
+  const uint64_t per_img = (uint64_t)pr.img_elems * (backward ? 4 : pr.s);
+  uint64_t n = std::max<uint64_t>(1, kMaxSpanBytes / per_img);
+  n = std::min<uint64_t>(n, 0x7fffffffull / (uint64_t)pr.launch.Q);
+  return (int)std::min<uint64_t>(n, (uint64_t)pr.batch);
+}
+
+int check_ptrs(std::initializer_list<const void *> ptrs) {
+  for (const void *p : ptrs) {
+    if (p == nullptr) return fail(DCNV4_ERR_RUNTIME, "null tensor pointer");
+    if (!aligned16(p)) return fail(DCNV4_ERR_RUNTIME, "tensor pointer %p is not 16-byte aligned", p);
+  }
+  return DCNV4_OK;
+}
+
+int hip_fail(const char *what, hipError_t e) {
+  return fail(DCNV4_ERR_RUNTIME, "%s: %s", what, hipGetErrorString(e));
+}
+
+const char *at(const void *base, size_t elems, int s) { return static_cast<const char *>(base) + elems * s; }
+char *at(void *base, size_t elems, int s) { return static_cast<char *>(base) + elems * s; }
+
+}  // namespace
+}  // namespace dcn
+
+using namespace dcn;
+
+extern "C" {
+
+int dcnv4_gfx950_abi_version(void) { return DCNV4_GFX950_ABI_VERSION; }
+
+const char *dcnv4_gfx950_last_error(void) { return g_error; }
+
+int dcnv4_gfx950_forward(const void *value, const void *offset_mask, void *output, int dtype, int batch,
+                         int height_in, int width_in, int group, int group_channels, int kernel_h,
+                         int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h,
+                         int dilation_w, float offset_scale, int im2col_step, int remove_center,
+                         int padded_offset_dim, int softmax, int d_stride, int block_thread, void *stream) {
+  DcnProblem pr;
+  if (int rc = dcn_prepare(&pr, false, dtype, batch, height_in, width_in, group, group_channels, kernel_h,
+                           kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, offset_scale,
+                           im2col_step, remove_center, padded_offset_dim, softmax, d_stride, block_thread))
+    return rc;
+  if (int rc = check_ptrs({value, offset_mask, output})) return rc;
+  const int per = images_per_launch(pr, false);
+  for (int b0 = 0; b0 < batch; b0 += per) {
+    const int nb = std::min(per, batch - b0);
+    DcnLaunch L = pr.launch;
+    L.value = at(value, b0 * pr.img_elems, pr.s);
+    L.offset_mask = at(offset_mask, b0 * pr.img_om_elems, pr.s);
+    L.out = at(output, b0 * pr.img_out_elems, pr.s);
+    L.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
+    L.n_pix = nb * L.Q;
+    if (hipError_t e = launch_dcnv4_forward(dtype, L, static_cast<hipStream_t>(stream)))
+      return hip_fail("dcnv4 forward launch", e);
+  }
+  return DCNV4_OK;
+}
+
+size_t dcnv4_gfx950_backward_workspace_bytes(int dtype, int batch, int height_in, int width_in, int group,
+                                             int group_channels) {
+  if (elem_bytes(dtype) != 2 || batch <= 0 || height_in <= 0 || width_in <= 0 || group <= 0 || group_channels <= 0)
+    return 0;
+  return round16((size_t)batch * height_in * width_in * group * group_channels * sizeof(float));
+}
+
+int dcnv4_gfx950_backward(const void *value, const void *offset_mask, const void *grad_output, void *grad_value,
+                          void *grad_offset_mask, void *workspace, size_t workspace_bytes, int dtype, int batch,
+                          int height_in, int width_in, int group, int group_channels, int kernel_h, int kernel_w,
+                          int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w,
+                          float offset_scale, int im2col_step, int remove_center, int padded_offset_dim,
+                          int softmax, int d_stride, int block_thread, void *stream) {
+  DcnProblem pr;
+  if (int rc = dcn_prepare(&pr, true, dtype, batch, height_in, width_in, group, group_channels, kernel_h,
+                           kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, offset_scale,
+                           im2col_step, remove_center, padded_offset_dim, softmax, d_stride, block_thread))
+    return rc;
+  if (int rc = check_ptrs({value, offset_mask, grad_output, grad_value, grad_offset_mask})) return rc;
+  const size_t need = dcnv4_gfx950_backward_workspace_bytes(dtype, batch, height_in, width_in, group, group_channels);
+  if (need > 0) {
+    if (workspace == nullptr || !aligned16(workspace) || workspace_bytes < need)
+      return fail(DCNV4_ERR_RUNTIME, "workspace of %zu bytes needed, got %zu at %p", need, workspace_bytes, workspace);
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const size_t total = (size_t)batch * pr.img_elems;
+  float *acc = need > 0 ? static_cast<float *>(workspace) : static_cast<float *>(grad_value);
+  if (hipError_t e = clear_async(acc, total, st)) return hip_fail("clear launch", e);
+  const int per = images_per_launch(pr, true);
+  for (int b0 = 0; b0 < batch; b0 += per) {
+    const int nb = std::min(per, batch - b0);
+    DcnLaunch L = pr.launch;
+    L.value = at(value, b0 * pr.img_elems, pr.s);
+    L.offset_mask = at(offset_mask, b0 * pr.img_om_elems, pr.s);
+    L.grad_out = at(grad_output, b0 * pr.img_out_elems, pr.s);
+    L.grad_value_acc = acc + b0 * pr.img_elems;
+    L.grad_offset_mask = at(grad_offset_mask, b0 * pr.img_om_elems, pr.s);
+    L.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
+    L.n_pix = nb * L.Q;
+    if (hipError_t e = launch_dcnv4_backward(dtype, L, st)) return hip_fail("dcnv4 backward launch", e);
+  }
+  if (need > 0)
+    if (hipError_t e = narrow_async(dtype, acc, grad_value, total, st)) return hip_fail("cast launch", e);
+  return DCNV4_OK;
+}
+
+int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_shapes,
+                                     const int64_t *level_start_index, const void *sampling_loc_attn,
+                                     void *output, int dtype, int batch, int spatial_size, int num_heads,
+                                     int head_channels, int num_levels, int num_query, int num_points,
+                                     int im2col_step, int d_stride, int block_thread, void *stream) {
+  FdaProblem pr;
+  if (int rc = fda_prepare(&pr, false, dtype, batch, spatial_size, num_heads, head_channels, num_levels, num_query,
+                           num_points, im2col_step, d_stride, block_thread))
+    return rc;
+  if (int rc = check_ptrs({value, sampling_loc_attn, output})) return rc;
+  if (spatial_shapes == nullptr || level_start_index == nullptr) return fail(DCNV4_ERR_RUNTIME, "null level tensors");
+  const int per = images_per_launch(pr, false);
+  for (int b0 = 0; b0 < batch; b0 += per) {
+    const int nb = std::min(per, batch - b0);
+    FdaLaunch F = pr.launch;
+    F.value = at(value, b0 * pr.img_elems, pr.s);
+    F.sla = at(sampling_loc_attn, b0 * pr.img_row_elems, pr.s);
+    F.out = at(output, b0 * pr.img_out_elems, pr.s);
+    F.shapes = spatial_shapes;
+    F.level_start = level_start_index;
+    F.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
+    F.n_row = nb * F.Q;
+    if (hipError_t e = launch_fda_forward(dtype, F, static_cast<hipStream_t>(stream)))
+      return hip_fail("flash_deform_attn forward launch", e);
+  }
+  return DCNV4_OK;
+}
+
+size_t flash_deform_attn_gfx950_backward_workspace_bytes(int dtype, int batch, int spatial_size, int num_heads,
+                                                         int head_channels) {
+  if (elem_bytes(dtype) != 2 || batch <= 0 || spatial_size <= 0 || num_heads <= 0 || head_channels <= 0) return 0;
+  return round16((size_t)batch * spatial_size * num_heads * head_channels * sizeof(float));
+}
+
+int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_shapes,
+                                      const int64_t *level_start_index, const void *sampling_loc_attn,
+                                      const void *grad_output, void *grad_value, void *grad_sampling_loc_attn,
+                                      void *workspace, size_t workspace_bytes, int dtype, int batch,
+                                      int spatial_size, int num_heads, int head_channels, int num_levels,
+                                      int num_query, int num_points, int im2col_step, int d_stride,
+                                      int block_thread, void *stream) {
+  FdaProblem pr;
+  if (int rc = fda_prepare(&pr, true, dtype, batch, spatial_size, num_heads, head_channels, num_levels, num_query,
+                           num_points, im2col_step, d_stride, block_thread))
+    return rc;
+  if (int rc = check_ptrs({value, sampling_loc_attn, grad_output, grad_value, grad_sampling_loc_attn})) return rc;
+  if (spatial_shapes == nullptr || level_start_index == nullptr) return fail(DCNV4_ERR_RUNTIME, "null level tensors");
+  const size_t need =
+      flash_deform_attn_gfx950_backward_workspace_bytes(dtype, batch, spatial_size, num_heads, head_channels);
+  if (need > 0) {
+    if (workspace == nullptr || !aligned16(workspace) || workspace_bytes < need)
+      return fail(DCNV4_ERR_RUNTIME, "workspace of %zu bytes needed, got %zu at %p", need, workspace_bytes, workspace);
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const size_t total = (size_t)batch * pr.img_elems;
+  float *acc = need > 0 ? static_cast<float *>(workspace) : static_cast<float *>(grad_value);
+  if (hipError_t e = clear_async(acc, total, st)) return hip_fail("clear launch", e);
+  const int per = images_per_launch(pr, true);
+  for (int b0 = 0; b0 < batch; b0 += per) {
+    const int nb = std::min(per, batch - b0);
+    FdaLaunch F = pr.launch;
+    F.value = at(value, b0 * pr.img_elems, pr.s);
+    F.sla = at(sampling_loc_attn, b0 * pr.img_row_elems, pr.s);
+    F.grad_out = at(grad_output, b0 * pr.img_out_elems, pr.s);
+    F.grad_value_acc = acc + b0 * pr.img_elems;
+    F.grad_sla = at(grad_sampling_loc_attn, b0 * pr.img_row_elems, pr.s);
+    F.shapes = spatial_shapes;
+    F.level_start = level_start_index;
+    F.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
+    F.n_row = nb * F.Q;
+    if (hipError_t e = launch_fda_backward(dtype, F, st)) return hip_fail("flash_deform_attn backward launch", e);
+  }
+  if (need > 0)
+    if (hipError_t e = narrow_async(dtype, acc, grad_value, total, st)) return hip_fail("cast launch", e);
+  return DCNV4_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,256 @@
+// Flash deformable attention kernels for gfx950 (wave64): multi-level bilinear sampling with
+// the softmax over all L*K taps fused in.
+//
+// Replaces the reference's forward_kernel_reg (DCNv4_op/src/cuda/flash_deform_im2col_cuda.cuh:129-209)
+// and backward_kernel_warp_primitive (DCNv4_op/src/cuda/flash_deform_col2im_cuda.cuh:171-318).
+//
+// A workgroup owns `nq_block` consecutive queries (all heads).  Their sampling_loc_attn rows
+// are one contiguous span: streamed once into LDS as fp32 and shared by the channel lanes of a
+// (query, head).  One lane owns `cpt` contiguous channels (16 bytes).  The softmax needs only a
+// running max and sum per (query, head); each tap's probability is recomputed from its logit,
+// so L and K stay run-time values.  Backward applies the Jacobian in closed form,
+// p_i (a_i - sum_j p_j a_j), where the reference loops over all (L*K)^2 pairs
+// (flash_deform_col2im_cuda.cuh:301-316); a tap outside its level contributes a_i = 0.
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace dcn {
+namespace {
+
+struct Level { int H, W, start; };
+
+__device__ __forceinline__ Level load_level(const FdaLaunch &p, int l) {
+  Level lv;
+  lv.H = (int)p.shapes[2 * l];
+  lv.W = (int)p.shapes[2 * l + 1];
+  lv.start = (int)p.level_start[l];
+  return lv;
+}
+
+__device__ __forceinline__ void softmax_stats(const float *m, int n, float &mx, float &inv) {
+  mx = m[0];
+  for (int k = 1; k < n; ++k) mx = fmaxf(mx, m[k]);
+  float s = 0.f;
+  for (int k = 0; k < n; ++k) s += __expf(m[k] - mx);
+  inv = 1.f / s;
+}
+
+// ------------------------------------------------------------------------------- forward
+template <typename Tag, int CPT, int KT>
+__global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLaunch p) {
+  extern __shared__ float lds[];
+  typedef Pack<Tag, CPT> pack;
+  const int LK = p.L * p.K, row_len = 3 * LK;
+  const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
+  const int row0 = (int)blk * p.nq_block;
+  const int nrow = min(p.nq_block, p.n_row - row0);
+  const int span = nrow * p.G * row_len;
+  const bool vec16 = ((size_t)p.G * row_len * Tag::kBytes) % 16 == 0;
+  stage_rows_to_lds<Tag>(lds, (const char *)p.sla + (size_t)row0 * p.G * row_len * Tag::kBytes, span, vec16);
+  __syncthreads();
+
+  const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
+  const int tpgp_log2 = p.lanes.tpgp_log2;
+  const int items = (nrow * p.G) << tpgp_log2;
+  const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
+  const int K = KT > 0 ? KT : p.K;
+
+  for (int it = threadIdx.x; it < items; it += blockDim.x) {
+    const int chunk = it & ((1 << tpgp_log2) - 1);
+    if (chunk >= p.lanes.tpg) continue;
+    const int rg = it >> tpgp_log2;                 // (row, head) index inside the workgroup
+    const int lr = rg / p.G, g = rg - lr * p.G;
+    const int b = (row0 + lr) / p.Q;
+    const float *s = lds + rg * row_len;
+    float mx, inv;
+    softmax_stats(s + 2 * LK, LK, mx, inv);
+    const uint32_t lane_base = (uint32_t)(g * p.D + chunk * CPT) * Tag::kBytes;
+
+    float acc[CPT];
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) acc[c] = 0.f;
+
+    for (int l = 0; l < p.L; ++l) {
+      const Level lv = load_level(p, l);
+      const uint32_t base = (uint32_t)(b * p.N + lv.start) * pix_bytes + lane_base;
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        const int t = l * K + k;
+        const float x = sub_rn(mul_rn(s[2 * t], (float)lv.W), 0.5f);       // flash_deform_im2col_cuda.cuh:188-189
+        const float y = sub_rn(mul_rn(s[2 * t + 1], (float)lv.H), 0.5f);
+        const float pr = __expf(s[2 * LK + t] - mx) * inv;
+        const Tap tp = make_tap(y, x, lv.H, lv.W, base, pix_bytes);
+        typename pack::raw_t raw[4];
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn) raw[cn] = buffer_load<pack::kBytes>(value, tp.off[cn]);
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn) {
+          float v[CPT];
+          pack::decode(raw[cn], v);
+          const float w = pr * tp.w[cn];
+#pragma unroll
+          for (int c = 0; c < CPT; ++c) acc[c] = fmaf(w, v[c], acc[c]);
+        }
+      }
+    }
+    char *dst = (char *)p.out + ((size_t)(row0 + lr) * (p.G * p.D) + g * p.D + chunk * CPT) * Tag::kBytes;
+    *reinterpret_cast<typename pack::raw_t *>(dst) = pack::encode(acc);
+  }
+}
+
+// ------------------------------------------------------------------------------- backward
+template <typename Tag, int CPT, int KT>
+__global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLaunch p) {
+  extern __shared__ float lds[];
+  typedef Pack<Tag, CPT> pack;
+  const int LK = p.L * p.K, row_len = 3 * LK;
+  const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
+  const int row0 = (int)blk * p.nq_block;
+  const int nrow = min(p.nq_block, p.n_row - row0);
+  const int span = nrow * p.G * row_len;
+  const bool vec16 = ((size_t)p.G * row_len * Tag::kBytes) % 16 == 0;
+  float *s_in = lds, *s_grad = lds + p.nq_block * p.G * row_len;
+  stage_rows_to_lds<Tag>(s_in, (const char *)p.sla + (size_t)row0 * p.G * row_len * Tag::kBytes, span, vec16);
+  __syncthreads();      // every slot of s_grad is written below: no clearing needed
+
+  const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
+  const __amdgpu_buffer_rsrc_t gacc = make_rsrc(p.grad_value_acc, p.value_bytes / Tag::kBytes * 4);
+  const int tpgp_log2 = p.lanes.tpgp_log2, width = 1 << tpgp_log2;
+  const int items = (nrow * p.G) << tpgp_log2;
+  const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
+  const int K = KT > 0 ? KT : p.K;
+
+  for (int it = threadIdx.x; it < items; it += blockDim.x) {
+    const int chunk = it & (width - 1);
+    const bool active = chunk < p.lanes.tpg;
+    const int rg = it >> tpgp_log2;
+    const int lr = rg / p.G, g = rg - lr * p.G;
+    const int b = (row0 + lr) / p.Q;
+    const float *s = s_in + rg * row_len;
+    float *gs = s_grad + rg * row_len;
+    float mx, inv;
+    softmax_stats(s + 2 * LK, LK, mx, inv);
+    const uint32_t lane_base = (uint32_t)(g * p.D + (active ? chunk : 0) * CPT) * Tag::kBytes;
+
+    float go[CPT];
+    {
+      const char *src = (const char *)p.grad_out + ((size_t)(row0 + lr) * (p.G * p.D)) * Tag::kBytes + lane_base;
+      pack::decode(*reinterpret_cast<const typename pack::raw_t *>(src), go);
+      if (!active) {
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) go[c] = 0.f;
+      }
+    }
+    float dot_rg = 0.f;
+
+    for (int l = 0; l < p.L; ++l) {
+      const Level lv = load_level(p, l);
+      const uint32_t base = (uint32_t)(b * p.N + lv.start) * pix_bytes + lane_base;
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        const int t = l * K + k;
+        const float x = sub_rn(mul_rn(s[2 * t], (float)lv.W), 0.5f);
+        const float y = sub_rn(mul_rn(s[2 * t + 1], (float)lv.H), 0.5f);
+        const float pr = __expf(s[2 * LK + t] - mx) * inv;
+        Tap tp = make_tap(y, x, lv.H, lv.W, base, pix_bytes);
+        if (!active) {
+#pragma unroll
+          for (int cn = 0; cn < 4; ++cn) tp.off[cn] = kDropOffset;
+        }
+        typename pack::raw_t raw[4];
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn) raw[cn] = buffer_load<pack::kBytes>(value, tp.off[cn]);
+        float dots[4];
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn) {
+          float v[CPT];
+          pack::decode(raw[cn], v);
+          float d = 0.f;
+#pragma unroll
+          for (int c = 0; c < CPT; ++c) d = fmaf(v[c], go[c], d);
+          dots[cn] = d;
+          const float w = pr * tp.w[cn];
+          const uint32_t aoff = (tp.off[cn] == kDropOffset) ? kDropOffset : tp.off[cn] * (4 / Tag::kBytes);
+#pragma unroll
+          for (int c = 0; c < CPT; ++c)
+            __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(go[c] * w, gacc, aoff + 4 * c, 0, 0);
+        }
+        const float hy = 1.f - tp.ly, hx = 1.f - tp.lx;
+        float gx = hy * (dots[1] - dots[0]) + tp.ly * (dots[3] - dots[2]);
+        float gy = hx * (dots[2] - dots[0]) + tp.lx * (dots[3] - dots[1]);
+        float gz = tp.w[0] * dots[0] + tp.w[1] * dots[1] + tp.w[2] * dots[2] + tp.w[3] * dots[3];
+        gx = cluster_sum(gx, width);
+        gy = cluster_sum(gy, width);
+        gz = cluster_sum(gz, width);
+        if (chunk == 0) {
+          gs[2 * t] = gx * (float)lv.W * pr;          // flash_deform_col2im_cuda.cuh:273-276
+          gs[2 * t + 1] = gy * (float)lv.H * pr;
+          gs[2 * LK + t] = gz;
+        }
+        dot_rg = fmaf(pr, gz, dot_rg);
+      }
+    }
+    if (chunk == 0) {
+      for (int t = 0; t < LK; ++t) {
+        const float pr = __expf(s[2 * LK + t] - mx) * inv;
+        gs[2 * LK + t] = pr * (gs[2 * LK + t] - dot_rg);
+      }
+    }
+  }
+  __syncthreads();
+  unstage_rows_from_lds<Tag>((char *)p.grad_sla + (size_t)row0 * p.G * row_len * Tag::kBytes, s_grad, span, vec16);
+}
+
+template <typename Tag, int CPT, bool BWD>
+hipError_t launch_k(const FdaLaunch &p, hipStream_t stream, dim3 grid, dim3 block, size_t lds) {
+#define FDA_LAUNCH(KT)                                                                                     \
+  do {                                                                                                     \
+    if (BWD) hipLaunchKernelGGL((fda_backward_kernel<Tag, CPT, KT>), grid, block, lds, stream, p);         \
+    else hipLaunchKernelGGL((fda_forward_kernel<Tag, CPT, KT>), grid, block, lds, stream, p);              \
+  } while (0)
+  if (p.K == 4) FDA_LAUNCH(4);
+  else if (p.K == 8) FDA_LAUNCH(8);
+  else FDA_LAUNCH(0);
+#undef FDA_LAUNCH
+  return hipGetLastError();
+}
+
+template <typename Tag, bool BWD>
+hipError_t launch_by_cpt(const FdaLaunch &p, hipStream_t stream) {
+  const dim3 grid((p.n_row + p.nq_block - 1) / p.nq_block), block(kBlockThreads);
+  const size_t lds = BWD ? fda_backward_lds_bytes(p) : fda_forward_lds_bytes(p);
+#define FDA_CASE(N)                                                                       \
+  case N:                                                                                 \
+    if constexpr (N * Tag::kBytes <= 16) return launch_k<Tag, N, BWD>(p, stream, grid, block, lds); \
+    break;
+  switch (p.lanes.cpt) {
+    FDA_CASE(1) FDA_CASE(2) FDA_CASE(4) FDA_CASE(8)
+  }
+#undef FDA_CASE
+  return hipErrorInvalidValue;
+}
+
+template <bool BWD> hipError_t launch_by_dtype(int dtype, const FdaLaunch &p, hipStream_t stream) {
+  switch (dtype) {
+    case F32::kCode: return launch_by_cpt<F32, BWD>(p, stream);
+    case F16::kCode: return launch_by_cpt<F16, BWD>(p, stream);
+    case BF16::kCode: return launch_by_cpt<BF16, BWD>(p, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+size_t fda_forward_lds_bytes(const FdaLaunch &p) {
+  return (size_t)p.nq_block * p.G * 3 * p.L * p.K * sizeof(float);
+}
+size_t fda_backward_lds_bytes(const FdaLaunch &p) { return 2 * fda_forward_lds_bytes(p); }
+
+hipError_t launch_fda_forward(int dtype, const FdaLaunch &p, hipStream_t stream) {
+  return launch_by_dtype<false>(dtype, p, stream);
+}
+hipError_t launch_fda_backward(int dtype, const FdaLaunch &p, hipStream_t stream) {
+  return launch_by_dtype<true>(dtype, p, stream);
+}
+
+}  // namespace dcn

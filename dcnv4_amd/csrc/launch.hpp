@@ -1,0 +1,69 @@
+// Host-visible launch descriptors: the C-ABI entry points (capi.hip) fill these and call the
+// launchers defined next to the kernels.  Everything is plain data passed by value to kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace dcn {
+
+// Largest span (bytes) one launch may address through a 32-bit buffer offset.  Value tensors
+// larger than this are cut into batch chunks by the entry points.
+constexpr uint64_t kMaxSpanBytes = 0x7fff0000ull;
+constexpr int kMaxTaps = 64;       // DCNv4: kh*kw - remove_center; attention: L*K
+constexpr int kMaxLevels = 16;
+constexpr int kBlockThreads = 256;
+constexpr size_t kMaxDynamicLds = 64 * 1024;
+
+struct LaneMap {
+  int cpt;          // channels per lane (power of two, cpt * elem_bytes <= 16)
+  int tpg;          // lanes that hold one (pixel, group): D / cpt
+  int tpgp_log2;    // log2 of tpg rounded up to a power of two (cluster width for reductions)
+};
+
+// DCNv4 (reference: DCNv4_op/src/cuda/dcnv4_im2col_cuda.cuh:246-325 launcher arguments)
+struct DcnLaunch {
+  const void *value;        // [n_img, H, W, G*D]
+  const void *offset_mask;  // [n_pix, P_pad]
+  const void *grad_out;     // [n_pix, G*D]            (backward)
+  void *out;                // [n_pix, G*D]            (forward)
+  float *grad_value_acc;    // [n_img, H, W, G*D] fp32, zeroed (backward)
+  void *grad_offset_mask;   // [n_pix, P_pad]          (backward)
+  uint32_t value_bytes;
+  int n_pix;                // images in this launch * Ho * Wo
+  int Q, Wo, H, W, G, D;
+  int kh, kw, sh, sw, ph, pw, dh, dw;
+  int Kp, P_pad, remove_center, softmax;
+  float offset_scale;
+  int npix_block;           // output pixels per workgroup
+  LaneMap lanes;
+};
+
+// Flash deformable attention (reference: DCNv4_op/src/cuda/flash_deform_im2col_cuda.cuh:211-272)
+struct FdaLaunch {
+  const void *value;        // [n_img, N, G, D]
+  const void *sla;          // [n_row, G, 3*L*K]       n_row = images * Q
+  const void *grad_out;     // [n_row, G*D]
+  void *out;                // [n_row, G*D]
+  float *grad_value_acc;    // [n_img, N, G, D] fp32, zeroed
+  void *grad_sla;           // [n_row, G, 3*L*K]
+  const int64_t *shapes;    // [L, 2] (H_l, W_l), device memory
+  const int64_t *level_start;  // [L], device memory
+  uint32_t value_bytes;
+  int n_row;
+  int Q, N, G, D, L, K;
+  int nq_block;             // queries per workgroup
+  LaneMap lanes;
+};
+
+// Each returns hipSuccess or the launch error.  dtype: 0 fp32, 1 fp16, 2 bf16.
+hipError_t launch_dcnv4_forward(int dtype, const DcnLaunch &p, hipStream_t stream);
+hipError_t launch_dcnv4_backward(int dtype, const DcnLaunch &p, hipStream_t stream);
+hipError_t launch_fda_forward(int dtype, const FdaLaunch &p, hipStream_t stream);
+hipError_t launch_fda_backward(int dtype, const FdaLaunch &p, hipStream_t stream);
+
+size_t dcnv4_forward_lds_bytes(const DcnLaunch &p);
+size_t dcnv4_backward_lds_bytes(const DcnLaunch &p);
+size_t fda_forward_lds_bytes(const FdaLaunch &p);
+size_t fda_backward_lds_bytes(const FdaLaunch &p);
+
+}  // namespace dcn

@@ -1,0 +1,151 @@
+"""Drop-in for the reference's ``DCNv4.ext`` pybind module (DCNv4_op/src/vision.cpp:14-21).
+
+Four functions with the reference's positional signatures (DCNv4_op/src/dcnv4.h:19-107).  Each
+checks its tensors the way the reference's host wrappers do (DCNv4_op/src/cuda/dcnv4_cuda.cu:34-60,
+flash_deform_attn_cuda.cu:31-62), allocates the results with torch, and hands raw device pointers
+plus torch's current HIP stream to the C ABI.  ``d_stride`` / ``block_thread`` are launch hints:
+any value the reference accepts is accepted; results never depend on them.
+"""
+import torch
+
+from . import _lib
+
+_L = _lib.load()
+
+_DTYPES = {torch.float32: _lib.DTYPE_F32, torch.float16: _lib.DTYPE_F16, torch.bfloat16: _lib.DTYPE_BF16}
+
+
+def _dtype_code(t, name):
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise RuntimeError(f"{name}: dtype {t.dtype} is not supported on gfx950 (float32, float16, bfloat16)") from None
+
+
+def _check(t, name, dtype=None):
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} tensor has to be contiguous")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor (Not implemented on the CPU)")
+    if dtype is not None and t.dtype != dtype:
+        raise RuntimeError(f"{name} has dtype {t.dtype}, expected {dtype}")
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _hint(v):
+    # the C ABI treats 0 as "choose for me"; the reference's tables only ever pass positive values
+    return int(v) if v is not None else 0
+
+
+def _out_hw(h, w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w):
+    return ((h + 2 * pad_h - (dilation_h * (kernel_h - 1) + 1)) // stride_h + 1,
+            (w + 2 * pad_w - (dilation_w * (kernel_w - 1) + 1)) // stride_w + 1)
+
+
+def dcnv4_forward(value, p_offset, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h,
+                  dilation_w, group, group_channels, offset_scale, im2col_step, remove_center, d_stride,
+                  block_thread, softmax):
+    _check(value, "input")
+    _check(p_offset, "offset", value.dtype)
+    if value.dim() != 4 or p_offset.dim() != 4:
+        raise RuntimeError("input and offset_mask must be 4-d (N, H, W, C)")
+    code = _dtype_code(value, "input")
+    batch, h, w, channels = value.shape
+    if channels != group * group_channels:
+        raise RuntimeError(f"Input channels and group times group channels wont match: ({channels} vs {group * group_channels}).")
+    ho, wo = _out_hw(h, w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w)
+    if tuple(p_offset.shape[:3]) != (batch, ho, wo):
+        raise RuntimeError(f"offset_mask shape {tuple(p_offset.shape)} does not match output ({batch}, {ho}, {wo}, *)")
+    with torch.cuda.device(value.device):
+        output = torch.empty((batch, ho, wo, channels), dtype=value.dtype, device=value.device)
+        _lib.check(_L.dcnv4_gfx950_forward(
+            value.data_ptr(), p_offset.data_ptr(), output.data_ptr(), code, batch, h, w, group, group_channels,
+            kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, float(offset_scale),
+            int(im2col_step), int(remove_center), p_offset.shape[3], int(bool(softmax)), _hint(d_stride),
+            _hint(block_thread), _stream()))
+    return output
+
+
+def dcnv4_backward(value, p_offset, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h,
+                   dilation_w, group, group_channels, offset_scale, im2col_step, grad_output, remove_center,
+                   d_stride, block_thread, softmax):
+    _check(value, "input")
+    _check(p_offset, "offset", value.dtype)
+    _check(grad_output, "grad_output", value.dtype)
+    if value.dim() != 4 or p_offset.dim() != 4:
+        raise RuntimeError("input and offset_mask must be 4-d (N, H, W, C)")
+    code = _dtype_code(value, "input")
+    batch, h, w, channels = value.shape
+    if channels != group * group_channels:
+        raise RuntimeError(f"Input channels and group times group channels wont match: ({channels} vs {group * group_channels}).")
+    ho, wo = _out_hw(h, w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w)
+    if tuple(p_offset.shape[:3]) != (batch, ho, wo) or grad_output.numel() != batch * ho * wo * channels:
+        raise RuntimeError("offset_mask / grad_output shapes do not match the output extent")
+    with torch.cuda.device(value.device):
+        grad_input = torch.empty_like(value)
+        grad_offset = torch.empty_like(p_offset)
+        ws_bytes = _L.dcnv4_gfx950_backward_workspace_bytes(code, batch, h, w, group, group_channels)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=value.device) if ws_bytes else None
+        _lib.check(_L.dcnv4_gfx950_backward(
+            value.data_ptr(), p_offset.data_ptr(), grad_output.data_ptr(), grad_input.data_ptr(),
+            grad_offset.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes, code, batch, h, w, group,
+            group_channels, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w,
+            float(offset_scale), int(im2col_step), int(remove_center), p_offset.shape[3], int(bool(softmax)),
+            _hint(d_stride), _hint(block_thread), _stream()))
+    return [grad_input, grad_offset]
+
+
+def _fda_common(value, spatial_shapes, level_start_index, sampling_loc_attn, K):
+    _check(value, "value")
+    _check(spatial_shapes, "spatial_shapes", torch.int64)
+    _check(level_start_index, "level_start_index", torch.int64)
+    _check(sampling_loc_attn, "sampling_loc_attn", value.dtype)
+    if value.dim() != 4 or sampling_loc_attn.dim() != 4:
+        raise RuntimeError("value must be (N, S, M, D) and sampling_loc_attn (N, Lq, M, L*K*3)")
+    batch, spatial_size, num_heads, channels = value.shape
+    num_levels = spatial_shapes.shape[0]
+    num_query = sampling_loc_attn.shape[1]
+    if level_start_index.numel() != num_levels:
+        raise RuntimeError("level_start_index must have one entry per level")
+    if tuple(sampling_loc_attn.shape) != (batch, num_query, num_heads, num_levels * K * 3):
+        raise RuntimeError(f"sampling_loc_attn shape {tuple(sampling_loc_attn.shape)} != "
+                           f"{(batch, num_query, num_heads, num_levels * K * 3)}")
+    return batch, spatial_size, num_heads, channels, num_levels, num_query
+
+
+def flash_deform_attn_forward(value, spatial_shapes, level_start_index, sampling_loc_attn, im2col_step=64, K=8,
+                              d_stride=8, block_thread=0):
+    batch, spatial_size, num_heads, channels, num_levels, num_query = _fda_common(
+        value, spatial_shapes, level_start_index, sampling_loc_attn, K)
+    code = _dtype_code(value, "value")
+    with torch.cuda.device(value.device):
+        output = torch.empty((batch, num_query, num_heads * channels), dtype=value.dtype, device=value.device)
+        _lib.check(_L.flash_deform_attn_gfx950_forward(
+            value.data_ptr(), spatial_shapes.data_ptr(), level_start_index.data_ptr(), sampling_loc_attn.data_ptr(),
+            output.data_ptr(), code, batch, spatial_size, num_heads, channels, num_levels, num_query, int(K),
+            int(im2col_step), _hint(d_stride), _hint(block_thread), _stream()))
+    return output
+
+
+def flash_deform_attn_backward(value, spatial_shapes, level_start_index, sampling_loc_attn, grad_output,
+                               im2col_step=64, K=8, d_stride=2, block_thread=0):
+    batch, spatial_size, num_heads, channels, num_levels, num_query = _fda_common(
+        value, spatial_shapes, level_start_index, sampling_loc_attn, K)
+    _check(grad_output, "grad_output", value.dtype)
+    if grad_output.numel() != batch * num_query * num_heads * channels:
+        raise RuntimeError("grad_output shape does not match the output")
+    code = _dtype_code(value, "value")
+    with torch.cuda.device(value.device):
+        grad_value = torch.empty_like(value)
+        grad_sla = torch.empty_like(sampling_loc_attn)
+        ws_bytes = _L.flash_deform_attn_gfx950_backward_workspace_bytes(code, batch, spatial_size, num_heads, channels)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=value.device) if ws_bytes else None
+        _lib.check(_L.flash_deform_attn_gfx950_backward(
+            value.data_ptr(), spatial_shapes.data_ptr(), level_start_index.data_ptr(), sampling_loc_attn.data_ptr(),
+            grad_output.data_ptr(), grad_value.data_ptr(), grad_sla.data_ptr(),
+            ws.data_ptr() if ws is not None else None, ws_bytes, code, batch, spatial_size, num_heads, channels,
+            num_levels, num_query, int(K), int(im2col_step), _hint(d_stride), _hint(block_thread), _stream()))
+    return [grad_value, grad_sla]

@@ -1,0 +1,132 @@
+/*
+ * C ABI of libdcnv4_gfx950.so: the DCNv4 deformable convolution and flash deformable
+ * attention operators for AMD MI355X (gfx950).
+ *
+ * These four operators are what the reference exposes to Python as the pybind11 module
+ * `DCNv4.ext` (DCNv4_op/src/vision.cpp:14-21, prototypes DCNv4_op/src/dcnv4.h:19-107).  Here
+ * they are plain C functions over raw device pointers so that any host language can bind
+ * them; tensor allocation, dtype discovery and stream lookup stay with the caller.
+ *
+ * Conventions
+ *   - every data pointer is device memory, dense row-major, 16-byte aligned;
+ *   - `dtype` is one of DCNV4_DTYPE_*; all tensors of a call share it; arithmetic is fp32;
+ *   - `stream` is a hipStream_t (NULL = the default stream); calls only enqueue work, they
+ *     never synchronise, allocate or free;
+ *   - the return value is DCNV4_OK or an error code; dcnv4_gfx950_last_error() then holds a
+ *     message for the calling thread.  DCNV4_ERR_INVALID_ARGUMENT corresponds to the
+ *     reference's std::invalid_argument (ValueError in Python: unsupported kernel shape, level
+ *     count, channel stride); DCNV4_ERR_RUNTIME to its AT_ASSERTM / launch failures
+ *     (RuntimeError in Python);
+ *   - `d_stride` (channels per lane) and `block_thread` (lanes per workgroup) are the
+ *     reference's launch hints; 0 lets the library choose.  Results do not depend on them.
+ */
+#ifndef DCNV4_GFX950_H
+#define DCNV4_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DCNV4_GFX950_ABI_VERSION 1
+
+#define DCNV4_DTYPE_F32 0
+#define DCNV4_DTYPE_F16 1
+#define DCNV4_DTYPE_BF16 2
+
+#define DCNV4_OK 0
+#define DCNV4_ERR_INVALID_ARGUMENT 1
+#define DCNV4_ERR_RUNTIME 2
+
+/* ABI version of the loaded library (DCNV4_GFX950_ABI_VERSION it was built with). */
+int dcnv4_gfx950_abi_version(void);
+
+/* Message of the last failed call on this thread ("" if none). The pointer stays valid until
+ * the next failing call on the same thread. */
+const char *dcnv4_gfx950_last_error(void);
+
+/*
+ * DCNv4 forward.  Replaces dcnv4_forward / dcnv4_cuda_forward
+ * (DCNv4_op/src/dcnv4.h:64-83, DCNv4_op/src/cuda/dcnv4_cuda.cu:26-90).
+ *   value        [batch, height_in, width_in, group*group_channels]
+ *   offset_mask  [batch, height_out, width_out, padded_offset_dim]; per group 2K offsets
+ *                (x,y interleaved, kernel-tap order x-major) then K modulation scalars,
+ *                K = kernel_h*kernel_w - remove_center; tail up to padded_offset_dim unused
+ *   output       [batch, height_out, width_out, group*group_channels]  (fully overwritten)
+ *   height_out = (height_in + 2*pad_h - (dilation_h*(kernel_h-1)+1)) / stride_h + 1, same for w
+ *   softmax != 0 normalises the K modulation scalars of a group with a softmax
+ */
+int dcnv4_gfx950_forward(const void *value, const void *offset_mask, void *output, int dtype,
+                         int batch, int height_in, int width_in, int group, int group_channels,
+                         int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h,
+                         int pad_w, int dilation_h, int dilation_w, float offset_scale,
+                         int im2col_step, int remove_center, int padded_offset_dim, int softmax,
+                         int d_stride, int block_thread, void *stream);
+
+/* Scratch bytes dcnv4_gfx950_backward needs for these sizes (0 for fp32). */
+size_t dcnv4_gfx950_backward_workspace_bytes(int dtype, int batch, int height_in, int width_in,
+                                             int group, int group_channels);
+
+/*
+ * DCNv4 backward.  Replaces dcnv4_backward / dcnv4_cuda_backward
+ * (DCNv4_op/src/dcnv4.h:85-107, DCNv4_op/src/cuda/dcnv4_cuda.cu:92-175).
+ *   grad_output       like output
+ *   grad_value        like value        (fully overwritten; need not be cleared)
+ *   grad_offset_mask  like offset_mask  (fully overwritten, tail = 0)
+ *   workspace         device scratch of at least ..._workspace_bytes(), 16-byte aligned;
+ *                     contents are destroyed; may be NULL when the size is 0
+ */
+int dcnv4_gfx950_backward(const void *value, const void *offset_mask, const void *grad_output,
+                          void *grad_value, void *grad_offset_mask, void *workspace,
+                          size_t workspace_bytes, int dtype, int batch, int height_in,
+                          int width_in, int group, int group_channels, int kernel_h, int kernel_w,
+                          int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h,
+                          int dilation_w, float offset_scale, int im2col_step, int remove_center,
+                          int padded_offset_dim, int softmax, int d_stride, int block_thread,
+                          void *stream);
+
+/*
+ * Flash deformable attention forward.  Replaces flash_deform_attn_forward /
+ * flash_deform_attn_cuda_forward (DCNv4_op/src/dcnv4.h:19-36,
+ * DCNv4_op/src/cuda/flash_deform_attn_cuda.cu:26-84).
+ *   value              [batch, spatial_size, num_heads, head_channels]
+ *   spatial_shapes     [num_levels, 2] int64 (H_l, W_l), device memory
+ *   level_start_index  [num_levels] int64, device memory
+ *   sampling_loc_attn  [batch, num_query, num_heads, num_levels*num_points*3]: 2*L*K
+ *                      normalised (x,y) locations then L*K attention logits
+ *   output             [batch, num_query, num_heads*head_channels]  (fully overwritten)
+ */
+int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_shapes,
+                                     const int64_t *level_start_index,
+                                     const void *sampling_loc_attn, void *output, int dtype,
+                                     int batch, int spatial_size, int num_heads,
+                                     int head_channels, int num_levels, int num_query,
+                                     int num_points, int im2col_step, int d_stride,
+                                     int block_thread, void *stream);
+
+size_t flash_deform_attn_gfx950_backward_workspace_bytes(int dtype, int batch, int spatial_size,
+                                                         int num_heads, int head_channels);
+
+/*
+ * Flash deformable attention backward.  Replaces flash_deform_attn_backward /
+ * flash_deform_attn_cuda_backward (DCNv4_op/src/dcnv4.h:38-62,
+ * DCNv4_op/src/cuda/flash_deform_attn_cuda.cu:86-163).
+ *   grad_value like value, grad_sampling_loc_attn like sampling_loc_attn; both fully
+ *   overwritten.  A tap outside its level contributes zero to the softmax Jacobian.
+ */
+int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_shapes,
+                                      const int64_t *level_start_index,
+                                      const void *sampling_loc_attn, const void *grad_output,
+                                      void *grad_value, void *grad_sampling_loc_attn,
+                                      void *workspace, size_t workspace_bytes, int dtype,
+                                      int batch, int spatial_size, int num_heads,
+                                      int head_channels, int num_levels, int num_query,
+                                      int num_points, int im2col_step, int d_stride,
+                                      int block_thread, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DCNV4_GFX950_H */

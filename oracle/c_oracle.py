@@ -1,5 +1,9 @@
 """TEST INFRASTRUCTURE ONLY: numpy/ctypes front end of oracle/sampling_oracle.c.
 
+``coord_f32=True`` rounds the sampling-coordinate arithmetic to fp32 the way the reference's
+kernels do for fp32/fp16/bf16 tensors (the mode GPU parity tests use); the default keeps
+everything in float64 (the mode the mathematical pins use).
+
 Every function takes and returns float64 numpy arrays in the operators' own
 layouts (NHWC value, packed offset_mask, packed sampling_loc_attn) and follows the
 reference's host wrappers for shapes: DCNv4_op/src/cuda/dcnv4_cuda.cu:26-175,
@@ -31,11 +35,11 @@ def lib():
     if _lib is None:
         _lib = ctypes.CDLL(build())
         i, d = ctypes.c_int, ctypes.c_double
-        dcn_tail = [i] * 13 + [d, i, i, i]
+        dcn_tail = [i] * 13 + [d, i, i, i, i]
         _lib.oracle_dcnv4_forward.argtypes = [_dp, _dp, _dp] + dcn_tail
         _lib.oracle_dcnv4_backward.argtypes = [_dp, _dp, _dp, _dp, _dp] + dcn_tail
-        _lib.oracle_flash_deform_attn_forward.argtypes = [_dp, _ip, _ip, _dp, _dp] + [i] * 7
-        _lib.oracle_flash_deform_attn_backward.argtypes = [_dp, _ip, _ip, _dp, _dp, _dp, _dp] + [i] * 7
+        _lib.oracle_flash_deform_attn_forward.argtypes = [_dp, _ip, _ip, _dp, _dp] + [i] * 8
+        _lib.oracle_flash_deform_attn_backward.argtypes = [_dp, _ip, _ip, _dp, _dp, _dp, _dp] + [i] * 8
         _lib.oracle_out_extent.argtypes = [i] * 5
         _lib.oracle_out_extent.restype = i
         for f in (_lib.oracle_dcnv4_forward, _lib.oracle_dcnv4_backward,
@@ -74,19 +78,19 @@ def _dcn_check(value, offset_mask, kh, kw, sh, sw, ph, pw, dh, dw, group, group_
 
 
 def dcnv4_forward(value, offset_mask, kh, kw, sh, sw, ph, pw, dh, dw, group, group_channels,
-                  offset_scale, remove_center=0, softmax=False):
+                  offset_scale, remove_center=0, softmax=False, coord_f32=False):
     value, offset_mask = _f64(value), _f64(offset_mask)
     B, H, W, Ho, Wo, P_pad = _dcn_check(value, offset_mask, kh, kw, sh, sw, ph, pw, dh, dw, group,
                                         group_channels, remove_center)
     out = np.empty((B, Ho, Wo, group * group_channels), dtype=np.float64)
     lib().oracle_dcnv4_forward(_p(value), _p(offset_mask), _p(out), B, H, W, group, group_channels,
                                kh, kw, sh, sw, ph, pw, dh, dw, float(offset_scale),
-                               int(bool(remove_center)), int(bool(softmax)), P_pad)
+                               int(bool(remove_center)), int(bool(softmax)), P_pad, int(bool(coord_f32)))
     return out
 
 
 def dcnv4_backward(value, offset_mask, grad_out, kh, kw, sh, sw, ph, pw, dh, dw, group,
-                   group_channels, offset_scale, remove_center=0, softmax=False):
+                   group_channels, offset_scale, remove_center=0, softmax=False, coord_f32=False):
     value, offset_mask, grad_out = _f64(value), _f64(offset_mask), _f64(grad_out)
     B, H, W, Ho, Wo, P_pad = _dcn_check(value, offset_mask, kh, kw, sh, sw, ph, pw, dh, dw, group,
                                         group_channels, remove_center)
@@ -95,7 +99,7 @@ def dcnv4_backward(value, offset_mask, grad_out, kh, kw, sh, sw, ph, pw, dh, dw,
     gv, gom = np.empty_like(value), np.empty_like(offset_mask)
     lib().oracle_dcnv4_backward(_p(value), _p(offset_mask), _p(grad_out), _p(gv), _p(gom), B, H, W,
                                 group, group_channels, kh, kw, sh, sw, ph, pw, dh, dw,
-                                float(offset_scale), int(bool(remove_center)), int(bool(softmax)), P_pad)
+                                float(offset_scale), int(bool(remove_center)), int(bool(softmax)), P_pad, int(bool(coord_f32)))
     return gv, gom
 
 
@@ -110,16 +114,16 @@ def _fda_check(value, shapes, level_start, sla, K):
     return B, N, G, D, L, Q
 
 
-def flash_deform_attn_forward(value, shapes, level_start, sla, K):
+def flash_deform_attn_forward(value, shapes, level_start, sla, K, coord_f32=False):
     value, sla, shapes, level_start = _f64(value), _f64(sla), _i64(shapes), _i64(level_start)
     B, N, G, D, L, Q = _fda_check(value, shapes, level_start, sla, K)
     out = np.empty((B, Q, G * D), dtype=np.float64)
     lib().oracle_flash_deform_attn_forward(_p(value), _p(shapes), _p(level_start), _p(sla), _p(out),
-                                           B, N, G, D, L, K, Q)
+                                           B, N, G, D, L, K, Q, int(bool(coord_f32)))
     return out
 
 
-def flash_deform_attn_backward(value, shapes, level_start, sla, grad_out, K):
+def flash_deform_attn_backward(value, shapes, level_start, sla, grad_out, K, coord_f32=False):
     value, sla, grad_out = _f64(value), _f64(sla), _f64(grad_out)
     shapes, level_start = _i64(shapes), _i64(level_start)
     B, N, G, D, L, Q = _fda_check(value, shapes, level_start, sla, K)
@@ -127,5 +131,5 @@ def flash_deform_attn_backward(value, shapes, level_start, sla, grad_out, K):
         raise ValueError("grad_out shape")
     gv, gs = np.empty_like(value), np.empty_like(sla)
     lib().oracle_flash_deform_attn_backward(_p(value), _p(shapes), _p(level_start), _p(sla),
-                                            _p(grad_out), _p(gv), _p(gs), B, N, G, D, L, K, Q)
+                                            _p(grad_out), _p(gv), _p(gs), B, N, G, D, L, K, Q, int(bool(coord_f32)))
     return gv, gs

@@ -24,6 +24,12 @@
  * reference reads an unwritten shared-memory slot there,
  * flash_deform_col2im_cuda.cuh:272-293).
  *
+ * Coordinate precision: the reference forms every sampling coordinate in its opmath type, which
+ * is fp32 for fp32/fp16/bf16 tensors (dcnv4_im2col_cuda.cuh:203-224, flash_deform_im2col_cuda.cuh:
+ * 184-189).  With coord32 != 0 the oracle rounds exactly those operations to fp32, in source
+ * order and without fused multiply-add, and does everything downstream (weights, sums) in
+ * double; with coord32 == 0 coordinates are double too (the mathematical ideal the pins use).
+ *
  * All tensors are dense row-major double arrays in the operator's own layouts.
  * Loops over the batch run under OpenMP; every image is independent, so the
  * gradient scatter needs no atomics.
@@ -77,6 +83,7 @@ int oracle_out_extent(int in, int pad, int dil, int k, int stride) {
 typedef struct {
   int B, H, W, G, D, kh, kw, sh, sw, ph, pw, dh, dw, remove_center, softmax, P_pad;
   double offset_scale;
+  int coord32;
 } dcn_args_t;
 
 /* Sampling position of kernel tap (i = x index, j = y index) for output pixel
@@ -85,16 +92,33 @@ static inline void dcn_position(const dcn_args_t *a, int ho, int wo, int i, int 
                                 double off_x, double off_y, double *y, double *x) {
   const int half_w = (a->dw * (a->kw - 1)) >> 1, half_h = (a->dh * (a->kh - 1)) >> 1;
   const int p0_w = half_w - a->pw + wo * a->sw, p0_h = half_h - a->ph + ho * a->sh;
+  if (a->coord32) {       /* every operation rounded to fp32; built with -ffp-contract=off */
+    const float sc = (float)a->offset_scale;
+    const float bx = (float)p0_w - (float)half_w * sc, by = (float)p0_h - (float)half_h * sc;
+    const float tx = ((float)(i * a->dw) + (float)off_x) * sc, ty = ((float)(j * a->dh) + (float)off_y) * sc;
+    *x = (double)(bx + tx);
+    *y = (double)(by + ty);
+    return;
+  }
   *x = (p0_w - half_w * a->offset_scale) + (i * a->dw + off_x) * a->offset_scale;
   *y = (p0_h - half_h * a->offset_scale) + (j * a->dh + off_y) * a->offset_scale;
+}
+
+/* Attention tap position: loc * extent - 0.5 (flash_deform_im2col_cuda.cuh:188-189). */
+static inline double fda_position(double loc, int extent, int coord32) {
+  if (coord32) {
+    const float prod = (float)loc * (float)extent;
+    return (double)(prod - 0.5f);
+  }
+  return loc * extent - 0.5;
 }
 
 void oracle_dcnv4_forward(const double *value, const double *offset_mask, double *out,
                           int B, int H, int W, int G, int D, int kh, int kw, int sh, int sw,
                           int ph, int pw, int dh, int dw, double offset_scale,
-                          int remove_center, int softmax, int P_pad) {
+                          int remove_center, int softmax, int P_pad, int coord32) {
   dcn_args_t a = {B, H, W, G, D, kh, kw, sh, sw, ph, pw, dh, dw, remove_center, softmax, P_pad,
-                  offset_scale};
+                  offset_scale, coord32};
   const int Ho = oracle_out_extent(H, ph, dh, kh, sh), Wo = oracle_out_extent(W, pw, dw, kw, sw);
   const int Kp = kh * kw - (remove_center ? 1 : 0), C = G * D;
 #pragma omp parallel for collapse(2) schedule(static)
@@ -132,9 +156,9 @@ void oracle_dcnv4_backward(const double *value, const double *offset_mask, const
                            double *grad_value, double *grad_om,
                            int B, int H, int W, int G, int D, int kh, int kw, int sh, int sw,
                            int ph, int pw, int dh, int dw, double offset_scale,
-                           int remove_center, int softmax, int P_pad) {
+                           int remove_center, int softmax, int P_pad, int coord32) {
   dcn_args_t a = {B, H, W, G, D, kh, kw, sh, sw, ph, pw, dh, dw, remove_center, softmax, P_pad,
-                  offset_scale};
+                  offset_scale, coord32};
   const int Ho = oracle_out_extent(H, ph, dh, kh, sh), Wo = oracle_out_extent(W, pw, dw, kw, sw);
   const int Kp = kh * kw - (remove_center ? 1 : 0), C = G * D;
   memset(grad_value, 0, sizeof(double) * (size_t)B * H * W * C);
@@ -188,7 +212,7 @@ void oracle_dcnv4_backward(const double *value, const double *offset_mask, const
 
 void oracle_flash_deform_attn_forward(const double *value, const int64_t *shapes,
                                       const int64_t *level_start, const double *sla, double *out,
-                                      int B, int N, int G, int D, int L, int K, int Q) {
+                                      int B, int N, int G, int D, int L, int K, int Q, int coord32) {
   const int LK = L * K;
 #pragma omp parallel for collapse(2) schedule(static)
   for (int b = 0; b < B; ++b)
@@ -205,7 +229,7 @@ void oracle_flash_deform_attn_forward(const double *value, const int64_t *shapes
           const int Hl = (int)shapes[2 * l], Wl = (int)shapes[2 * l + 1];
           for (int k = 0; k < K; ++k) {
             const int t = l * K + k; tap_t tp;
-            const double x = s[2 * t] * Wl - 0.5, y = s[2 * t + 1] * Hl - 0.5;   /* :188-189 */
+            const double x = fda_position(s[2 * t], Wl, coord32), y = fda_position(s[2 * t + 1], Hl, coord32);
             if (!make_tap(y, x, Hl, Wl, &tp)) continue;
             for (int cn = 0; cn < 4; ++cn) {
               if (!tp.ok[cn]) continue;
@@ -222,7 +246,7 @@ void oracle_flash_deform_attn_forward(const double *value, const int64_t *shapes
 void oracle_flash_deform_attn_backward(const double *value, const int64_t *shapes,
                                        const int64_t *level_start, const double *sla,
                                        const double *grad_out, double *grad_value, double *grad_sla,
-                                       int B, int N, int G, int D, int L, int K, int Q) {
+                                       int B, int N, int G, int D, int L, int K, int Q, int coord32) {
   const int LK = L * K;
   memset(grad_value, 0, sizeof(double) * (size_t)B * N * G * D);
   memset(grad_sla, 0, sizeof(double) * (size_t)B * Q * G * 3 * LK);
@@ -241,7 +265,7 @@ void oracle_flash_deform_attn_backward(const double *value, const int64_t *shape
           const int Hl = (int)shapes[2 * l], Wl = (int)shapes[2 * l + 1];
           for (int k = 0; k < K; ++k) {
             const int t = l * K + k; tap_t tp;
-            const double x = s[2 * t] * Wl - 0.5, y = s[2 * t + 1] * Hl - 0.5;
+            const double x = fda_position(s[2 * t], Wl, coord32), y = fda_position(s[2 * t + 1], Hl, coord32);
             double gx = 0.0, gy = 0.0, gz = 0.0;
             if (make_tap(y, x, Hl, Wl, &tp))
               for (int cn = 0; cn < 4; ++cn) {

@@ -1,0 +1,87 @@
+"""Test-side helpers that call libdcnv4_gfx950.so through its C ABI with torch tensors as device memory,
+and run the CPU oracle on the same bits."""
+import numpy as np
+import torch
+
+from dcnv4_amd import _lib
+
+CODES = {torch.float32: _lib.DTYPE_F32, torch.float16: _lib.DTYPE_F16, torch.bfloat16: _lib.DTYPE_BF16}
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def dcn_out_hw(H, W, kh, kw, sh, sw, ph, pw, dh, dw):
+    return ((H + 2 * ph - (dh * (kh - 1) + 1)) // sh + 1, (W + 2 * pw - (dw * (kw - 1) + 1)) // sw + 1)
+
+
+def dcnv4_forward(value, om, geom, G, D, scale, rc=0, softmax=0, im2col_step=256, d_stride=0, block_thread=0):
+    L = _lib.load()
+    B, H, W, _ = value.shape
+    Ho, Wo = dcn_out_hw(H, W, *geom)
+    out = torch.full((B, Ho, Wo, G * D), float("nan"), dtype=value.dtype, device=value.device)
+    rc_ = L.dcnv4_gfx950_forward(value.data_ptr(), om.data_ptr(), out.data_ptr(), CODES[value.dtype], B, H, W, G, D,
+                                 *geom, float(scale), im2col_step, rc, om.shape[-1], softmax, d_stride, block_thread,
+                                 _stream())
+    _lib.check(rc_)
+    return out
+
+
+def dcnv4_backward(value, om, go, geom, G, D, scale, rc=0, softmax=0, im2col_step=256, d_stride=0, block_thread=0):
+    L = _lib.load()
+    B, H, W, _ = value.shape
+    gv = torch.full_like(value, float("nan"))
+    gom = torch.full_like(om, float("nan"))
+    nbytes = L.dcnv4_gfx950_backward_workspace_bytes(CODES[value.dtype], B, H, W, G, D)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=value.device)
+    rc_ = L.dcnv4_gfx950_backward(value.data_ptr(), om.data_ptr(), go.data_ptr(), gv.data_ptr(), gom.data_ptr(),
+                                  ws.data_ptr(), nbytes, CODES[value.dtype], B, H, W, G, D, *geom, float(scale),
+                                  im2col_step, rc, om.shape[-1], softmax, d_stride, block_thread, _stream())
+    _lib.check(rc_)
+    return gv, gom
+
+
+def fda_forward(value, shapes, starts, sla, K, im2col_step=64, d_stride=0, block_thread=0):
+    L = _lib.load()
+    B, N, G, D = value.shape
+    Q = sla.shape[1]
+    out = torch.full((B, Q, G * D), float("nan"), dtype=value.dtype, device=value.device)
+    rc_ = L.flash_deform_attn_gfx950_forward(value.data_ptr(), shapes.data_ptr(), starts.data_ptr(), sla.data_ptr(),
+                                             out.data_ptr(), CODES[value.dtype], B, N, G, D, shapes.shape[0], Q, K,
+                                             im2col_step, d_stride, block_thread, _stream())
+    _lib.check(rc_)
+    return out
+
+
+def fda_backward(value, shapes, starts, sla, go, K, im2col_step=64, d_stride=0, block_thread=0):
+    L = _lib.load()
+    B, N, G, D = value.shape
+    Q = sla.shape[1]
+    gv = torch.full_like(value, float("nan"))
+    gs = torch.full_like(sla, float("nan"))
+    nbytes = L.flash_deform_attn_gfx950_backward_workspace_bytes(CODES[value.dtype], B, N, G, D)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=value.device)
+    rc_ = L.flash_deform_attn_gfx950_backward(value.data_ptr(), shapes.data_ptr(), starts.data_ptr(), sla.data_ptr(),
+                                              go.data_ptr(), gv.data_ptr(), gs.data_ptr(), ws.data_ptr(), nbytes,
+                                              CODES[value.dtype], B, N, G, D, shapes.shape[0], Q, K, im2col_step,
+                                              d_stride, block_thread, _stream())
+    _lib.check(rc_)
+    return gv, gs
+
+
+def f64(t):
+    """Exact widening of a (possibly half-precision) tensor to a float64 numpy array."""
+    return t.detach().cpu().to(torch.float64).numpy()
+
+
+def assert_close(got, want, rtol, atol, what=""):
+    got = f64(got) if isinstance(got, torch.Tensor) else got
+    assert np.isfinite(got).all(), f"{what}: non-finite values (unwritten output?)"
+    err = np.abs(got - want)
+    tol = atol + rtol * np.abs(want)
+    bad = err > tol
+    if bad.any():
+        i = np.unravel_index(np.argmax(err - tol), err.shape)
+        raise AssertionError(f"{what}: {bad.sum()} / {bad.size} elements off; worst at {i}: got {got[i]!r} want {want[i]!r} "
+                             f"(rtol {rtol}, atol {atol})")

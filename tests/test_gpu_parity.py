@@ -1,0 +1,188 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle on identical bits.
+
+Tolerances (stated by the task for this path): forward rtol 1e-4 / atol 1e-5 in fp32 and 1e-2 in
+fp16; gradients 1e-3 relative in fp32 (atomic summation order differs run to run).  The oracle is
+always fed the dtype-quantised inputs widened exactly to float64.
+"""
+import zlib
+
+import numpy as np
+import pytest
+import torch
+
+from tests import cabi
+from tests.inputs import make_dcnv4_inputs, make_fda_inputs
+
+pytestmark = pytest.mark.gpu
+
+FWD_TOL = {torch.float32: (1e-4, 1e-5), torch.float16: (1e-2, 1e-3), torch.bfloat16: (2e-2, 2e-2)}
+GRAD_TOL = {torch.float32: (1e-3, 1e-4), torch.float16: (1e-2, 1e-2), torch.bfloat16: (4e-2, 8e-2)}
+
+# B, H, W, G, D, (kh, kw, sh, sw, ph, pw, dh, dw), remove_center, offset_scale, offset_range
+DCN_CASES = {
+    "cfg1_56x56_c64_g4": (2, 56, 56, 4, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
+    "stage_28x28_c128_g8": (3, 28, 28, 8, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 3.0),
+    "stage_7x7_c512_g32": (5, 7, 7, 32, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 3.0),
+    "wide_g80": (1, 9, 11, 80, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 4.0),
+    "g7_c112_scale_half": (2, 14, 14, 7, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 0.5, 3.0),
+    "remove_center": (2, 12, 10, 4, 16, (3, 3, 1, 1, 1, 1, 1, 1), 1, 1.3, 2.5),
+    "stride2": (2, 15, 17, 3, 16, (3, 3, 2, 2, 1, 1, 1, 1), 0, 2.0, 2.0),
+    "dilation2_pad2": (1, 13, 12, 2, 32, (3, 3, 1, 1, 2, 2, 2, 2), 0, 1.0, 1.5),
+    "kernel_1x3_mixed_pad": (1, 9, 8, 2, 8, (1, 3, 1, 1, 0, 1, 1, 1), 0, 0.7, 2.0),
+    "kernel_5x5": (1, 10, 10, 2, 16, (5, 5, 1, 1, 2, 2, 1, 1), 0, 1.0, 2.0),
+    "kernel_3x1_stride_2x1": (1, 10, 9, 2, 4, (3, 1, 2, 1, 2, 0, 2, 1), 0, 1.0, 2.0),
+    "d1_scalar_lanes": (1, 6, 7, 5, 1, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
+    "d6_three_lane_cluster": (2, 6, 5, 3, 6, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
+    "d48_six_lane_cluster": (1, 8, 8, 2, 48, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
+    "d64": (1, 8, 9, 2, 64, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
+    "far_offsets_mostly_outside": (1, 5, 5, 4, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 9.0),
+    "single_pixel": (1, 1, 1, 1, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 1.0),
+}
+
+
+def _dcn_inputs(case, dtype, seed=0):
+    B, H, W, G, D, geom, rc, scale, rng = case
+    v, om, go = make_dcnv4_inputs(B, H, W, G, D, *geom, remove_center=rc, offset_range=rng, seed=seed, dtype=dtype)
+    return v, om, go, (geom, G, D, scale, rc)
+
+
+def _oracle_args(geom, G, D, scale, rc):
+    return (*geom, G, D, scale, rc)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("name", list(DCN_CASES))
+def test_dcnv4_forward_and_backward_match_oracle(oracle, name, dtype):
+    v, om, go, (geom, G, D, scale, rc) = _dcn_inputs(DCN_CASES[name], dtype, seed=zlib.crc32(name.encode()) % 1000)
+    print(f"case {name} dtype {dtype}", flush=True)
+    want = oracle.dcnv4_forward(cabi.f64(v), cabi.f64(om), *_oracle_args(geom, G, D, scale, rc), coord_f32=True)
+    wgv, wgom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *_oracle_args(geom, G, D, scale, rc), coord_f32=True)
+    vd, omd, god = v.cuda(), om.cuda(), go.cuda()
+    out = cabi.dcnv4_forward(vd, omd, geom, G, D, scale, rc)
+    gv, gom = cabi.dcnv4_backward(vd, omd, god, geom, G, D, scale, rc)
+    torch.cuda.synchronize()
+    cabi.assert_close(out, want, *FWD_TOL[dtype], what="output")
+    cabi.assert_close(gv, wgv, *GRAD_TOL[dtype], what="grad_value")
+    cabi.assert_close(gom, wgom, *GRAD_TOL[dtype], what="grad_offset_mask")
+    used = G * 3 * (geom[0] * geom[1] - rc)
+    assert (gom[..., used:] == 0).all(), "padded tail of grad_offset_mask must be exactly zero"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16], ids=["fp32", "fp16"])
+def test_dcnv4_softmax_flag_matches_oracle(oracle, dtype):
+    v, om, go, (geom, G, D, scale, rc) = _dcn_inputs(DCN_CASES["remove_center"], dtype, seed=5)
+    args = _oracle_args(geom, G, D, scale, rc)
+    want = oracle.dcnv4_forward(cabi.f64(v), cabi.f64(om), *args, softmax=True, coord_f32=True)
+    wgv, wgom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *args, softmax=True, coord_f32=True)
+    out = cabi.dcnv4_forward(v.cuda(), om.cuda(), geom, G, D, scale, rc, softmax=1)
+    gv, gom = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), geom, G, D, scale, rc, softmax=1)
+    cabi.assert_close(out, want, *FWD_TOL[dtype], what="output")
+    cabi.assert_close(gv, wgv, *GRAD_TOL[dtype], what="grad_value")
+    cabi.assert_close(gom, wgom, *GRAD_TOL[dtype], what="grad_offset_mask")
+
+
+def test_dcnv4_unpadded_offset_mask_rows(oracle):
+    # P_pad = G*K*3 = 54, not a multiple of 8: rows are not 16-byte aligned, scalar staging path
+    B, H, W, G, D = 2, 6, 7, 2, 16
+    geom = (3, 3, 1, 1, 1, 1, 1, 1)
+    v, om, go = make_dcnv4_inputs(B, H, W, G, D, seed=3, dtype=torch.float16)
+    om = om[..., :54].contiguous()
+    args = (*geom, G, D, 1.0, 0)
+    want = oracle.dcnv4_forward(cabi.f64(v), cabi.f64(om), *args, coord_f32=True)
+    wgv, wgom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *args, coord_f32=True)
+    out = cabi.dcnv4_forward(v.cuda(), om.cuda(), geom, G, D, 1.0)
+    gv, gom = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), geom, G, D, 1.0)
+    cabi.assert_close(out, want, *FWD_TOL[torch.float16], what="output")
+    cabi.assert_close(gv, wgv, *GRAD_TOL[torch.float16], what="grad_value")
+    cabi.assert_close(gom, wgom, *GRAD_TOL[torch.float16], what="grad_offset_mask")
+
+
+@pytest.mark.parametrize("d_stride,block_thread", [(1, 64), (2, 128), (4, 512), (8, 1024), (16, 32)])
+def test_dcnv4_launch_hints_do_not_change_results(oracle, d_stride, block_thread):
+    v, om, go, (geom, G, D, scale, rc) = _dcn_inputs(DCN_CASES["g7_c112_scale_half"], torch.float16, seed=9)
+    args = _oracle_args(geom, G, D, scale, rc)
+    want = oracle.dcnv4_forward(cabi.f64(v), cabi.f64(om), *args, coord_f32=True)
+    wgv, wgom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *args, coord_f32=True)
+    out = cabi.dcnv4_forward(v.cuda(), om.cuda(), geom, G, D, scale, rc, d_stride=d_stride, block_thread=block_thread)
+    gv, gom = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), geom, G, D, scale, rc, d_stride=d_stride,
+                                  block_thread=block_thread)
+    cabi.assert_close(out, want, *FWD_TOL[torch.float16], what="output")
+    cabi.assert_close(gv, wgv, *GRAD_TOL[torch.float16], what="grad_value")
+    cabi.assert_close(gom, wgom, *GRAD_TOL[torch.float16], what="grad_offset_mask")
+
+
+def test_dcnv4_zero_offsets_unit_mask_is_box_sum_on_gpu():
+    B, H, W, G, D, K = 2, 20, 24, 4, 16, 9
+    v, om, _ = make_dcnv4_inputs(B, H, W, G, D, seed=1)
+    om.zero_()
+    body = om[..., : G * K * 3].reshape(B, H, W, G, K * 3)
+    body[..., 2 * K:] = 1.0
+    out = cabi.dcnv4_forward(v.cuda(), om.cuda(), (3, 3, 1, 1, 1, 1, 1, 1), G, D, 1.0)
+    box = torch.nn.functional.avg_pool2d(v.permute(0, 3, 1, 2).double(), 3, 1, 1) * 9
+    cabi.assert_close(out, box.permute(0, 2, 3, 1).numpy(), 1e-5, 1e-5, what="box sum")
+
+
+def test_dcnv4_infinite_and_nan_offsets_are_dropped_not_propagated():
+    B, H, W, G, D, K = 1, 6, 6, 1, 16, 9
+    v, om, go = make_dcnv4_inputs(B, H, W, G, D, seed=2)
+    om[..., 0] = float("inf")
+    om[..., 3] = float("nan")
+    om[..., 4] = -1e30
+    out = cabi.dcnv4_forward(v.cuda(), om.cuda(), (3, 3, 1, 1, 1, 1, 1, 1), G, D, 1.0)
+    gv, _ = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), (3, 3, 1, 1, 1, 1, 1, 1), G, D, 1.0)
+    assert torch.isfinite(out).all() and torch.isfinite(gv).all()
+
+
+# B, shapes, G, D, K, Q, (loc_lo, loc_hi)
+FDA_CASES = {
+    "detr_small_4lvl_k4": (2, [(16, 16), (8, 8), (4, 4), (2, 2)], 8, 32, 4, None, (0.0, 1.0)),
+    "k8_one_level": (1, [(20, 30)], 8, 32, 8, 77, (-0.1, 1.1)),
+    "five_levels": (1, [(8, 12), (6, 6), (4, 5), (2, 2), (1, 3)], 2, 16, 4, 50, (-0.3, 1.3)),
+    "k3_generic_points": (2, [(7, 5), (3, 4)], 3, 8, 3, 19, (0.0, 1.0)),
+    "d6_heads5": (1, [(6, 6), (3, 3)], 5, 6, 4, 11, (0.0, 1.0)),
+    "d64_two_levels": (1, [(9, 9), (5, 5)], 4, 64, 4, 33, (0.0, 1.0)),
+    "one_query": (1, [(4, 4)], 1, 32, 4, 1, (0.0, 1.0)),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("name", list(FDA_CASES))
+def test_flash_deform_attn_forward_and_backward_match_oracle(oracle, name, dtype):
+    B, shapes, G, D, K, Q, (lo, hi) = FDA_CASES[name]
+    print(f"case {name} dtype {dtype}", flush=True)
+    v, shp, st, sla, go = make_fda_inputs(B, shapes, G, D, K, Q, seed=zlib.crc32(name.encode()) % 1000, dtype=dtype, loc_lo=lo, loc_hi=hi)
+    want = oracle.flash_deform_attn_forward(cabi.f64(v), shp.numpy(), st.numpy(), cabi.f64(sla), K, coord_f32=True)
+    wgv, wgs = oracle.flash_deform_attn_backward(cabi.f64(v), shp.numpy(), st.numpy(), cabi.f64(sla), cabi.f64(go), K, coord_f32=True)
+    vd, sd, gd, shd, std = v.cuda(), sla.cuda(), go.cuda(), shp.cuda(), st.cuda()
+    out = cabi.fda_forward(vd, shd, std, sd, K)
+    gv, gs = cabi.fda_backward(vd, shd, std, sd, gd, K)
+    torch.cuda.synchronize()
+    cabi.assert_close(out, want, *FWD_TOL[dtype], what="output")
+    cabi.assert_close(gv, wgv, *GRAD_TOL[dtype], what="grad_value")
+    cabi.assert_close(gs, wgs, *GRAD_TOL[dtype], what="grad_sampling_loc_attn")
+
+
+def test_c_abi_rejects_bad_arguments():
+    from dcnv4_amd import _lib
+    v = torch.zeros(2, 4, 4, 16, device="cuda")
+    om = torch.zeros(2, 4, 4, 32, device="cuda")
+    geom = (3, 3, 1, 1, 1, 1, 1, 1)
+    with pytest.raises(ValueError, match="d_stride"):
+        cabi.dcnv4_forward(v, om, geom, 1, 16, 1.0, d_stride=3)
+    with pytest.raises(RuntimeError, match="im2col_step"):
+        cabi.dcnv4_forward(torch.zeros(3, 4, 4, 16, device="cuda"), torch.zeros(3, 4, 4, 32, device="cuda"), geom, 1, 16,
+                           1.0, im2col_step=2)
+    with pytest.raises(RuntimeError, match="smaller than"):
+        cabi.dcnv4_forward(v, om[..., :24].contiguous(), geom, 1, 16, 1.0)
+    with pytest.raises(ValueError, match="taps"):
+        cabi.dcnv4_forward(v, om, (9, 9, 1, 1, 4, 4, 1, 1), 1, 16, 1.0)
+    with pytest.raises(RuntimeError, match="aligned"):
+        cabi.dcnv4_forward(v.view(-1)[1:17].view(1, 1, 1, 16), torch.zeros(1, 1, 1, 32, device="cuda"), geom, 1, 16, 1.0)
+    L = _lib.load()
+    rc = L.dcnv4_gfx950_backward(v.data_ptr(), om.data_ptr(), v.data_ptr(), v.data_ptr(), om.data_ptr(), None, 0,
+                                 _lib.DTYPE_F16, 2, 4, 4, 1, 16, *geom, 1.0, 64, 0, 32, 0, 0, 0, None)
+    assert rc == _lib.ERR_RUNTIME and b"workspace" in L.dcnv4_gfx950_last_error()
+    shp = torch.tensor([[2, 2]] * 17, device="cuda")
+    with pytest.raises(ValueError, match="scales"):
+        cabi.fda_forward(torch.zeros(1, 68, 1, 16, device="cuda"), shp, torch.zeros(17, dtype=torch.int64, device="cuda"),
+                         torch.zeros(1, 1, 1, 17 * 3, device="cuda"), 1)

@@ -253,3 +253,24 @@ def test_fda_logit_gradients_sum_to_zero_and_vanish_for_out_of_range_locations(o
     sla[..., :16] = 7.0
     gv, gs = oracle.flash_deform_attn_backward(value.numpy(), shp.numpy(), start.numpy(), sla.numpy(), go.numpy(), K)
     assert np.all(gv == 0.0) and np.all(gs == 0.0)
+
+
+def test_fp32_coordinate_mode_tracks_the_float64_mode(oracle):
+    # same inputs, coordinates rounded to fp32 vs kept in double: only ulp-level coordinate noise may differ
+    B, H, W, G, D = 1, 20, 24, 2, 4
+    args = (3, 3, 1, 1, 1, 1, 1, 1, G, D, 1.3, 0)
+    value, om, go = make_dcnv4_inputs(B, H, W, G, D, seed=41)          # fp32-representable inputs
+    v, o, g = value.double().numpy(), om.double().numpy(), go.double().numpy()
+    a = oracle.dcnv4_forward(v, o, *args)
+    b = oracle.dcnv4_forward(v, o, *args, coord_f32=True)
+    assert np.abs(a - b).max() < 2e-4 and np.abs(a - b).max() > 0.0
+    ga, gb = oracle.dcnv4_backward(v, o, g, *args), oracle.dcnv4_backward(v, o, g, *args, coord_f32=True)
+    assert np.abs(ga[0] - gb[0]).max() < 2e-4 and np.abs(ga[1] - gb[1]).max() < 2e-3
+    value, shp, start, sla, go = make_fda_inputs(1, [(30, 40), (7, 9)], 2, 4, 4, Q=50, seed=42)
+    v, s, g = value.double().numpy(), sla.double().numpy(), go.double().numpy()
+    a = oracle.flash_deform_attn_forward(v, shp.numpy(), start.numpy(), s, 4)
+    b = oracle.flash_deform_attn_forward(v, shp.numpy(), start.numpy(), s, 4, coord_f32=True)
+    assert np.abs(a - b).max() < 2e-4
+    ga = oracle.flash_deform_attn_backward(v, shp.numpy(), start.numpy(), s, g, 4)
+    gb = oracle.flash_deform_attn_backward(v, shp.numpy(), start.numpy(), s, g, 4, coord_f32=True)
+    assert np.abs(ga[0] - gb[0]).max() < 2e-4 and np.abs(ga[1] - gb[1]).max() < 5e-3
