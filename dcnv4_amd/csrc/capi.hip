@@ -44,12 +44,16 @@ int ceil_log2(int v) {
 
 // Channels per lane: the widest power-of-two vector (<= 16 bytes) that divides D, unless a
 // valid d_stride hint asks for a narrower one.  Reference table: dcnv4_im2col_cuda.cuh:342-415.
-int choose_lanes(int D, int s, int d_stride, LaneMap *lm) {
+int choose_lanes(int D, int s, int d_stride, bool scatter, LaneMap *lm) {
   if (d_stride != 0 && d_stride != 1 && d_stride != 2 && d_stride != 4 && d_stride != 8 && d_stride != 16)
     return fail(DCNV4_ERR_INVALID_ARGUMENT, "invalid d_stride %d", d_stride);
   int cpt = 1;
   while (cpt * 2 * s <= 16 && D % (cpt * 2) == 0) cpt *= 2;
   if (d_stride > 0 && d_stride < cpt && D % d_stride == 0) cpt = d_stride;
+  // Kernels that scatter with fp32 atomics want one channel per lane: the lanes of a group then
+  // cover one contiguous run of dwords per atomic instruction, and the L2 atomic units retire
+  // about one dword per clock per channel however the dwords are spread over lanes.
+  else if (scatter && d_stride == 0 && D <= kWave) cpt = 1;
   lm->cpt = cpt;
   lm->tpg = D / cpt;
   lm->tpgp_log2 = ceil_log2(lm->tpg);
@@ -144,7 +148,7 @@ int dcn_prepare(DcnProblem *pr, bool backward, int dtype, int batch, int H, int 
 
   DcnLaunch &L = pr->launch;
   L = DcnLaunch{};
-  if (int rc = choose_lanes(D, s, d_stride, &L.lanes)) return rc;
+  if (int rc = choose_lanes(D, s, d_stride, backward, &L.lanes)) return rc;
   const int width = 1 << L.lanes.tpgp_log2;
   if (backward && width > kWave)
     return fail(DCNV4_ERR_INVALID_ARGUMENT, "backward needs group_channels/%d <= 64 lanes per group, got %d",
@@ -202,7 +206,7 @@ int fda_prepare(FdaProblem *pr, bool backward, int dtype, int batch, int N, int 
 
   FdaLaunch &F = pr->launch;
   F = FdaLaunch{};
-  if (int rc = choose_lanes(D, s, d_stride, &F.lanes)) return rc;
+  if (int rc = choose_lanes(D, s, d_stride, backward, &F.lanes)) return rc;
   const int width = 1 << F.lanes.tpgp_log2;
   if (backward && width > kWave)
     return fail(DCNV4_ERR_INVALID_ARGUMENT, "backward needs head_channels/%d <= 64 lanes per head, got %d",

@@ -22,8 +22,9 @@ def _vector_channels(group_channels, elem_bytes):
     return cpt
 
 
-def _spec(group, group_channels, elem_bytes):
-    d_stride = _vector_channels(group_channels, elem_bytes)
+def _spec(group, group_channels, elem_bytes, scatter=False):
+    # backward scatters with one channel per lane (contiguous dwords per atomic instruction)
+    d_stride = 1 if scatter and group_channels <= 64 else _vector_channels(group_channels, elem_bytes)
     lanes_per_group = 1
     while lanes_per_group < group_channels // d_stride:
         lanes_per_group *= 2
@@ -43,7 +44,7 @@ def find_spec_bwd(B, H, W, G, C, elem_bytes=2):
     key = f"{B}x{H}x{W}x{G}x{C}"
     if key in GFX950_BWD_TABLE:
         return GFX950_BWD_TABLE[key][0], GFX950_BWD_TABLE[key][1]
-    return _spec(G, C, elem_bytes)
+    return _spec(G, C, elem_bytes, scatter=True)
 
 
 def findspec_attn(B, Q, G, C, elem_bytes=2):
@@ -51,4 +52,4 @@ def findspec_attn(B, Q, G, C, elem_bytes=2):
 
 
 def findspec_attn_bwd(B, Q, G, C, elem_bytes=2):
-    return _spec(G, C, elem_bytes)
+    return _spec(G, C, elem_bytes, scatter=True)
