@@ -13,13 +13,13 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "libdcnv4_gfx950.so")
-SOURCES = ["capi.hip", "dcnv4_kernels.hip", "fda_kernels.hip"]
+SOURCES = ["capi.hip", "dcnv4_kernels.hip", "dcnv4_grad_value.hip", "fda_kernels.hip"]
 HEADERS = [os.path.join(CSRC, "common.hpp"), os.path.join(CSRC, "launch.hpp"),
            os.path.join(os.path.dirname(HERE), "include", "dcnv4_gfx950.h")]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 instructions.
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC", "-fno-gpu-rdc",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wall", "-Wno-pass-failed", "-Wno-unused-function", "-Wno-unknown-attributes"]
 

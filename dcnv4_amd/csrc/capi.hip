@@ -7,6 +7,7 @@
 #include <algorithm>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 
 #include "../../include/dcnv4_gfx950.h"
 #include "common.hpp"
@@ -112,7 +113,70 @@ hipError_t narrow_async(int dtype, const float *src, void *dst, size_t n, hipStr
 
 size_t round16(size_t v) { return (v + 15) & ~size_t(15); }
 
+__global__ void init_state_kernel(GradState *st) {
+  if (threadIdx.x == 0) *st = GradState{0u, 0u, 0u, 0u};
+}
+
+constexpr size_t kStateBytes = 256;     // GradState, padded
+constexpr int kTiledMaxGroupChannels = 64;
+
+bool tiled_grad_value(int D) { return D <= kTiledMaxGroupChannels; }
+
+// Tuning override for the reach of the tiled grad_value kernel (pixels); results never depend on it.
+int reach_setting() {
+  static const int v = [] {
+    const char *e = getenv("DCNV4_GFX950_REACH");
+    const int r = e ? atoi(e) : 5;
+    return r < 0 ? 0 : (r > 64 ? 64 : r);
+  }();
+  return v;
+}
+
+// Tile, channel chunk and strip of the tiled grad_value kernel such that its LDS footprint fits.
+int plan_grad_value_tiles(DcnLaunch *L) {
+  const int D = L->D;
+  L->reach = reach_setting();
+  L->ng_chunk = std::max(1, std::min(L->G, kTiledMaxGroupChannels / std::max(D, 16)));
+  // power-of-two tiles (the reach rule uses shifts); shrink until the LDS footprint fits
+  L->tile_h_log2 = 4;
+  L->tile_w_log2 = 4;
+  while (L->tile_h_log2 > 0 && (1 << (L->tile_h_log2 - 1)) >= L->H) --L->tile_h_log2;
+  while (L->tile_w_log2 > 0 && (1 << (L->tile_w_log2 - 1)) >= L->W) --L->tile_w_log2;
+  auto visited = [&](int tile, int stride) { return (tile + 2 * L->reach + stride - 1) / stride + 1; };
+  for (;;) {
+    L->tile_h = 1 << L->tile_h_log2;
+    L->tile_w = 1 << L->tile_w_log2;
+    const int row = visited(L->tile_w, L->sw);
+    bool fits = false;
+    for (int rows = 4; rows >= 1 && !fits; --rows) {       // stage up to 4 visited rows per strip
+      L->strip_pix = rows * row;
+      fits = dcnv4_grad_value_lds_bytes(*L) <= kMaxLdsPerWorkgroup - 2048;
+    }
+    if (fits) break;
+    if (L->tile_h_log2 > 0 && L->tile_h_log2 >= L->tile_w_log2) --L->tile_h_log2;
+    else if (L->tile_w_log2 > 0) --L->tile_w_log2;
+    else return fail(DCNV4_ERR_RUNTIME, "kernel with %d taps and %d group channels does not fit the tiled backward", L->Kp, D);
+  }
+  const long long contributions = (long long)visited(L->tile_h, L->sh) * visited(L->tile_w, L->sw) * L->Kp;
+  L->fix_bits = 62 - ceil_log2((int)std::min<long long>(contributions, 1 << 30));
+  return DCNV4_OK;
+}
+
 // ---------------------------------------------------------------- DCNv4
+// Output pixels per workgroup: about block_thread (default 256) lanes of whole pixels, capped by
+// the LDS that the staged offset_mask rows (and, backward, their gradients) take.
+int choose_block_pixels(DcnLaunch *L, int block_thread, bool backward) {
+  const int lanes_per_pix = L->G << L->lanes.tpgp_log2;
+  const int want = block_thread > 0 ? block_thread : kBlockThreads;
+  int npix = std::max(1, want / lanes_per_pix);
+  const size_t lds_per_pix = (size_t)L->P_pad * sizeof(float) * (backward ? 2 : 1);
+  while (npix > 1 && npix * lds_per_pix > kMaxDynamicLds) --npix;
+  if (npix * lds_per_pix > kMaxDynamicLds)
+    return fail(DCNV4_ERR_RUNTIME, "offset_mask row of %d elements does not fit in LDS", L->P_pad);
+  L->npix_block = npix;
+  return DCNV4_OK;
+}
+
 struct DcnProblem {
   DcnLaunch launch;      // geometry common to every chunk
   int batch, Ho, Wo, s;
@@ -158,14 +222,7 @@ int dcn_prepare(DcnProblem *pr, bool backward, int dtype, int batch, int H, int 
   L.Kp = Kp; L.P_pad = P_pad; L.remove_center = remove_center; L.softmax = softmax ? 1 : 0;
   L.offset_scale = offset_scale;
 
-  const int lanes_per_pix = G * width;
-  const int want = block_thread > 0 ? block_thread : kBlockThreads;
-  int npix = std::max(1, want / lanes_per_pix);
-  const size_t lds_per_pix = (size_t)P_pad * sizeof(float) * (backward ? 2 : 1);
-  while (npix > 1 && npix * lds_per_pix > kMaxDynamicLds) --npix;
-  if (npix * lds_per_pix > kMaxDynamicLds)
-    return fail(DCNV4_ERR_RUNTIME, "offset_mask row of %d elements does not fit in LDS", P_pad);
-  L.npix_block = npix;
+  if (int rc = choose_block_pixels(&L, block_thread, backward)) return rc;
 
   pr->batch = batch; pr->Ho = Ho; pr->Wo = Wo; pr->s = s;
   pr->img_elems = (size_t)H * W * G * D;
@@ -291,8 +348,10 @@ int dcnv4_gfx950_forward(const void *value, const void *offset_mask, void *outpu
 
 size_t dcnv4_gfx950_backward_workspace_bytes(int dtype, int batch, int height_in, int width_in, int group,
                                              int group_channels) {
-  if (elem_bytes(dtype) != 2 || batch <= 0 || height_in <= 0 || width_in <= 0 || group <= 0 || group_channels <= 0)
+  if (elem_bytes(dtype) == 0 || batch <= 0 || height_in <= 0 || width_in <= 0 || group <= 0 || group_channels <= 0)
     return 0;
+  if (tiled_grad_value(group_channels)) return kStateBytes;
+  if (elem_bytes(dtype) != 2) return 0;
   return round16((size_t)batch * height_in * width_in * group * group_channels * sizeof(float));
 }
 
@@ -315,6 +374,45 @@ int dcnv4_gfx950_backward(const void *value, const void *offset_mask, const void
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   const size_t total = (size_t)batch * pr.img_elems;
+
+  if (tiled_grad_value(group_channels)) {
+    // 1. grad_offset_mask + statistics  2. tiled grad_value (plain stores)  3. fallback scatter
+    //    for corners beyond the reach / non-finite statistics (returns at once otherwise)
+    DcnLaunch base = pr.launch;
+    if (int rc = plan_grad_value_tiles(&base)) return rc;
+    base.state = static_cast<GradState *>(workspace);
+    hipLaunchKernelGGL(init_state_kernel, dim3(1), dim3(64), 0, st, base.state);
+    if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);
+    const int per = images_per_launch(pr, false);
+    for (int pass = 0; pass < 3; ++pass) {
+      for (int b0 = 0; b0 < batch; b0 += per) {
+        const int nb = std::min(per, batch - b0);
+        DcnLaunch L = base;
+        L.value = at(value, b0 * pr.img_elems, pr.s);
+        L.offset_mask = at(offset_mask, b0 * pr.img_om_elems, pr.s);
+        L.grad_out = at(grad_output, b0 * pr.img_out_elems, pr.s);
+        L.grad_value = at(grad_value, b0 * pr.img_elems, pr.s);
+        L.grad_offset_mask = at(grad_offset_mask, b0 * pr.img_om_elems, pr.s);
+        L.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
+        L.n_pix = nb * L.Q;
+        L.n_img = nb;
+        hipError_t e = hipSuccess;
+        if (pass == 0) {
+          // gathers want 16-byte lanes; the lane map chosen for scatter is only used by pass 2
+          if (int rc = choose_lanes(group_channels, pr.s, 0, false, &L.lanes)) return rc;
+          if (int rc = choose_block_pixels(&L, 0, true)) return rc;
+          e = launch_dcnv4_backward(dtype, L, kBwdOffsetMask, st);
+        } else if (pass == 1) {
+          e = launch_dcnv4_grad_value(dtype, L, st);
+        } else {
+          e = launch_dcnv4_backward(dtype, L, kBwdFallback, st);
+        }
+        if (e) return hip_fail("dcnv4 backward launch", e);
+      }
+    }
+    return DCNV4_OK;
+  }
+
   float *acc = need > 0 ? static_cast<float *>(workspace) : static_cast<float *>(grad_value);
   if (hipError_t e = clear_async(acc, total, st)) return hip_fail("clear launch", e);
   const int per = images_per_launch(pr, true);
@@ -328,7 +426,7 @@ int dcnv4_gfx950_backward(const void *value, const void *offset_mask, const void
     L.grad_offset_mask = at(grad_offset_mask, b0 * pr.img_om_elems, pr.s);
     L.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
     L.n_pix = nb * L.Q;
-    if (hipError_t e = launch_dcnv4_backward(dtype, L, st)) return hip_fail("dcnv4 backward launch", e);
+    if (hipError_t e = launch_dcnv4_backward(dtype, L, kBwdFull, st)) return hip_fail("dcnv4 backward launch", e);
   }
   if (need > 0)
     if (hipError_t e = narrow_async(dtype, acc, grad_value, total, st)) return hip_fail("cast launch", e);

@@ -129,6 +129,8 @@ struct Tap {
   uint32_t off[4];
   float w[4];
   float ly, lx;     // fractional parts; d w / d y = (-hx,-lx,hx,lx), d w / d x = (-hy,hy,-ly,ly)
+  int y0, x0;       // integer position of corner 0 (-1 .. H-1 / W-1 when the tap is inside)
+  uint32_t valid;   // bit c set when corner c lies inside the image
 };
 
 // base = byte offset of (image, row 0, col 0, this lane's channels); pix_bytes = bytes per pixel.
@@ -150,7 +152,54 @@ __device__ __forceinline__ Tap make_tap(float y, float x, int H, int W, uint32_t
   t.off[1] = (top && rig) ? o00 + pix_bytes : kDropOffset;
   t.off[2] = (bot && lef) ? o00 + row : kDropOffset;
   t.off[3] = (bot && rig) ? o00 + row + pix_bytes : kDropOffset;
+  t.y0 = y0; t.x0 = x0;
+  t.valid = (uint32_t)(top && lef) | ((uint32_t)(top && rig) << 1) | ((uint32_t)(bot && lef) << 2) |
+            ((uint32_t)(bot && rig) << 3);
   return t;
+}
+
+// ---------------------------------------------------------------- tiled grad_value: reach rule
+// grad_value is accumulated by workgroups that each own a 2^th x 2^tw tile of the input and
+// visit every output pixel whose reference point p0 (the centre tap at zero offset) lies within
+// `reach` pixels of the tile.  A corner is "near" when the tile that owns it visits the output
+// pixel it comes from; all other in-image corners are left to the fallback scatter.  For one
+// output pixel the near corners form a box: the union of the tiles that visit it.  Both the
+// statistics pass and the fallback pass must use exactly this box.
+struct NearBox { int y_lo, y_hi, x_lo, x_hi; };     // half-open, in input pixels
+
+__device__ __forceinline__ NearBox near_box(int p0y, int p0x, int tile_h_log2, int tile_w_log2, int reach) {
+  // tiles t with t*T - reach <= p0 < (t+1)*T + reach  <=>  floor((p0-reach-T)/T)+1 <= t <= floor((p0+reach)/T)
+  NearBox b;
+  b.y_lo = (((p0y - reach) >> tile_h_log2)) << tile_h_log2;            // arithmetic shifts = floor division
+  b.y_hi = (((p0y + reach) >> tile_h_log2) + 1) << tile_h_log2;
+  b.x_lo = (((p0x - reach) >> tile_w_log2)) << tile_w_log2;
+  b.x_hi = (((p0x + reach) >> tile_w_log2) + 1) << tile_w_log2;
+  return b;
+}
+
+__device__ __forceinline__ bool corner_is_near(const NearBox &b, int cy, int cx) {
+  return cy >= b.y_lo && cy < b.y_hi && cx >= b.x_lo && cx < b.x_hi;
+}
+
+__device__ __forceinline__ int ceil_div_signed(int a, int b) {    // b > 0
+  return a >= 0 ? (a + b - 1) / b : -((-a) / b);
+}
+
+// ---------------------------------------------------------------- small shared helpers
+// Running max and reciprocal sum for a softmax over n logits held in LDS.
+__device__ __forceinline__ void softmax_stats(const float *m, int n, float &mx, float &inv) {
+  mx = m[0];
+  for (int k = 1; k < n; ++k) mx = fmaxf(mx, m[k]);
+  float s = 0.f;
+  for (int k = 0; k < n; ++k) s += __expf(m[k] - mx);
+  inv = 1.f / s;
+}
+
+// Kernel-tap decode for a 3x3 kernel with (kp == 8) or without (kp == 9) the centre removed:
+// x index i outer, y index j inner (dcnv4_im2col_cuda.cuh:216-236).
+__device__ __forceinline__ void tap_ij_3x3(int kp, int k, int &i, int &j) {
+  const int kk = (kp == 8 && k >= 4) ? k + 1 : k;
+  i = kk / 3; j = kk - 3 * i;
 }
 
 // ---------------------------------------------------------------- cross-lane sums
@@ -219,7 +268,7 @@ __device__ __forceinline__ void unstage_rows_from_lds(void *dst, const float *sr
         const f32x4 v = *reinterpret_cast<const f32x4 *>(src + i * EPV + j);
         f[j] = v.x; f[j + 1] = v.y; f[j + 2] = v.z; f[j + 3] = v.w;
       }
-      __builtin_nontemporal_store(Pack<Tag, EPV>::encode(f), d + i);
+      d[i] = Pack<Tag, EPV>::encode(f);
     }
   } else {
     typedef typename RawWord<Tag::kBytes>::type elem_t;

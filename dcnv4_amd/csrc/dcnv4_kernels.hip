@@ -36,22 +36,6 @@ __device__ __forceinline__ PixelGeom pixel_geometry(const DcnLaunch &p, int pix,
   return geo;
 }
 
-// softmax statistics over the Kp modulation scalars of one (pixel, group); only used when the
-// (reference-latent, dcnv4_im2col_cuda.cuh:173-193) softmax flag is set.
-__device__ __forceinline__ void softmax_stats(const float *m, int n, float &mx, float &inv) {
-  mx = m[0];
-  for (int k = 1; k < n; ++k) mx = fmaxf(mx, m[k]);
-  float s = 0.f;
-  for (int k = 0; k < n; ++k) s += __expf(m[k] - mx);
-  inv = 1.f / s;
-}
-
-// Kernel-tap decode for the two unrolled 3x3 instantiations (x index outer, y index inner).
-template <int KP> __device__ __forceinline__ void tap_ij(int k, int &i, int &j) {
-  const int kk = (KP == 8 && k >= 4) ? k + 1 : k;
-  i = kk / 3; j = kk - 3 * i;
-}
-
 // ------------------------------------------------------------------------------- forward
 template <typename Tag, int CPT, int KP>
 __global__ void __launch_bounds__(kBlockThreads) dcnv4_forward_kernel(const DcnLaunch p) {
@@ -108,7 +92,7 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_forward_kernel(const DcnL
 #pragma unroll
       for (int k = 0; k < KP; ++k) {
         int i, j;
-        tap_ij<KP>(k, i, j);
+        tap_ij_3x3(KP, k, i, j);
         one_tap(k, i, j);
       }
     } else {
@@ -127,10 +111,48 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_forward_kernel(const DcnL
 }
 
 // ------------------------------------------------------------------------------- backward
-template <typename Tag, int CPT, int KP>
+// Adds v to element `elem` of a tensor of dtype Tag with one hardware atomic (packed pair for the
+// 16-bit types, the untouched half gets +0).
+template <typename Tag>
+__device__ __forceinline__ void atomic_add_element(void *base, size_t elem, float v) {
+  if constexpr (Tag::kBytes == 4) {
+    unsafeAtomicAdd(reinterpret_cast<float *>(base) + elem, v);
+  } else {
+    char *addr = reinterpret_cast<char *>(base) + (elem & ~size_t(1)) * 2;
+    const bool hi = elem & 1;
+    const f32x2 pair = {hi ? 0.f : v, hi ? v : 0.f};
+    if constexpr (Tag::kCode == F16::kCode)
+      __builtin_amdgcn_global_atomic_fadd_v2f16((__attribute__((address_space(1))) f16x2 *)addr,
+                                                __builtin_convertvector(pair, f16x2));
+    else
+      __builtin_amdgcn_global_atomic_fadd_v2bf16((__attribute__((address_space(1))) bf16x2 *)addr,
+                                                 __builtin_convertvector(pair, bf16x2));
+  }
+}
+
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  for (int o = 32; o > 0; o >>= 1) v = max(v, (uint32_t)__shfl_xor((int)v, o, kWave));
+  return v;
+}
+
+// One kernel body, three roles (BackwardMode):
+//   kBwdFull        grad_offset_mask, and grad_value scattered with fp32 buffer atomics into a
+//                   cleared fp32 image (any group width; the generic path)
+//   kBwdOffsetMask  grad_offset_mask only, plus the statistics the tiled grad_value kernel needs
+//                   (max |grad_out|, max |modulation|, "some corner is beyond the reach" flag)
+//   kBwdFallback    no gradients of offsets; scatters into grad_value, in its own dtype, the
+//                   corners the tiled kernel does not cover: the far ones, or all of them when the
+//                   statistics are not finite.  Exits at once when there is nothing to do.
+template <typename Tag, int CPT, int KP, int MODE>
 __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const DcnLaunch p) {
   extern __shared__ float lds[];
   typedef Pack<Tag, CPT> pack;
+  bool scatter_all = false;
+  if constexpr (MODE == kBwdFallback) {
+    const uint32_t gmax = p.state->go_max_bits, mmax = p.state->mask_max_bits;
+    scatter_all = gmax >= 0x7f800000u || mmax >= 0x7f800000u;
+    if (!scatter_all && p.state->far_flag == 0) return;
+  }
   const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
   const int pix0 = (int)blk * p.npix_block;
   const int npix = min(p.npix_block, p.n_pix - pix0);
@@ -138,7 +160,8 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
   float *s_om = lds, *s_grad = lds + p.npix_block * p.P_pad;
   stage_rows_to_lds<Tag>(s_om, (const char *)p.offset_mask + (size_t)pix0 * p.P_pad * Tag::kBytes,
                          npix * p.P_pad, vec16);
-  for (int i = threadIdx.x; i < npix * p.P_pad; i += blockDim.x) s_grad[i] = 0.f;
+  if constexpr (MODE != kBwdFallback)
+    for (int i = threadIdx.x; i < npix * p.P_pad; i += blockDim.x) s_grad[i] = 0.f;
   __syncthreads();
 
   const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
@@ -148,26 +171,41 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
   const int items = (npix * p.G) << tpgp_log2;
   const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
   const int Kp = p.Kp;
+  const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
+  uint32_t go_max = 0, mask_max = 0, far = 0;
 
   for (int it = threadIdx.x; it < items; it += blockDim.x) {
     const int chunk = it & (width - 1);
     const bool active = chunk < p.lanes.tpg;       // false only on padding lanes of a non-2^n cluster
     const int pg = it >> tpgp_log2;
     const int lp = pg / p.G, g = pg - lp * p.G;
-    const PixelGeom geo = pixel_geometry<Tag>(p, pix0 + lp, g, active ? chunk : 0);
+    const int pix = pix0 + lp;
+    const PixelGeom geo = pixel_geometry<Tag>(p, pix, g, active ? chunk : 0);
     const float *om = s_om + lp * p.P_pad + g * 3 * Kp;
     float *gom = s_grad + lp * p.P_pad + g * 3 * Kp;
     float mx = 0.f, inv = 1.f;
     if (p.softmax) softmax_stats(om + 2 * Kp, Kp, mx, inv);
+    // reference point of this output pixel (centre tap, zero offset), for the reach rule
+    NearBox box = {0, 0, 0, 0};
+    if constexpr (MODE != kBwdFull) {
+      const int q = pix % p.Q;
+      box = near_box(half_h - p.ph + (q / p.Wo) * p.sh, half_w - p.pw + (q % p.Wo) * p.sw, p.tile_h_log2,
+                     p.tile_w_log2, p.reach);
+    }
+    const size_t img_elem0 = (size_t)(pix / p.Q) * (size_t)(p.H * p.W) * (size_t)(p.G * p.D);
 
     float go[CPT];
     {
       const char *src = (const char *)p.grad_out +
-                        ((size_t)(pix0 + lp) * (p.G * p.D) + g * p.D + (active ? chunk : 0) * CPT) * Tag::kBytes;
+                        ((size_t)pix * (p.G * p.D) + g * p.D + (active ? chunk : 0) * CPT) * Tag::kBytes;
       pack::decode(*reinterpret_cast<const typename pack::raw_t *>(src), go);
       if (!active) {
 #pragma unroll
         for (int c = 0; c < CPT; ++c) go[c] = 0.f;
+      }
+      if constexpr (MODE == kBwdOffsetMask) {
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) go_max = max(go_max, __builtin_bit_cast(uint32_t, fabsf(go[c])));
       }
     }
     float dot_pg = 0.f;     // sum_k p_k * gz_k, softmax Jacobian only
@@ -179,8 +217,28 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
       if (p.softmax) m = __expf(m - mx) * inv;
       Tap t = make_tap(y, x, p.H, p.W, geo.img_base, pix_bytes);
       if (!active) {
+        t.valid = 0;
 #pragma unroll
         for (int cn = 0; cn < 4; ++cn) t.off[cn] = kDropOffset;
+      }
+      if constexpr (MODE == kBwdFallback) {
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn) {
+          if (!(t.valid & (1u << cn))) continue;
+          const int cy = t.y0 + (cn >> 1), cx = t.x0 + (cn & 1);
+          if (!scatter_all && corner_is_near(box, cy, cx)) continue;
+          const float w = m * t.w[cn];
+          const size_t e0 = img_elem0 + (size_t)(cy * p.W + cx) * (p.G * p.D) + g * p.D + chunk * CPT;
+#pragma unroll
+          for (int c = 0; c < CPT; ++c) atomic_add_element<Tag>(p.grad_value, e0 + c, go[c] * w);
+        }
+        return;
+      }
+      if constexpr (MODE == kBwdOffsetMask) {
+        mask_max = max(mask_max, __builtin_bit_cast(uint32_t, fabsf(m)));
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn)
+          if ((t.valid & (1u << cn)) && !corner_is_near(box, t.y0 + (cn >> 1), t.x0 + (cn & 1))) far = 1;
       }
       typename pack::raw_t raw[4];
 #pragma unroll
@@ -194,12 +252,14 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
 #pragma unroll
         for (int c = 0; c < CPT; ++c) d = fmaf(v[c], go[c], d);
         dots[cn] = d;
-        // scatter: grad_value[corner] += grad_out * m * w   (common.h:153,164,174,184)
-        const float w = m * t.w[cn];
-        const uint32_t aoff = (t.off[cn] == kDropOffset) ? kDropOffset : t.off[cn] * (4 / Tag::kBytes);
+        if constexpr (MODE == kBwdFull) {
+          // scatter: grad_value[corner] += grad_out * m * w   (common.h:153,164,174,184)
+          const float w = m * t.w[cn];
+          const uint32_t aoff = (t.off[cn] == kDropOffset) ? kDropOffset : t.off[cn] * (4 / Tag::kBytes);
 #pragma unroll
-        for (int c = 0; c < CPT; ++c)
-          __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(go[c] * w, gacc, aoff + 4 * c, 0, 0);
+          for (int c = 0; c < CPT; ++c)
+            __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(go[c] * w, gacc, aoff + 4 * c, 0, 0);
+        }
       }
       const float hy = 1.f - t.ly, hx = 1.f - t.lx;
       float gx = hy * (dots[1] - dots[0]) + t.ly * (dots[3] - dots[2]);   // common.h:188-201
@@ -220,7 +280,7 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
 #pragma unroll
       for (int k = 0; k < KP; ++k) {
         int i, j;
-        tap_ij<KP>(k, i, j);
+        tap_ij_3x3(KP, k, i, j);
         one_tap(k, i, j);
       }
     } else {
@@ -232,11 +292,35 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
           ++k;
         }
     }
-    if (p.softmax && chunk == 0) {      // p_k (g_k - sum_j p_j g_j), dcnv4_col2im_cuda.cuh:352-365
-      for (int k = 0; k < Kp; ++k) {
-        const float pk = __expf(om[2 * Kp + k] - mx) * inv;
-        gom[2 * Kp + k] = pk * (gom[2 * Kp + k] - dot_pg);
+    if constexpr (MODE != kBwdFallback) {
+      if (p.softmax && chunk == 0) {      // p_k (g_k - sum_j p_j g_j), dcnv4_col2im_cuda.cuh:352-365
+        for (int k = 0; k < Kp; ++k) {
+          const float pk = __expf(om[2 * Kp + k] - mx) * inv;
+          gom[2 * Kp + k] = pk * (gom[2 * Kp + k] - dot_pg);
+        }
       }
+    }
+  }
+  if constexpr (MODE == kBwdFallback) return;
+  if constexpr (MODE == kBwdOffsetMask) {
+    // Same-address atomics retire slowly at the memory side: fold the workgroup's statistics in
+    // LDS first and only touch the global word when it would actually grow.
+    __shared__ uint32_t s_stat[3];
+    if (threadIdx.x < 3) s_stat[threadIdx.x] = 0u;
+    __syncthreads();
+    go_max = wave_max_u32(go_max);
+    mask_max = wave_max_u32(mask_max);
+    far = wave_max_u32(far);
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+      atomicMax(&s_stat[0], go_max);
+      atomicMax(&s_stat[1], mask_max);
+      atomicMax(&s_stat[2], far);
+    }
+    __syncthreads();
+    if (threadIdx.x < 3) {
+      uint32_t *dst = &p.state->go_max_bits + threadIdx.x;
+      const uint32_t mine = s_stat[threadIdx.x];
+      if (mine > __hip_atomic_load(dst, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(dst, mine);
     }
   }
   __syncthreads();
@@ -253,25 +337,26 @@ hipError_t launch_fwd_k(const DcnLaunch &p, hipStream_t stream, dim3 grid, dim3 
   return hipGetLastError();
 }
 
-template <typename Tag, int CPT>
+template <typename Tag, int CPT, int MODE>
 hipError_t launch_bwd_k(const DcnLaunch &p, hipStream_t stream, dim3 grid, dim3 block, size_t lds) {
   const bool k3 = p.kh == 3 && p.kw == 3;
-  if (k3 && !p.remove_center) hipLaunchKernelGGL((dcnv4_backward_kernel<Tag, CPT, 9>), grid, block, lds, stream, p);
-  else if (k3 && p.remove_center) hipLaunchKernelGGL((dcnv4_backward_kernel<Tag, CPT, 8>), grid, block, lds, stream, p);
-  else hipLaunchKernelGGL((dcnv4_backward_kernel<Tag, CPT, 0>), grid, block, lds, stream, p);
+  if (k3 && !p.remove_center) hipLaunchKernelGGL((dcnv4_backward_kernel<Tag, CPT, 9, MODE>), grid, block, lds, stream, p);
+  else if (k3 && p.remove_center) hipLaunchKernelGGL((dcnv4_backward_kernel<Tag, CPT, 8, MODE>), grid, block, lds, stream, p);
+  else hipLaunchKernelGGL((dcnv4_backward_kernel<Tag, CPT, 0, MODE>), grid, block, lds, stream, p);
   return hipGetLastError();
 }
 
-template <typename Tag, bool BWD>
+// MODE < 0 selects the forward kernel.
+template <typename Tag, int MODE>
 hipError_t launch_by_cpt(const DcnLaunch &p, hipStream_t stream) {
   const dim3 grid((p.n_pix + p.npix_block - 1) / p.npix_block), block(kBlockThreads);
-  const size_t lds = BWD ? dcnv4_backward_lds_bytes(p) : dcnv4_forward_lds_bytes(p);
-#define DCN_CASE(N)                                                         \
-  case N:                                                                   \
-    if constexpr (N * Tag::kBytes <= 16) {                                  \
-      return BWD ? launch_bwd_k<Tag, N>(p, stream, grid, block, lds)        \
-                 : launch_fwd_k<Tag, N>(p, stream, grid, block, lds);       \
-    }                                                                       \
+  const size_t lds = MODE >= 0 ? dcnv4_backward_lds_bytes(p) : dcnv4_forward_lds_bytes(p);
+#define DCN_CASE(N)                                                              \
+  case N:                                                                        \
+    if constexpr (N * Tag::kBytes <= 16) {                                       \
+      if constexpr (MODE >= 0) return launch_bwd_k<Tag, N, MODE>(p, stream, grid, block, lds); \
+      else return launch_fwd_k<Tag, N>(p, stream, grid, block, lds);             \
+    }                                                                            \
     break;
   switch (p.lanes.cpt) {
     DCN_CASE(1) DCN_CASE(2) DCN_CASE(4) DCN_CASE(8)
@@ -280,11 +365,11 @@ hipError_t launch_by_cpt(const DcnLaunch &p, hipStream_t stream) {
   return hipErrorInvalidValue;
 }
 
-template <bool BWD> hipError_t launch_by_dtype(int dtype, const DcnLaunch &p, hipStream_t stream) {
+template <int MODE> hipError_t launch_by_dtype(int dtype, const DcnLaunch &p, hipStream_t stream) {
   switch (dtype) {
-    case F32::kCode: return launch_by_cpt<F32, BWD>(p, stream);
-    case F16::kCode: return launch_by_cpt<F16, BWD>(p, stream);
-    case BF16::kCode: return launch_by_cpt<BF16, BWD>(p, stream);
+    case F32::kCode: return launch_by_cpt<F32, MODE>(p, stream);
+    case F16::kCode: return launch_by_cpt<F16, MODE>(p, stream);
+    case BF16::kCode: return launch_by_cpt<BF16, MODE>(p, stream);
   }
   return hipErrorInvalidValue;
 }
@@ -295,10 +380,15 @@ size_t dcnv4_forward_lds_bytes(const DcnLaunch &p) { return (size_t)p.npix_block
 size_t dcnv4_backward_lds_bytes(const DcnLaunch &p) { return 2 * dcnv4_forward_lds_bytes(p); }
 
 hipError_t launch_dcnv4_forward(int dtype, const DcnLaunch &p, hipStream_t stream) {
-  return launch_by_dtype<false>(dtype, p, stream);
+  return launch_by_dtype<-1>(dtype, p, stream);
 }
-hipError_t launch_dcnv4_backward(int dtype, const DcnLaunch &p, hipStream_t stream) {
-  return launch_by_dtype<true>(dtype, p, stream);
+hipError_t launch_dcnv4_backward(int dtype, const DcnLaunch &p, int mode, hipStream_t stream) {
+  switch (mode) {
+    case kBwdFull: return launch_by_dtype<kBwdFull>(dtype, p, stream);
+    case kBwdOffsetMask: return launch_by_dtype<kBwdOffsetMask>(dtype, p, stream);
+    case kBwdFallback: return launch_by_dtype<kBwdFallback>(dtype, p, stream);
+  }
+  return hipErrorInvalidValue;
 }
 
 }  // namespace dcn

@@ -27,14 +27,6 @@ __device__ __forceinline__ Level load_level(const FdaLaunch &p, int l) {
   return lv;
 }
 
-__device__ __forceinline__ void softmax_stats(const float *m, int n, float &mx, float &inv) {
-  mx = m[0];
-  for (int k = 1; k < n; ++k) mx = fmaxf(mx, m[k]);
-  float s = 0.f;
-  for (int k = 0; k < n; ++k) s += __expf(m[k] - mx);
-  inv = 1.f / s;
-}
-
 // ------------------------------------------------------------------------------- forward
 template <typename Tag, int CPT, int KT>
 __global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLaunch p) {

@@ -12,7 +12,22 @@ constexpr uint64_t kMaxSpanBytes = 0x7fff0000ull;
 constexpr int kMaxTaps = 64;       // DCNv4: kh*kw - remove_center; attention: L*K
 constexpr int kMaxLevels = 16;
 constexpr int kBlockThreads = 256;
-constexpr size_t kMaxDynamicLds = 64 * 1024;
+constexpr size_t kMaxDynamicLds = 64 * 1024;      // without raising the per-kernel limit
+constexpr size_t kMaxLdsPerWorkgroup = 160 * 1024;  // gfx950
+
+// Device-side scratch word block shared by the kernels of one backward call (16 bytes).
+struct GradState {
+  uint32_t go_max_bits;    // max |grad_out| as IEEE bits (ordered like unsigned ints for x >= 0; NaN sorts last)
+  uint32_t mask_max_bits;  // max |modulation| (after softmax when enabled)
+  uint32_t far_flag;       // some in-image corner lies outside the reach the tiled scatter covers
+  uint32_t reserved;
+};
+
+enum BackwardMode {
+  kBwdFull = 0,        // grad_offset_mask + fp32 atomic scatter of grad_value (generic path)
+  kBwdOffsetMask = 1,  // grad_offset_mask + GradState statistics, no scatter
+  kBwdFallback = 2,    // scatter of the corners the tiled kernel skipped, atomics in the tensor dtype
+};
 
 struct LaneMap {
   int cpt;          // channels per lane (power of two, cpt * elem_bytes <= 16)
@@ -36,6 +51,16 @@ struct DcnLaunch {
   float offset_scale;
   int npix_block;           // output pixels per workgroup
   LaneMap lanes;
+  // tiled grad_value path
+  void *grad_value;         // [n_img, H, W, G*D] in the tensor dtype
+  GradState *state;
+  int n_img;
+  int tile_h, tile_w;       // input-space tile one workgroup owns (powers of two)
+  int tile_h_log2, tile_w_log2;
+  int reach;                // corners up to `reach` pixels outside the tile of their output pixel are covered
+  int ng_chunk;             // groups per workgroup (channel chunk = ng_chunk * D)
+  int strip_pix;            // output pixels staged per strip
+  int fix_bits;             // fractional bits of the 64-bit fixed-point accumulators
 };
 
 // Flash deformable attention (reference: DCNv4_op/src/cuda/flash_deform_im2col_cuda.cuh:211-272)
@@ -57,7 +82,9 @@ struct FdaLaunch {
 
 // Each returns hipSuccess or the launch error.  dtype: 0 fp32, 1 fp16, 2 bf16.
 hipError_t launch_dcnv4_forward(int dtype, const DcnLaunch &p, hipStream_t stream);
-hipError_t launch_dcnv4_backward(int dtype, const DcnLaunch &p, hipStream_t stream);
+hipError_t launch_dcnv4_backward(int dtype, const DcnLaunch &p, int mode, hipStream_t stream);
+hipError_t launch_dcnv4_grad_value(int dtype, const DcnLaunch &p, hipStream_t stream);
+size_t dcnv4_grad_value_lds_bytes(const DcnLaunch &p);
 hipError_t launch_fda_forward(int dtype, const FdaLaunch &p, hipStream_t stream);
 hipError_t launch_fda_backward(int dtype, const FdaLaunch &p, hipStream_t stream);
 
