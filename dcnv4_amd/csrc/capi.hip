@@ -136,7 +136,7 @@ int reach_setting() {
 int plan_grad_value_tiles(DcnLaunch *L) {
   const int D = L->D;
   L->reach = reach_setting();
-  L->ng_chunk = std::max(1, std::min(L->G, kTiledMaxGroupChannels / std::max(D, 16)));
+  L->ng_chunk = std::max(1, std::min(L->G, kTiledMaxGroupChannels / std::max(D, 16)));   // <= 4
   // power-of-two tiles (the reach rule uses shifts); shrink until the LDS footprint fits
   L->tile_h_log2 = 4;
   L->tile_w_log2 = 4;
@@ -148,9 +148,9 @@ int plan_grad_value_tiles(DcnLaunch *L) {
     L->tile_w = 1 << L->tile_w_log2;
     const int row = visited(L->tile_w, L->sw);
     bool fits = false;
-    for (int rows = 4; rows >= 1 && !fits; --rows) {       // stage up to 4 visited rows per strip
-      L->strip_pix = rows * row;
-      fits = dcnv4_grad_value_lds_bytes(*L) <= kMaxLdsPerWorkgroup - 2048;
+    for (int rows = 4; rows >= 1 && !fits; --rows) {       // up to 4 visited rows per strip
+      L->strip_pix = std::min(rows * row, 1023);           // pixel index field of a hit record
+      fits = dcnv4_grad_value_lds_bytes(*L) <= kMaxLdsPerWorkgroup - 256;
     }
     if (fits) break;
     if (L->tile_h_log2 > 0 && L->tile_h_log2 >= L->tile_w_log2) --L->tile_h_log2;

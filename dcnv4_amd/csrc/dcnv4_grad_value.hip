@@ -8,26 +8,23 @@
 //
 //   * a workgroup OWNS a tile_h x tile_w tile of the input image for a chunk of groups, and is
 //     the only writer of that part of grad_value: plain stores, no clearing pass, no cast pass;
-//   * it visits every output pixel whose reference point lies within `reach` pixels of the tile
-//     (strip by strip, offset_mask slices staged in LDS), recomputes the bilinear corners, and
-//     accumulates the corners that land inside its tile into LDS with 64-bit integer atomics on
-//     fixed-point values: results are bit-reproducible, independent of scheduling;
+//   * it visits every output pixel whose reference point lies within `reach` pixels of the tile,
+//     strip by strip, in two phases per strip:
+//       A  tap-parallel: one lane per (pixel, group, kernel tap) recomputes the sampling position
+//          and, when a corner lands inside the tile, appends a hit record (four accumulator cells,
+//          four weights, pixel) to a per-group list in LDS; the strip's grad_out is parked in LDS;
+//       B  channel-parallel: a row of 16 lanes takes one hit record, lane c owns channel c (+16j),
+//          and adds its four corner contributions with 64-bit integer LDS atomics on fixed-point
+//          values.  Row r of every wave serves group r of the chunk, so with 16 channels per group
+//          one ds_add_u64 instruction touches 64 distinct channels: two conflict-free bank sweeps;
 //   * fixed point: contributions are normalised by the global maxima of |grad_out| and
 //     |modulation| (GradState, produced by the grad_offset_mask kernel that runs first) and carry
 //     `fix_bits` fractional bits, i.e. an absolute resolution of 2^-fix_bits of the largest possible
-//     contribution - finer than fp32 accumulation unless a sum is > 2^25 times smaller than that;
+//     contribution - finer than fp32 accumulation unless a sum is > 2^25 times smaller than that.
+//     Integer sums make the result bit-reproducible, independent of scheduling;
 //   * corners farther than `reach` from their output pixel's tile, and the case of non-finite
 //     statistics, are left to the fallback scatter kernel (dcnv4_kernels.hip, kBwdFallback),
 //     which runs afterwards and does nothing in the common case.
-//
-// Lane layout: a row of 16 lanes owns one (output pixel, group); lane c owns channels c, c+16, ...
-// A wave is four rows - the four groups of one pixel when ng_chunk = 4, D = 16 - so one
-// ds_add_u64 instruction covers 64 distinct channels of 4 cells: exactly two conflict-free
-// sweeps of the 64 LDS banks.  The 16 lanes of a row first work tap-parallel (lane t computes
-// tap t: position, weights, cell index, validity), then each tap's results are broadcast along
-// the row with DPP row_newbcast and every lane adds its own channel.
-#include <utility>
-
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -36,20 +33,10 @@ namespace {
 
 constexpr int kValThreads = 1024;
 constexpr int kRow = 16;
+constexpr int kWaves = kValThreads / kWave;
 constexpr int kTrashPad = 64;
-constexpr int kStageBatch = 8;     // independent staging loads in flight per thread
-constexpr int kPassBatch = 4;      // row passes whose grad_out loads are issued together
-
-template <int K> __device__ __forceinline__ float row_bcast_f(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x150 + K, 0xf, 0xf, false));
-}
-template <int K> __device__ __forceinline__ int row_bcast_i(int v) {
-  return __builtin_amdgcn_update_dpp(0, v, 0x150 + K, 0xf, 0xf, false);
-}
-__device__ __forceinline__ int row_bcast_dyn(int v, int k) {   // k < 16, same for the whole wave
-  const int lane = threadIdx.x & (kWave - 1);
-  return __builtin_amdgcn_ds_bpermute(((lane & ~(kRow - 1)) + k) << 2, v);
-}
+constexpr int kMaxChunkGroups = 4;      // rows of a wave <-> groups of the chunk
+constexpr int kCellBits = 9;            // cell index 0..n_cells (n_cells = trash), tiles up to 16x16
 
 // float (|t| < 2^62) -> two's-complement 64-bit integer, exact (t carries 24 significant bits).
 __device__ __forceinline__ unsigned long long to_fixed(float t) {
@@ -59,10 +46,9 @@ __device__ __forceinline__ unsigned long long to_fixed(float t) {
   return ((unsigned long long)(uint32_t)hi << 32) | lo;
 }
 
-struct RowTap {       // what lane t of a row holds for tap t
-  int cell_off;       // ((y0 - tile_y0) * tile_w + (x0 - tile_x0)) * ch_stride; corners add 0, 1, tile_w, tile_w+1 cells
-  int valid;          // bit c: corner c is inside the image and inside this tile
-  float w[4];         // modulation * bilinear weight on the fixed-point grid, 0 for corners that are not valid
+struct HitMeta {
+  uint32_t cells012;    // accumulator cell of corners 0,1,2 (9 bits each); n_cells = "nowhere" (weight 0)
+  uint32_t cell3_px;    // cell of corner 3 | strip-local pixel << 9
 };
 
 template <typename Tag, int KP, int CPL>
@@ -81,13 +67,15 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   const int ty0 = ty << p.tile_h_log2, tx0 = tx << p.tile_w_log2;
   const int th = min(p.tile_h, p.H - ty0), tw = min(p.tile_w, p.W - tx0);
   const int n_cells = p.tile_h * p.tile_w;
-  // the slots past the tile absorb the zero-valued adds of lanes whose corner is not in the tile,
-  // and of lanes whose channel index runs past D (group widths that are not multiples of 16)
-  const int trash_off = n_cells * ch_stride;
-  const int n_acc = trash_off + ch_stride + kTrashPad;
+  // the slots past the tile absorb the zero-valued adds of corners outside the tile, and of lanes
+  // whose channel index runs past D (group widths that are not multiples of 16)
+  const int n_acc = ((n_cells + 1) * ch_stride + kTrashPad + 1) & ~1;      // even: keeps the lists 16-byte aligned
+  const int list_cap = p.strip_pix * Kp;                // hit records per group list
   unsigned long long *acc = lds64;
-  float *s_om = reinterpret_cast<float *>(lds64 + n_acc);
-  const int slice = ng * 3 * Kp;                        // staged offset_mask elements per pixel
+  f32x4 *hit_w = reinterpret_cast<f32x4 *>(lds64 + n_acc);                       // [ng_chunk][list_cap]
+  HitMeta *hit_meta = reinterpret_cast<HitMeta *>(hit_w + p.ng_chunk * list_cap);  // [ng_chunk][list_cap]
+  float *s_go = reinterpret_cast<float *>(hit_meta + p.ng_chunk * list_cap);       // [strip_pix][ch_stride]
+  uint32_t *s_count = reinterpret_cast<uint32_t *>(s_go + p.strip_pix * ch_stride);  // [kMaxChunkGroups]
 
   const uint32_t gmax = p.state->go_max_bits, mmax = p.state->mask_max_bits;
   const bool finite = gmax < 0x7f800000u && mmax < 0x7f800000u;
@@ -111,146 +99,179 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   typedef typename RawWord<Tag::kBytes>::type elem_t;
   const elem_t *om_g = reinterpret_cast<const elem_t *>(p.offset_mask);
   const elem_t *go_g = reinterpret_cast<const elem_t *>(p.grad_out);
+  auto load_f = [](const elem_t *ptr) { float f[1]; Pack<Tag, 1>::decode(*ptr, f); return f[0]; };
 
   if (finite && nwx > 0 && ho_hi > ho_lo && (gmax | mmax) != 0) {
     const int rows_per_strip = max(1, p.strip_pix / nwx);
-    for (int hs = ho_lo; hs < ho_hi; hs += rows_per_strip) {
-      const int nrows = min(rows_per_strip, ho_hi - hs);
-      const int npx = nrows * nwx;
-      __syncthreads();      // previous strip fully consumed (and acc cleared, first time round)
-      // stage the strip's offset_mask slices: thread -> (pixel, element), all loads of a thread
-      // issued back to back before the first LDS write so their latencies overlap
-      {
-        const int e_lanes = slice <= 128 ? 128 : (slice <= 256 ? 256 : 1024);
-        const int e0 = threadIdx.x & (e_lanes - 1), px_step = kValThreads / e_lanes;
-        for (int e = e0; e < slice; e += e_lanes) {
-          for (int pxb = threadIdx.x / e_lanes; pxb < npx; pxb += kStageBatch * px_step) {
-            elem_t raw[kStageBatch];
+    const float inv_nwx = 1.f / (float)nwx;
+    constexpr int kStageRounds = 2;     // pixels per wave whose grad_out is prefetched (16 waves: 32 pixels)
+    constexpr int kStageChunks = 1;     // 64-channel chunks of a pixel that are prefetched
+    struct Prefetch {
+      elem_t ox, oy, m;                               // phase A, first round: this lane's tap
+      elem_t go[kStageRounds][kStageChunks];          // staging: this lane's channel of up to two pixels
+    };
+
+    // phase A work item of (round, wave, lane): group, pixel, tap; valid == false past the end
+    struct Item { int gl, px, t, ho, wo; bool valid; const elem_t *om; };
+    auto item_of = [&](int wk, int hs, int npx) {
+      Item it;
+      const int per_group = npx * Kp, waves_per_group = (per_group + kWave - 1) / kWave;
+      it.gl = wk / waves_per_group;                                          // scalar: same for the wave
+      const int j = (wk - it.gl * waves_per_group) * kWave + lane;
+      it.valid = it.gl < ng && j < per_group;
+      it.px = KP > 0 ? j / KP : j / Kp;
+      it.t = j - it.px * Kp;
+      if (!it.valid) { it.gl = 0; it.px = 0; it.t = 0; }
+      const int r = (int)(((float)it.px + 0.5f) * inv_nwx);                  // exact: px < 1024
+      it.ho = hs + r; it.wo = wo_lo + (it.px - r * nwx);
+      it.om = om_g + ((size_t)b * p.Q + (size_t)it.ho * p.Wo + it.wo) * p.P_pad + (g0 + it.gl) * 3 * Kp;
+      return it;
+    };
+    auto go_row = [&](int px, int hs) {
+      const int r = px / nwx, wx = px - r * nwx;
+      return go_g + ((size_t)b * p.Q + (size_t)(hs + r) * p.Wo + wo_lo + wx) * C + g0 * D;
+    };
+    // loads of the next strip, issued before the current strip's phase B so their latency hides there
+    auto prefetch = [&](int hs, int npx) {
+      Prefetch pf;
+      const Item it = item_of(wave, hs, npx);
+      pf.ox = pf.oy = pf.m = elem_t(0);
+      if (it.valid) { pf.ox = it.om[2 * it.t]; pf.oy = it.om[2 * it.t + 1]; pf.m = it.om[2 * Kp + it.t]; }
 #pragma unroll
-            for (int u = 0; u < kStageBatch; ++u) {
-              const int px = pxb + u * px_step;
-              raw[u] = elem_t(0);
-              if (px < npx) {
-                const int r = px / nwx, wx = px - r * nwx;
-                raw[u] = om_g[((size_t)b * p.Q + (size_t)(hs + r) * p.Wo + wo_lo + wx) * p.P_pad + g0 * 3 * Kp + e];
-              }
-            }
+      for (int u = 0; u < kStageRounds; ++u) {
+        const int px = wave + u * kWaves;
 #pragma unroll
-            for (int u = 0; u < kStageBatch; ++u) {
-              const int px = pxb + u * px_step;
-              if (px < npx) {
-                float f[1];
-                Pack<Tag, 1>::decode(raw[u], f);
-                s_om[px * slice + e] = f[0];
-              }
+        for (int v = 0; v < kStageChunks; ++v) {
+          const int ch = lane + v * kWave;
+          pf.go[u][v] = elem_t(0);
+          if (px < npx && ch < ng * D) pf.go[u][v] = go_row(px, hs)[ch];
+        }
+      }
+      return pf;
+    };
+    auto to_f = [](elem_t raw) { float f[1]; Pack<Tag, 1>::decode(raw, f); return f[0]; };
+
+    int hs = ho_lo;
+    int npx = min(rows_per_strip, ho_hi - hs) * nwx;
+    Prefetch pf = prefetch(hs, npx);
+    if (threadIdx.x < 2 * kMaxChunkGroups) s_count[threadIdx.x] = 0u;
+
+    for (int s_idx = 0; hs < ho_hi; ++s_idx) {
+      uint32_t *count = s_count + (s_idx & 1) * kMaxChunkGroups;
+      __syncthreads();      // previous strip's phase B is done (first time: acc and counters are clear)
+
+      // ---- park the strip's grad_out (this chunk's channels), normalised to [-1, 1]: a wave per pixel
+      for (int px = wave, u = 0; px < npx; px += kWaves, ++u)
+        for (int ch = lane, v = 0; ch < ch_stride; ch += kWave, ++v) {
+          float g = 0.f;
+          if (ch < ng * D) g = (u < kStageRounds && v < kStageChunks) ? to_f(u == 0 ? pf.go[0][0] : pf.go[kStageRounds - 1][0])
+                                                                     : load_f(go_row(px, hs) + ch);
+          s_go[px * ch_stride + ch] = ldexpf(g, -e_go);
+        }
+
+      // ---- phase A: one lane per (group, pixel, tap); a wave never mixes groups
+      const int n_wk = ng * ((npx * Kp + kWave - 1) / kWave);
+      for (int wk = wave, round = 0; wk < n_wk; wk += kWaves, ++round) {
+        const Item it = item_of(wk, hs, npx);
+        bool hit = false;
+        f32x4 w = {0.f, 0.f, 0.f, 0.f};
+        HitMeta meta = {0u, 0u};
+        if (it.valid) {
+          const float off_x = round == 0 ? to_f(pf.ox) : load_f(it.om + 2 * it.t);
+          const float off_y = round == 0 ? to_f(pf.oy) : load_f(it.om + 2 * it.t + 1);
+          int ti, tj;
+          if constexpr (KP > 0) {
+            tap_ij_3x3(KP, it.t, ti, tj);
+          } else {      // x index outer, y index inner, centre skipped when remove_center
+            int tt = it.t;
+            if (p.remove_center && tt >= (p.kw / 2) * p.kh + p.kh / 2) ++tt;
+            ti = tt / p.kh; tj = tt - ti * p.kh;
+          }
+          const float x_base = sub_rn((float)(cx0 + it.wo * p.sw), x_sub), y_base = sub_rn((float)(cy0 + it.ho * p.sh), y_sub);
+          const float x = add_rn(x_base, mul_rn(add_rn((float)(ti * p.dw), off_x), p.offset_scale));
+          const float y = add_rn(y_base, mul_rn(add_rn((float)(tj * p.dh), off_y), p.offset_scale));
+          const Tap tp = make_tap(y, x, p.H, p.W, 0u, 0u);
+          const int ly = tp.y0 - ty0, lx = tp.x0 - tx0;
+          const bool r0 = ly >= 0 && ly < th, r1 = ly + 1 >= 0 && ly + 1 < th;
+          const bool c0 = lx >= 0 && lx < tw, c1 = lx + 1 >= 0 && lx + 1 < tw;
+          const uint32_t valid = tp.valid & ((uint32_t)(r0 && c0) | ((uint32_t)(r0 && c1) << 1) |
+                                             ((uint32_t)(r1 && c0) << 2) | ((uint32_t)(r1 && c1) << 3));
+          hit = valid != 0;
+          if (hit) {
+            float m = round == 0 ? to_f(pf.m) : load_f(it.om + 2 * Kp + it.t);
+            if (p.softmax) {          // rare: normalise over this group's taps
+              float mx = load_f(it.om + 2 * Kp), sum = 0.f;
+              for (int k = 1; k < Kp; ++k) mx = fmaxf(mx, load_f(it.om + 2 * Kp + k));
+              for (int k = 0; k < Kp; ++k) sum += __expf(load_f(it.om + 2 * Kp + k) - mx);
+              m = __expf(m - mx) / sum;
             }
+            const float ms = ldexpf(m, p.fix_bits - e_m);
+            const int cell = (ly << p.tile_w_log2) + lx;
+            uint32_t cells[4];
+#pragma unroll
+            for (int cn = 0; cn < 4; ++cn) {
+              const bool ok = valid & (1u << cn);
+              cells[cn] = ok ? (uint32_t)(cell + (cn >> 1) * p.tile_w + (cn & 1)) : (uint32_t)n_cells;
+              w[cn] = ok ? ms * tp.w[cn] : 0.f;
+            }
+            meta.cells012 = cells[0] | (cells[1] << kCellBits) | (cells[2] << (2 * kCellBits));
+            meta.cell3_px = cells[3] | ((uint32_t)it.px << kCellBits);
+          }
+        }
+        // append the wave's hits to its group's list: one LDS counter bump per wave
+        const uint64_t mask = __builtin_amdgcn_ballot_w64(hit);
+        if (mask != 0) {
+          uint32_t base = 0;
+          if (lane == 0) base = atomicAdd(&count[it.gl], (uint32_t)__builtin_popcountll(mask));
+          base = __builtin_amdgcn_readfirstlane(base);
+          if (hit) {
+            const uint32_t slot = it.gl * list_cap + base +
+                                  __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+            hit_w[slot] = w;
+            hit_meta[slot] = meta;
           }
         }
       }
       __syncthreads();
 
-      const int n_items = npx * ng;
-      constexpr int kItemStep = kValThreads / kRow;       // rows of 16 lanes per workgroup pass
-      for (int itemb = wave * 4; itemb < n_items; itemb += kPassBatch * kItemStep) {
-       // grad_out of the next kPassBatch passes: loads issued together, latencies overlap
-       elem_t go_raw[kPassBatch][CPL];
-#pragma unroll
-       for (int u = 0; u < kPassBatch; ++u) {
-         const int item = itemb + u * kItemStep + row_in_wave;
-         const int px = item < n_items ? item / ng : 0, gl = item < n_items ? item - px * ng : 0;
-         const int r = px / nwx, wx = px - r * nwx;
-         const elem_t *gsrc = go_g + ((size_t)b * p.Q + (size_t)(hs + r) * p.Wo + wo_lo + wx) * C + (g0 + gl) * D;
-#pragma unroll
-         for (int j = 0; j < CPL; ++j) {
-           go_raw[u][j] = elem_t(0);
-           if (item < n_items && c + kRow * j < D) go_raw[u][j] = gsrc[c + kRow * j];
-         }
-       }
-#pragma unroll
-       for (int u = 0; u < kPassBatch; ++u) {
-        const int item0 = itemb + u * kItemStep;
-        if (item0 >= n_items) break;
-        const int item = item0 + row_in_wave;
-        const bool live = item < n_items;
-        const int px = live ? item / ng : 0, gl = live ? item - px * ng : 0;
-        const int r = px / nwx, wx = px - r * nwx;
-        const int ho = hs + r, wo = wo_lo + wx;
-        const float *om = s_om + px * slice + gl * 3 * Kp;
-        // this lane's channels of grad_out, normalised to [-1, 1]; channels past D stay 0
+      // next strip's loads fly while this strip's hits are applied; the other counter set is idle
+      const int hs_next = hs + rows_per_strip;
+      const int npx_next = hs_next < ho_hi ? min(rows_per_strip, ho_hi - hs_next) * nwx : 0;
+      if (npx_next > 0) pf = prefetch(hs_next, npx_next);
+      if (threadIdx.x < kMaxChunkGroups) s_count[((s_idx + 1) & 1) * kMaxChunkGroups + threadIdx.x] = 0u;
+
+      // ---- phase B: row r of each wave drains list r, 16 lanes = 16 channels (x CPL)
+      const uint32_t n_mine = row_in_wave < ng ? count[row_in_wave] : 0u;
+      uint32_t n_max = count[0];
+      for (int g = 1; g < ng; ++g) n_max = max(n_max, count[g]);
+      const int my_group = row_in_wave < ng ? row_in_wave : 0;      // idle rows only ever add zeros to the trash slots
+      unsigned long long *acc_lane = acc + my_group * D + c;
+      const float *go_lane = s_go + my_group * D + c;
+      for (uint32_t i = wave; i < n_max; i += kWaves) {
+        f32x4 w = {0.f, 0.f, 0.f, 0.f};
+        HitMeta meta = {(uint32_t)n_cells | ((uint32_t)n_cells << kCellBits) | ((uint32_t)n_cells << (2 * kCellBits)),
+                        (uint32_t)n_cells};
+        if (i < n_mine) {
+          w = hit_w[row_in_wave * list_cap + i];
+          meta = hit_meta[row_in_wave * list_cap + i];
+        }
+        const int px = meta.cell3_px >> kCellBits;
         float gn[CPL];
 #pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-          float f[1];
-          Pack<Tag, 1>::decode(go_raw[u][j], f);
-          gn[j] = ldexpf(f[0], -e_go);
+        for (int j = 0; j < CPL; ++j) gn[j] = (c + kRow * j < D) ? go_lane[px * ch_stride + kRow * j] : 0.f;
+        const uint32_t cells[4] = {meta.cells012 & 511u, (meta.cells012 >> kCellBits) & 511u,
+                                   (meta.cells012 >> (2 * kCellBits)) & 511u, meta.cell3_px & 511u};
+        const float wv[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn) {
+          unsigned long long *dst = acc_lane + __umul24(cells[cn], (uint32_t)ch_stride);
+#pragma unroll
+          for (int j = 0; j < CPL; ++j)
+            __hip_atomic_fetch_add(dst + kRow * j, to_fixed(gn[j] * wv[cn]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
-        float mx = 0.f, inv = 1.f;
-        if (p.softmax && live) softmax_stats(om + 2 * Kp, Kp, mx, inv);
-        const float x_base = sub_rn((float)(cx0 + wo * p.sw), x_sub), y_base = sub_rn((float)(cy0 + ho * p.sh), y_sub);
-        unsigned long long *acc_lane = acc + gl * D + c;
-
-        for (int t0 = 0; t0 < Kp; t0 += kRow) {           // 16 taps at a time, one per lane
-          RowTap rt;
-          rt.cell_off = trash_off; rt.valid = 0;
-          rt.w[0] = rt.w[1] = rt.w[2] = rt.w[3] = 0.f;
-          const int t = t0 + c;
-          if (live && t < Kp) {
-            int i, j;
-            if constexpr (KP > 0) {
-              tap_ij_3x3(KP, t, i, j);
-            } else {
-              // x index outer, y index inner, centre skipped when remove_center
-              int tt = t;
-              if (p.remove_center && tt >= (p.kw / 2) * p.kh + p.kh / 2) ++tt;
-              i = tt / p.kh; j = tt - i * p.kh;
-            }
-            const float x = add_rn(x_base, mul_rn(add_rn((float)(i * p.dw), om[2 * t]), p.offset_scale));
-            const float y = add_rn(y_base, mul_rn(add_rn((float)(j * p.dh), om[2 * t + 1]), p.offset_scale));
-            float m = om[2 * Kp + t];
-            if (p.softmax) m = __expf(m - mx) * inv;
-            const Tap tp = make_tap(y, x, p.H, p.W, 0u, 0u);
-            const int ly = tp.y0 - ty0, lx = tp.x0 - tx0;
-            const bool r0 = ly >= 0 && ly < th, r1 = ly + 1 >= 0 && ly + 1 < th;
-            const bool c0 = lx >= 0 && lx < tw, c1 = lx + 1 >= 0 && lx + 1 < tw;
-            rt.valid = (int)(tp.valid & ((uint32_t)(r0 && c0) | ((uint32_t)(r0 && c1) << 1) | ((uint32_t)(r1 && c0) << 2) |
-                                         ((uint32_t)(r1 && c1) << 3)));
-            rt.cell_off = ((ly << p.tile_w_log2) + lx) * ch_stride;
-            const float ms = ldexpf(m, p.fix_bits - e_m);
-#pragma unroll
-            for (int cn = 0; cn < 4; ++cn) rt.w[cn] = (rt.valid & (1 << cn)) ? ms * tp.w[cn] : 0.f;
-          }
-          auto scatter_tap = [&](int cell_off, int valid, float w0, float w1, float w2, float w3) {
-            if (__builtin_amdgcn_ballot_w64(valid != 0) == 0) return;       // nobody in the wave hits the tile
-            const float w[4] = {w0, w1, w2, w3};
-#pragma unroll
-            for (int cn = 0; cn < 4; ++cn) {
-              const bool ok = valid & (1 << cn);
-              if (__builtin_amdgcn_ballot_w64(ok) == 0) continue;
-              const int off = ok ? cell_off + ((cn >> 1) * p.tile_w + (cn & 1)) * ch_stride : trash_off;
-#pragma unroll
-              for (int j = 0; j < CPL; ++j)
-                __hip_atomic_fetch_add(acc_lane + off + kRow * j, to_fixed(gn[j] * w[cn]), __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_WORKGROUP);
-            }
-          };
-          if constexpr (KP > 0) {
-            auto unrolled = [&]<int... Ks>(std::integer_sequence<int, Ks...>) {
-              (scatter_tap(row_bcast_i<Ks>(rt.cell_off), row_bcast_i<Ks>(rt.valid), row_bcast_f<Ks>(rt.w[0]),
-                           row_bcast_f<Ks>(rt.w[1]), row_bcast_f<Ks>(rt.w[2]), row_bcast_f<Ks>(rt.w[3])), ...);
-            };
-            unrolled(std::make_integer_sequence<int, KP>{});
-          } else {
-            const int nt = min(kRow, Kp - t0);
-            for (int k = 0; k < nt; ++k)
-              scatter_tap(row_bcast_dyn(rt.cell_off, k), row_bcast_dyn(rt.valid, k),
-                          __builtin_bit_cast(float, row_bcast_dyn(__builtin_bit_cast(int, rt.w[0]), k)),
-                          __builtin_bit_cast(float, row_bcast_dyn(__builtin_bit_cast(int, rt.w[1]), k)),
-                          __builtin_bit_cast(float, row_bcast_dyn(__builtin_bit_cast(int, rt.w[2]), k)),
-                          __builtin_bit_cast(float, row_bcast_dyn(__builtin_bit_cast(int, rt.w[3]), k)));
-          }
-        }
-       }
       }
+      hs = hs_next;
+      npx = npx_next;
     }
   }
   __syncthreads();
@@ -307,8 +328,10 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
 }  // namespace
 
 size_t dcnv4_grad_value_lds_bytes(const DcnLaunch &p) {
-  return ((size_t)(p.tile_h * p.tile_w + 1) * p.ng_chunk * p.D + kTrashPad) * sizeof(unsigned long long) +
-         (size_t)p.strip_pix * p.ng_chunk * 3 * p.Kp * sizeof(float);
+  const size_t ch_stride = (size_t)p.ng_chunk * p.D, list = (size_t)p.ng_chunk * p.strip_pix * p.Kp;
+  return ((((size_t)(p.tile_h * p.tile_w + 1) * ch_stride + kTrashPad + 1) & ~size_t(1)) * sizeof(unsigned long long)) +  // accumulators
+         list * (sizeof(f32x4) + sizeof(HitMeta)) +                                                    // hit lists
+         (size_t)p.strip_pix * ch_stride * sizeof(float) + 2 * kMaxChunkGroups * sizeof(uint32_t);     // grad_out, two counter sets
 }
 
 hipError_t launch_dcnv4_grad_value(int dtype, const DcnLaunch &p, hipStream_t stream) {
