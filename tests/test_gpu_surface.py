@@ -1,0 +1,242 @@
+"""GPU tests of the Python surface (autograd Functions, nn.Modules) and of size-independent
+properties at the benchmark's full sizes, where the CPU oracle would take too long:
+adjoint identities (the operator is linear in value and in the modulation), bit-reproducibility,
+batch chunking, non-finite gradients, HIP-graph replay."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import torch_core
+from tests import cabi
+from tests.inputs import make_dcnv4_inputs, make_fda_inputs
+
+pytestmark = pytest.mark.gpu
+GEOM = (3, 3, 1, 1, 1, 1, 1, 1)
+
+
+def _rel_err(a, b):
+    a, b = a.double(), b.double()
+    return float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
+
+
+def test_dcnv4_function_autograd_matches_grid_sample_autograd():
+    import dcnv4_amd
+    B, H, W, G, D = 2, 12, 10, 4, 16
+    v, om, go = make_dcnv4_inputs(B, H, W, G, D, seed=4)
+    vd, omd = v.cuda().requires_grad_(True), om.cuda().requires_grad_(True)
+    out = dcnv4_amd.DCNv4Function.apply(vd, omd, *GEOM, G, D, 1.0, 256, 0)
+    out.backward(go.cuda())
+    v64, om64 = v.double().requires_grad_(True), om.double().requires_grad_(True)
+    ref = torch_core.dcnv4_core_torch(v64, om64, *GEOM, G, D, 1.0)
+    ref.backward(go.double())
+    assert out.shape == ref.shape and out.dtype == torch.float32
+    assert _rel_err(out.cpu(), ref.detach()) < 1e-4
+    assert _rel_err(vd.grad.cpu(), v64.grad) < 1e-3
+    assert _rel_err(omd.grad.cpu(), om64.grad) < 1e-3
+    assert vd.grad.dtype == torch.float32 and omd.grad.shape == om.shape
+
+
+def test_flash_deform_attn_function_autograd_matches_grid_sample_autograd():
+    import dcnv4_amd
+    shapes = [(10, 12), (5, 6), (3, 3)]
+    v, shp, st, sla, go = make_fda_inputs(2, shapes, 4, 32, 4, Q=60, seed=6)
+    vd, sd = v.cuda().requires_grad_(True), sla.cuda().requires_grad_(True)
+    out = dcnv4_amd.FlashDeformAttnFunction.apply(vd, shp.cuda(), st.cuda(), sd, 64, 4)
+    out.backward(go.cuda())
+    v64, s64 = v.double().requires_grad_(True), sla.double().requires_grad_(True)
+    ref = torch_core.msda_core_torch(v64, shapes, st.tolist(), s64, 4)
+    ref.backward(go.double())
+    assert out.shape == (2, 60, 128)
+    assert _rel_err(out.cpu(), ref.detach()) < 1e-4
+    assert _rel_err(vd.grad.cpu(), v64.grad) < 1e-3
+    assert _rel_err(sd.grad.cpu(), s64.grad) < 1e-3
+
+
+@pytest.mark.parametrize("kwargs", [dict(), dict(dw_kernel_size=3, center_feature_scale=True, remove_center=True, offset_scale=0.5),
+                                    dict(without_pointwise=True, output_bias=False)])
+def test_dcnv4_module_matches_a_reference_built_from_torch_ops(kwargs):
+    import dcnv4_amd
+    torch.manual_seed(0)
+    C, G, H, W, N = 64, 4, 9, 7, 2
+    m = dcnv4_amd.DCNv4(channels=C, group=G, **kwargs)
+    with torch.no_grad():       # the module initialises offsets to zero; give them something to do
+        m.offset_mask.weight.normal_(0, 0.3)
+        m.offset_mask.bias.normal_(0, 0.5)
+        if m.center_feature_scale:
+            m.center_feature_scale_proj_weight.normal_(0, 0.2)
+    x = torch.randn(N, H * W, C)
+
+    def reference(mod, inp):
+        xx = inp if mod.without_pointwise else mod.value_proj(inp)
+        xx = xx.reshape(N, H, W, -1)
+        src = inp
+        if mod.dw_kernel_size is not None:
+            src = mod.offset_mask_dw(inp.view(N, H, W, C).permute(0, 3, 1, 2)).permute(0, 2, 3, 1).reshape(N, H * W, C)
+        om = mod.offset_mask(src).reshape(N, H, W, -1)
+        y = torch_core.dcnv4_core_torch(xx, om, mod.kernel_size, mod.kernel_size, mod.stride, mod.stride, mod.pad, mod.pad,
+                                        mod.dilation, mod.dilation, mod.group, mod.group_channels, mod.offset_scale,
+                                        mod.remove_center)
+        if mod.center_feature_scale:
+            s = F.linear(y, mod.center_feature_scale_proj_weight, mod.center_feature_scale_proj_bias).sigmoid()
+            s = s[..., None].repeat(1, 1, 1, 1, mod.channels // mod.group).flatten(-2)
+            y = y * (1 - s) + xx * s
+        y = y.view(N, H * W, -1)
+        return y if mod.without_pointwise else mod.output_proj(y)
+
+    want = reference(m, x)
+    xg = x.clone().requires_grad_(True)
+    reference(m, xg).sum().backward()
+    md = m.cuda()
+    xd = x.cuda().requires_grad_(True)
+    got = md(xd, shape=(H, W), level_idx=0)
+    got.sum().backward()
+    assert _rel_err(got.detach().cpu(), want.detach()) < 2e-4
+    assert _rel_err(xd.grad.cpu(), xg.grad) < 2e-3
+
+
+def test_flash_deform_attn_module_matches_a_reference_built_from_torch_ops():
+    import dcnv4_amd
+    torch.manual_seed(1)
+    shapes = [(8, 8), (4, 4)]
+    m = dcnv4_amd.FlashDeformAttn(d_model=64, n_levels=2, n_heads=4, n_points=4)
+    with torch.no_grad():
+        m.attention_weights.weight.normal_(0, 0.2)
+        m.sampling_offsets.weight.normal_(0, 0.05)
+    N, Lq, S = 2, 30, 80
+    q, feat = torch.randn(N, Lq, 64), torch.randn(N, S, 64)
+    ref_pts = torch.rand(N, Lq, 2, 2)
+    shp = torch.tensor(shapes)
+    starts = torch.tensor([0, 64])
+    pad = torch.zeros(N, S, dtype=torch.bool)
+    pad[0, -5:] = True
+    value = m.value_proj(feat).masked_fill(pad[..., None], 0.0).view(N, S, 4, 16)
+    off = m.sampling_offsets(q).view(N, Lq, 4, 2, 4, 2)
+    logits = m.attention_weights(q).view(N, Lq, 4, 8)
+    norm = torch.stack([shp[..., 1], shp[..., 0]], -1)
+    loc = ref_pts[:, :, None, :, None, :] + off / norm[None, None, None, :, None, :]
+    sla = torch.cat([loc.flatten(-3).half().float(), logits], -1)       # locations pass through fp16 in the module
+    want = m.output_proj(torch_core.msda_core_torch(value, shapes, [0, 64], sla, 4))
+    md = m.cuda()
+    got = md(q.cuda(), ref_pts.cuda(), feat.cuda(), shp.cuda(), starts.cuda(), pad.cuda())
+    assert _rel_err(got.detach().cpu(), want.detach()) < 2e-4
+
+
+def test_backward_is_bit_reproducible():
+    B, H, W, G, D = 4, 28, 28, 8, 16
+    v, om, go = (t.cuda() for t in make_dcnv4_inputs(B, H, W, G, D, offset_range=3.0, seed=8, dtype=torch.float16))
+    first = cabi.dcnv4_backward(v, om, go, GEOM, G, D, 1.0)
+    for _ in range(3):
+        again = cabi.dcnv4_backward(v, om, go, GEOM, G, D, 1.0)
+        assert torch.equal(first[0], again[0]) and torch.equal(first[1], again[1])
+
+
+def test_nan_in_grad_output_propagates_like_the_oracle(oracle):
+    B, H, W, G, D = 1, 10, 10, 2, 16
+    v, om, go = make_dcnv4_inputs(B, H, W, G, D, seed=9)
+    go[0, 4, 5, 3] = float("nan")
+    go[0, 2, 2, 20] = float("inf")
+    wgv, wgom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *GEOM, G, D, 1.0, coord_f32=True)
+    gv, gom = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), GEOM, G, D, 1.0)
+    gv, gom = cabi.f64(gv), cabi.f64(gom)
+    assert np.array_equal(np.isfinite(gv), np.isfinite(wgv)) and np.array_equal(np.isnan(gv), np.isnan(wgv))
+    ok = np.isfinite(wgv)
+    np.testing.assert_allclose(gv[ok], wgv[ok], rtol=1e-3, atol=1e-4)
+    assert np.array_equal(np.isfinite(gom), np.isfinite(wgom))
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.float16, 3e-3)], ids=["fp32", "fp16"])
+def test_dcnv4_adjoint_identities_at_full_benchmark_size(dtype, tol):
+    # out is linear in value and in the modulation scalars, so with g = grad_out:
+    #   <g, out> = <grad_value, value> = <grad_mask, mask>          (B=64, 56x56, C=64, G=4)
+    torch.manual_seed(3)
+    B, H, W, G, D, K = 64, 56, 56, 4, 16, 9
+    dev = "cuda"
+    v = torch.randn(B, H, W, G * D, device=dev).to(dtype)
+    body = torch.cat([(torch.rand(B, H, W, G, 2 * K, device=dev) * 6 - 3), torch.randn(B, H, W, G, K, device=dev)], -1)
+    om = torch.zeros(B, H, W, 112, device=dev)
+    om[..., :108] = body.reshape(B, H, W, 108)
+    om = om.to(dtype)
+    g = torch.randn(B, H, W, G * D, device=dev).to(dtype)
+    out = cabi.dcnv4_forward(v, om, GEOM, G, D, 1.0)
+    gv, gom = cabi.dcnv4_backward(v, om, g, GEOM, G, D, 1.0)
+    lhs = (g.double() * out.double()).sum()
+    by_value = (gv.double() * v.double()).sum()
+    mask = om[..., :108].reshape(B, H, W, G, 27)[..., 18:].double()
+    gmask = gom[..., :108].reshape(B, H, W, G, 27)[..., 18:].double()
+    by_mask = (gmask * mask).sum()
+    scale = (g.double().abs() * out.double().abs()).sum()
+    assert abs(float(lhs - by_value)) / float(scale) < tol
+    assert abs(float(lhs - by_mask)) / float(scale) < tol
+    assert (gom[..., 108:] == 0).all()
+
+
+def test_flash_deform_attn_adjoint_identity_at_full_benchmark_size():
+    torch.manual_seed(4)
+    shapes = [(128, 128), (64, 64), (32, 32), (16, 16)]
+    B, G, D, L, K = 4, 8, 32, 4, 4
+    N = sum(h * w for h, w in shapes)
+    dev = "cuda"
+    shp = torch.tensor(shapes, device=dev)
+    sizes = [h * w for h, w in shapes]
+    st = torch.tensor([sum(sizes[:i]) for i in range(L)], device=dev)
+    v = torch.randn(B, N, G, D, device=dev)
+    sla = torch.cat([torch.rand(B, N, G, L * K * 2, device=dev), torch.randn(B, N, G, L * K, device=dev)], -1)
+    g = torch.randn(B, N, G * D, device=dev)
+    out = cabi.fda_forward(v, shp, st, sla, K)
+    gv, gs = cabi.fda_backward(v, shp, st, sla, g, K)
+    lhs = (g.double() * out.double()).sum()
+    rhs = (gv.double() * v.double()).sum()
+    scale = (g.double().abs() * out.double().abs()).sum()
+    assert abs(float(lhs - rhs)) / float(scale) < 2e-5
+    # softmax Jacobian rows sum to zero
+    assert float(gs[..., 2 * L * K:].double().sum(-1).abs().max()) < 1e-3
+
+
+def test_batches_beyond_the_32_bit_addressing_span_are_chunked_consistently():
+    # value of 2.7 GB: more than one launch can address with 32-bit buffer offsets
+    torch.manual_seed(5)
+    B, H, W, G, D, K = 20, 512, 512, 8, 16, 9
+    dev = "cuda"
+    v = torch.randn(B, H, W, G * D, device=dev)
+    om = torch.zeros(B, H, W, 216, device=dev)
+    om[..., : 2 * K * G] = torch.rand(B, H, W, 2 * K * G, device=dev) * 4 - 2      # not the packing order: any values do
+    om[..., 2 * K * G:] = torch.randn(B, H, W, K * G, device=dev)
+    out = cabi.dcnv4_forward(v, om, GEOM, G, D, 1.0)
+    for lo, hi in [(0, 3), (9, 12), (17, 20)]:
+        part = cabi.dcnv4_forward(v[lo:hi].contiguous(), om[lo:hi].contiguous(), GEOM, G, D, 1.0)
+        assert torch.equal(out[lo:hi], part)
+    del out
+    g = torch.randn(B, H, W, G * D, device=dev)
+    gv, gom = cabi.dcnv4_backward(v, om, g, GEOM, G, D, 1.0)
+    pv, pom = cabi.dcnv4_backward(v[9:12].contiguous(), om[9:12].contiguous(), g[9:12].contiguous(), GEOM, G, D, 1.0)
+    assert torch.equal(gom[9:12], pom)
+    assert _rel_err(gv[9:12], pv) < 1e-6       # fixed-point scale comes from the global maxima of each call
+
+
+def test_forward_and_backward_replay_correctly_from_a_hip_graph():
+    B, H, W, G, D = 4, 20, 20, 4, 16
+    v, om, go = (t.cuda() for t in make_dcnv4_inputs(B, H, W, G, D, seed=10, dtype=torch.float16))
+    import dcnv4_amd
+    from dcnv4_amd import ext
+    eager_out = ext.dcnv4_forward(v, om, *GEOM, G, D, 1.0, 64, 0, 0, 0, False)
+    eager_gv, eager_gom = ext.dcnv4_backward(v, om, *GEOM, G, D, 1.0, 64, go, 0, 0, 0, False)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                       # warm up on the capture stream (allocator, lazy init)
+        ext.dcnv4_forward(v, om, *GEOM, G, D, 1.0, 64, 0, 0, 0, False)
+        ext.dcnv4_backward(v, om, *GEOM, G, D, 1.0, 64, go, 0, 0, 0, False)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_out = ext.dcnv4_forward(v, om, *GEOM, G, D, 1.0, 64, 0, 0, 0, False)
+        g_gv, g_gom = ext.dcnv4_backward(v, om, *GEOM, G, D, 1.0, 64, go, 0, 0, 0, False)
+    for _ in range(3):
+        g_out.fill_(7.0)
+        g_gv.fill_(7.0)
+        g_gom.fill_(7.0)
+        (v.float() @ torch.ones(64, 8, device="cuda")).sum().item()      # unrelated eager work + sync between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_out, eager_out) and torch.equal(g_gv, eager_gv) and torch.equal(g_gom, eager_gom)

@@ -1,0 +1,118 @@
+"""CPU-only checks of the host side: the C ABI exports what the header declares, the ctypes
+signatures match the header, launch hints are well-formed, the nn.Modules keep the reference's
+parameter names and shapes, and everything refuses to run without a GPU instead of falling back."""
+import ctypes
+import math
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "dcnv4_gfx950.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    decls = re.findall(r"\b(?:int|size_t|const char \*)\s*\*?\s*(\w+)\s*\(([^;{]*)\)\s*;", text)
+    return {name: args for name, args in decls}
+
+
+def test_library_exports_every_symbol_the_header_declares():
+    from dcnv4_amd import _lib
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    declared = _declared_functions()
+    assert len(declared) == 8, sorted(declared)
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in include/dcnv4_gfx950.h but not exported"
+    assert set(declared) == set(_lib.SIGNATURES), "ctypes table and header list different functions"
+
+
+def test_ctypes_signatures_have_the_arity_of_the_header():
+    from dcnv4_amd import _lib
+    for name, args in _declared_functions().items():
+        args = args.strip()
+        n = 0 if args in ("", "void") else len([a for a in args.split(",") if a.strip()])
+        assert n == len(_lib.SIGNATURES[name][1]), f"{name}: header has {n} parameters"
+
+
+def test_abi_version_and_error_string_work_without_a_gpu():
+    from dcnv4_amd import _lib
+    lib = _lib.load()
+    assert lib.dcnv4_gfx950_abi_version() == _lib.ABI_VERSION
+    # argument errors are detected before anything touches the device
+    rc = lib.dcnv4_gfx950_forward(None, None, None, 7, 1, 4, 4, 1, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1.0, 64, 0, 32, 0, 0, 0, None)
+    assert rc == _lib.ERR_RUNTIME and b"dtype" in lib.dcnv4_gfx950_last_error()
+    rc = lib.dcnv4_gfx950_forward(None, None, None, 1, 1, 4, 4, 1, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1.0, 64, 0, 32, 0, 5, 0, None)
+    assert rc == _lib.ERR_INVALID_ARGUMENT and b"d_stride" in lib.dcnv4_gfx950_last_error()
+    rc = lib.flash_deform_attn_gfx950_forward(None, None, None, None, None, 1, 1, 16, 1, 16, 6, 4, 16, 64, 0, 0, None)
+    assert rc == _lib.ERR_INVALID_ARGUMENT and b"points" in lib.dcnv4_gfx950_last_error()
+    assert lib.dcnv4_gfx950_backward_workspace_bytes(1, 64, 56, 56, 4, 16) == 256
+    assert lib.dcnv4_gfx950_backward_workspace_bytes(1, 2, 8, 8, 1, 128) == 2 * 8 * 8 * 128 * 4
+    assert lib.dcnv4_gfx950_backward_workspace_bytes(0, 2, 8, 8, 1, 128) == 0
+
+
+def test_cpu_tensors_are_refused_like_the_reference():
+    import dcnv4_amd
+    v, om = torch.zeros(1, 4, 4, 16), torch.zeros(1, 4, 4, 32)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        dcnv4_amd.DCNv4Function.apply(v, om, 3, 3, 1, 1, 1, 1, 1, 1, 1, 16, 1.0, 256, 0)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        dcnv4_amd.ext.flash_deform_attn_forward(torch.zeros(1, 16, 1, 16), torch.tensor([[4, 4]]), torch.tensor([0]),
+                                                torch.zeros(1, 3, 1, 12), 64, 4, 8, 128)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        dcnv4_amd.ext.dcnv4_forward(v.transpose(1, 2), om, 3, 3, 1, 1, 1, 1, 1, 1, 1, 16, 1.0, 256, 0, 8, 128, False)
+
+
+def test_reference_package_name_is_importable():
+    import DCNv4
+    from DCNv4 import ext                                   # noqa: F401
+    from DCNv4.functions import DCNv4Function, FlashDeformAttnFunction      # noqa: F401
+    from DCNv4.modules import DCNv4 as Mod
+    assert Mod is DCNv4.DCNv4
+
+
+@pytest.mark.parametrize("G,C,es", [(4, 16, 2), (4, 16, 4), (80, 16, 2), (7, 16, 2), (8, 32, 2), (8, 32, 4), (3, 6, 2), (1, 1, 4)])
+def test_launch_hints_are_well_formed(G, C, es):
+    from dcnv4_amd.functions import launch_spec as ls
+    for fn in (ls.findspec, ls.find_spec_bwd):
+        d_stride, n_thread = fn(64, 56, 56, G, C, es)
+        assert d_stride in (1, 2, 4, 8) and C % d_stride == 0 and d_stride * es <= 16
+        lanes = 1
+        while lanes < C // d_stride:
+            lanes *= 2
+        assert n_thread % (G * lanes) == 0 and n_thread >= G * lanes
+    assert ls.find_spec_bwd(64, 56, 56, G, C, es)[0] == 1      # scatter layout: one channel per lane
+
+
+def test_dcnv4_module_keeps_the_reference_parameter_schema():
+    from dcnv4_amd import DCNv4
+    m = DCNv4(channels=112, group=7, offset_scale=0.5, dw_kernel_size=3, center_feature_scale=True, output_bias=False)
+    sd = {k: tuple(v.shape) for k, v in m.state_dict().items()}
+    K = 7 * 9
+    assert sd == {
+        "center_feature_scale_proj_weight": (7, 112), "center_feature_scale_proj_bias": (7,),
+        "offset_mask_dw.weight": (112, 1, 3, 3), "offset_mask_dw.bias": (112,),
+        "offset_mask.weight": (int(math.ceil(K * 3 / 8) * 8), 112), "offset_mask.bias": (int(math.ceil(K * 3 / 8) * 8),),
+        "value_proj.weight": (112, 112), "value_proj.bias": (112,), "output_proj.weight": (112, 112),
+    }
+    assert m.offset_mask.weight.abs().sum() == 0 and m.offset_mask.bias.abs().sum() == 0
+    assert DCNv4(channels=64, group=4, remove_center=True).offset_mask.out_features == 96
+    assert "value_proj.weight" not in DCNv4(channels=64, group=4, without_pointwise=True).state_dict()
+    with pytest.raises(ValueError):
+        DCNv4(channels=65, group=4)
+
+
+def test_flash_deform_attn_module_keeps_the_reference_parameter_schema():
+    from dcnv4_amd import FlashDeformAttn
+    m = FlashDeformAttn(d_model=256, n_levels=4, n_heads=8, n_points=4)
+    sd = {k: tuple(v.shape) for k, v in m.state_dict().items()}
+    assert sd == {"sampling_offsets.weight": (256, 256), "sampling_offsets.bias": (256,),
+                  "attention_weights.weight": (128, 256), "attention_weights.bias": (128,),
+                  "value_proj.weight": (256, 256), "value_proj.bias": (256,),
+                  "output_proj.weight": (256, 256), "output_proj.bias": (256,)}
+    bias = m.sampling_offsets.bias.view(8, 4, 4, 2)
+    assert torch.allclose(bias[0, 0, :, 0], torch.tensor([1.0, 2.0, 3.0, 4.0])) and bias[0, 0, :, 1].abs().max() < 1e-6
+    assert m.im2col_step == 64
