@@ -122,7 +122,7 @@ constexpr int kTiledMaxGroupChannels = 64;
 
 bool tiled_grad_value(int D) { return D <= kTiledMaxGroupChannels; }
 
-// Tuning override for the reach of the tiled grad_value kernel (pixels); results never depend on it.
+// Tuning override for the cap on the reach of the tiled grad_value kernel (pixels).
 int reach_setting() {
   static const int v = [] {
     const char *e = getenv("DCNV4_GFX950_REACH");

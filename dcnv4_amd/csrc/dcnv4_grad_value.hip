@@ -8,8 +8,8 @@
 //
 //   * a workgroup OWNS a tile_h x tile_w tile of the input image for a chunk of groups, and is
 //     the only writer of that part of grad_value: plain stores, no clearing pass, no cast pass;
-//   * it visits every output pixel whose reference point lies within `reach` pixels of the tile,
-//     strip by strip, in two phases per strip:
+//   * it visits every output pixel whose reference point lies within the reach the data needs
+//     (GradState::reach_needed, capped by the planned `reach`), strip by strip, in two phases:
 //       A  tap-parallel: one lane per (pixel, group, kernel tap) recomputes the sampling position
 //          and, when a corner lands inside the tile, appends a hit record (four accumulator cells,
 //          four weights, pixel) to a per-group list in LDS; the strip's grad_out is parked in LDS;
@@ -87,10 +87,13 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   // output pixels this tile visits: reference point within `reach` of the tile (near_box)
   const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
   const int cy0 = half_h - p.ph, cx0 = half_w - p.pw, Ho = p.Q / p.Wo;
-  const int ho_lo = max(0, ceil_div_signed(ty0 - p.reach - cy0, p.sh));
-  const int ho_hi = min(Ho, ceil_div_signed(ty0 + p.tile_h + p.reach - cy0, p.sh));
-  const int wo_lo = max(0, ceil_div_signed(tx0 - p.reach - cx0, p.sw));
-  const int wo_hi = min(p.Wo, ceil_div_signed(tx0 + p.tile_w + p.reach - cx0, p.sw));
+  // every in-image corner lies within reach_needed of its reference point, so a smaller window than the
+  // planned cap loses nothing; beyond the cap the fallback kernel takes over
+  const int reach = min(p.reach, (int)p.state->reach_needed);
+  const int ho_lo = max(0, ceil_div_signed(ty0 - reach - cy0, p.sh));
+  const int ho_hi = min(Ho, ceil_div_signed(ty0 + p.tile_h + reach - cy0, p.sh));
+  const int wo_lo = max(0, ceil_div_signed(tx0 - reach - cx0, p.sw));
+  const int wo_hi = min(p.Wo, ceil_div_signed(tx0 + p.tile_w + reach - cx0, p.sw));
   const int nwx = wo_hi - wo_lo;
   const int lane = threadIdx.x & (kWave - 1), c = lane & (kRow - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);

@@ -139,7 +139,7 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 //   kBwdFull        grad_offset_mask, and grad_value scattered with fp32 buffer atomics into a
 //                   cleared fp32 image (any group width; the generic path)
 //   kBwdOffsetMask  grad_offset_mask only, plus the statistics the tiled grad_value kernel needs
-//                   (max |grad_out|, max |modulation|, "some corner is beyond the reach" flag)
+//                   (max |grad_out|, max |modulation|, the reach the scatter needs)
 //   kBwdFallback    no gradients of offsets; scatters into grad_value, in its own dtype, the
 //                   corners the tiled kernel does not cover: the far ones, or all of them when the
 //                   statistics are not finite.  Exits at once when there is nothing to do.
@@ -151,7 +151,7 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
   if constexpr (MODE == kBwdFallback) {
     const uint32_t gmax = p.state->go_max_bits, mmax = p.state->mask_max_bits;
     scatter_all = gmax >= 0x7f800000u || mmax >= 0x7f800000u;
-    if (!scatter_all && p.state->far_flag == 0) return;
+    if (!scatter_all && p.state->reach_needed <= (uint32_t)p.reach) return;
   }
   const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
   const int pix0 = (int)blk * p.npix_block;
@@ -172,7 +172,7 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
   const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
   const int Kp = p.Kp;
   const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
-  uint32_t go_max = 0, mask_max = 0, far = 0;
+  uint32_t go_max = 0, mask_max = 0, reach_needed = 0;
 
   for (int it = threadIdx.x; it < items; it += blockDim.x) {
     const int chunk = it & (width - 1);
@@ -186,11 +186,14 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
     float mx = 0.f, inv = 1.f;
     if (p.softmax) softmax_stats(om + 2 * Kp, Kp, mx, inv);
     // reference point of this output pixel (centre tap, zero offset), for the reach rule
+    // reference point of this output pixel (centre tap at zero offset) and the box the tiled scatter covers
     NearBox box = {0, 0, 0, 0};
+    int p0y = 0, p0x = 0;
     if constexpr (MODE != kBwdFull) {
       const int q = pix % p.Q;
-      box = near_box(half_h - p.ph + (q / p.Wo) * p.sh, half_w - p.pw + (q % p.Wo) * p.sw, p.tile_h_log2,
-                     p.tile_w_log2, p.reach);
+      p0y = half_h - p.ph + (q / p.Wo) * p.sh;
+      p0x = half_w - p.pw + (q % p.Wo) * p.sw;
+      box = near_box(p0y, p0x, p.tile_h_log2, p.tile_w_log2, p.reach);
     }
     const size_t img_elem0 = (size_t)(pix / p.Q) * (size_t)(p.H * p.W) * (size_t)(p.G * p.D);
 
@@ -236,9 +239,11 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
       }
       if constexpr (MODE == kBwdOffsetMask) {
         mask_max = max(mask_max, __builtin_bit_cast(uint32_t, fabsf(m)));
-#pragma unroll
-        for (int cn = 0; cn < 4; ++cn)
-          if ((t.valid & (1u << cn)) && !corner_is_near(box, t.y0 + (cn >> 1), t.x0 + (cn & 1))) far = 1;
+        if (t.valid != 0) {     // distance of the in-image part of the 2x2 corner block from the reference point
+          const int d = max(max(p0y - max(t.y0, 0), min(t.y0 + 1, p.H - 1) - p0y),
+                            max(p0x - max(t.x0, 0), min(t.x0 + 1, p.W - 1) - p0x));
+          reach_needed = max(reach_needed, (uint32_t)max(d, 0));
+        }
       }
       typename pack::raw_t raw[4];
 #pragma unroll
@@ -310,11 +315,11 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
     __syncthreads();
     go_max = wave_max_u32(go_max);
     mask_max = wave_max_u32(mask_max);
-    far = wave_max_u32(far);
+    reach_needed = wave_max_u32(reach_needed);
     if ((threadIdx.x & (kWave - 1)) == 0) {
       atomicMax(&s_stat[0], go_max);
       atomicMax(&s_stat[1], mask_max);
-      atomicMax(&s_stat[2], far);
+      atomicMax(&s_stat[2], reach_needed);
     }
     __syncthreads();
     if (threadIdx.x < 3) {

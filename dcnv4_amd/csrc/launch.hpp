@@ -19,7 +19,7 @@ constexpr size_t kMaxLdsPerWorkgroup = 160 * 1024;  // gfx950
 struct GradState {
   uint32_t go_max_bits;    // max |grad_out| as IEEE bits (ordered like unsigned ints for x >= 0; NaN sorts last)
   uint32_t mask_max_bits;  // max |modulation| (after softmax when enabled)
-  uint32_t far_flag;       // some in-image corner lies outside the reach the tiled scatter covers
+  uint32_t reach_needed;   // largest Chebyshev distance (pixels) of an in-image corner from its output pixel's reference point
   uint32_t reserved;
 };
 
@@ -57,7 +57,7 @@ struct DcnLaunch {
   int n_img;
   int tile_h, tile_w;       // input-space tile one workgroup owns (powers of two)
   int tile_h_log2, tile_w_log2;
-  int reach;                // corners up to `reach` pixels outside the tile of their output pixel are covered
+  int reach;                // cap on the reach the tiled scatter covers; it uses min(reach, GradState::reach_needed)
   int ng_chunk;             // groups per workgroup (channel chunk = ng_chunk * D)
   int strip_pix;            // output pixels staged per strip
   int fix_bits;             // fractional bits of the 64-bit fixed-point accumulators
