@@ -133,7 +133,7 @@ int reach_setting() {
 }
 
 // Tile, channel chunk and strip of the tiled grad_value kernel such that its LDS footprint fits.
-int plan_grad_value_tiles(DcnLaunch *L) {
+int plan_grad_value_tiles(DcnLaunch *L, int elem_bytes_of_launch) {
   const int D = L->D;
   L->reach = reach_setting();
   L->ng_chunk = std::max(1, std::min(L->G, kTiledMaxGroupChannels / std::max(D, 16)));   // <= 4
@@ -159,6 +159,10 @@ int plan_grad_value_tiles(DcnLaunch *L) {
   }
   const long long contributions = (long long)visited(L->tile_h, L->sh) * visited(L->tile_w, L->sw) * L->Kp;
   L->fix_bits = 62 - ceil_log2((int)std::min<long long>(contributions, 1 << 30));
+  if (elem_bytes_of_launch == 2) L->fix_bits = std::min(L->fix_bits, 30);   // 32-bit conversion path for 16-bit tensors
+  // the tiled kernel addresses one image's offset_mask and grad_out with 32-bit element offsets
+  if (L->Q >= (1 << 24) || (uint64_t)L->Q * (uint64_t)L->P_pad >= (1ull << 31) || (uint64_t)L->Q * (uint64_t)(L->G * L->D) >= (1ull << 31))
+    return fail(DCNV4_ERR_RUNTIME, "one image of %d output pixels is too large for the tiled backward", L->Q);
   return DCNV4_OK;
 }
 
@@ -379,7 +383,7 @@ int dcnv4_gfx950_backward(const void *value, const void *offset_mask, const void
     // 1. grad_offset_mask + statistics  2. tiled grad_value (plain stores)  3. fallback scatter
     //    for corners beyond the reach / non-finite statistics (returns at once otherwise)
     DcnLaunch base = pr.launch;
-    if (int rc = plan_grad_value_tiles(&base)) return rc;
+    if (int rc = plan_grad_value_tiles(&base, pr.s)) return rc;
     base.state = static_cast<GradState *>(workspace);
     hipLaunchKernelGGL(init_state_kernel, dim3(1), dim3(64), 0, st, base.state);
     if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);

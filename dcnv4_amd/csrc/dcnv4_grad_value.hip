@@ -38,12 +38,20 @@ constexpr int kTrashPad = 64;
 constexpr int kMaxChunkGroups = 4;      // rows of a wave <-> groups of the chunk
 constexpr int kCellBits = 9;            // cell index 0..n_cells (n_cells = trash), tiles up to 16x16
 
-// float (|t| < 2^62) -> two's-complement 64-bit integer, exact (t carries 24 significant bits).
-__device__ __forceinline__ unsigned long long to_fixed(float t) {
-  const float th = floorf(t * 0x1p-32f);
-  const int hi = (int)th;
-  const uint32_t lo = (uint32_t)fmaf(th, -0x1p32f, t);
-  return ((unsigned long long)(uint32_t)hi << 32) | lo;
+// float -> two's-complement 64-bit integer.
+// WIDE: |t| < 2^62, exact (t carries 24 significant bits), six instructions.
+// !WIDE: |t| < 2^31, truncated toward zero, three instructions; used for 16-bit tensors, whose values
+// carry 8-11 significant bits (fix_bits is then 30: 2^-30 of the largest possible contribution).
+template <bool WIDE> __device__ __forceinline__ unsigned long long to_fixed(float t) {
+  if constexpr (WIDE) {
+    const float th = floorf(t * 0x1p-32f);
+    const int hi = (int)th;
+    const uint32_t lo = (uint32_t)fmaf(th, -0x1p32f, t);
+    return ((unsigned long long)(uint32_t)hi << 32) | lo;
+  } else {
+    const int v = (int)t;
+    return ((unsigned long long)(uint32_t)(v >> 31) << 32) | (uint32_t)v;
+  }
 }
 
 struct HitMeta {
@@ -106,49 +114,71 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
 
   if (finite && nwx > 0 && ho_hi > ho_lo && (gmax | mmax) != 0) {
     const int rows_per_strip = max(1, p.strip_pix / nwx);
+    const int npx_full = rows_per_strip * nwx;
     const float inv_nwx = 1.f / (float)nwx;
+    // this image's tensors, addressed with 32-bit element offsets (the entry point checks they fit)
+    const elem_t *om_img = om_g + (size_t)b * p.Q * p.P_pad;
+    const elem_t *go_img = go_g + (size_t)b * p.Q * C;
     constexpr int kStageRounds = 2;     // pixels per wave whose grad_out is prefetched (16 waves: 32 pixels)
-    constexpr int kStageChunks = 1;     // 64-channel chunks of a pixel that are prefetched
-    struct Prefetch {
-      elem_t ox, oy, m;                               // phase A, first round: this lane's tap
-      elem_t go[kStageRounds][kStageChunks];          // staging: this lane's channel of up to two pixels
-    };
 
-    // phase A work item of (round, wave, lane): group, pixel, tap; valid == false past the end
-    struct Item { int gl, px, t, ho, wo; bool valid; const elem_t *om; };
-    auto item_of = [&](int wk, int hs, int npx) {
+    // Phase A work item of a (wave slot, lane): group, strip-local pixel, tap.  The decode depends only
+    // on the strip geometry, not on the strip, so the first round's item is decoded once per lane.
+    struct Item {
+      bool in_range;
+      int gl, px, r, t, ti, tj;
+      uint32_t om_off;       // element offset of this (pixel, group)'s offset_mask slice for the first strip
+      float x_base;
+    };
+    const int per_group_full = npx_full * Kp, waves_per_group = (per_group_full + kWave - 1) / kWave;
+    const int n_wk = ng * waves_per_group;
+    auto item_of = [&](int wk) {
       Item it;
-      const int per_group = npx * Kp, waves_per_group = (per_group + kWave - 1) / kWave;
       it.gl = wk / waves_per_group;                                          // scalar: same for the wave
       const int j = (wk - it.gl * waves_per_group) * kWave + lane;
-      it.valid = it.gl < ng && j < per_group;
+      it.in_range = wk < n_wk && j < per_group_full;
       it.px = KP > 0 ? j / KP : j / Kp;
       it.t = j - it.px * Kp;
-      if (!it.valid) { it.gl = 0; it.px = 0; it.t = 0; }
-      const int r = (int)(((float)it.px + 0.5f) * inv_nwx);                  // exact: px < 1024
-      it.ho = hs + r; it.wo = wo_lo + (it.px - r * nwx);
-      it.om = om_g + ((size_t)b * p.Q + (size_t)it.ho * p.Wo + it.wo) * p.P_pad + (g0 + it.gl) * 3 * Kp;
+      if (!it.in_range) { it.gl = 0; it.px = 0; it.t = 0; }
+      it.r = (int)(((float)it.px + 0.5f) * inv_nwx);                         // exact: px < 1024
+      const int wo = wo_lo + (it.px - it.r * nwx);
+      if constexpr (KP > 0) {
+        tap_ij_3x3(KP, it.t, it.ti, it.tj);
+      } else {      // x index outer, y index inner, centre skipped when remove_center
+        int tt = it.t;
+        if (p.remove_center && tt >= (p.kw / 2) * p.kh + p.kh / 2) ++tt;
+        it.ti = tt / p.kh; it.tj = tt - it.ti * p.kh;
+      }
+      it.om_off = __umul24((uint32_t)((ho_lo + it.r) * p.Wo + wo), (uint32_t)p.P_pad) + (uint32_t)((g0 + it.gl) * 3 * Kp);
+      it.x_base = sub_rn((float)(cx0 + wo * p.sw), x_sub);
       return it;
     };
-    auto go_row = [&](int px, int hs) {
-      const int r = px / nwx, wx = px - r * nwx;
-      return go_g + ((size_t)b * p.Q + (size_t)(hs + r) * p.Wo + wo_lo + wx) * C + g0 * D;
+    const Item my_item = item_of(wave);
+    // staging: wave w parks pixel w (+16, ...) of the strip, lane = channel of the chunk
+    uint32_t go_off[kStageRounds];
+#pragma unroll
+    for (int u = 0; u < kStageRounds; ++u) {
+      const int px = wave + u * kWaves, r = px / nwx;
+      go_off[u] = (uint32_t)(((ho_lo + r) * p.Wo + wo_lo + (px - r * nwx)) * C + g0 * D + lane);
+    }
+    const uint32_t om_strip = (uint32_t)(rows_per_strip * p.Wo) * (uint32_t)p.P_pad;   // offset step per strip
+    const uint32_t go_strip = (uint32_t)(rows_per_strip * p.Wo * C);
+
+    struct Prefetch {
+      elem_t ox, oy, m;                 // phase A, first round: this lane's tap
+      elem_t go[kStageRounds];          // staging: this lane's channel of up to two pixels
     };
     // loads of the next strip, issued before the current strip's phase B so their latency hides there
-    auto prefetch = [&](int hs, int npx) {
+    auto prefetch = [&](int s_idx, int npx) {
       Prefetch pf;
-      const Item it = item_of(wave, hs, npx);
       pf.ox = pf.oy = pf.m = elem_t(0);
-      if (it.valid) { pf.ox = it.om[2 * it.t]; pf.oy = it.om[2 * it.t + 1]; pf.m = it.om[2 * Kp + it.t]; }
+      if (my_item.in_range && my_item.px < npx) {
+        const elem_t *om = om_img + (my_item.om_off + (uint32_t)s_idx * om_strip);
+        pf.ox = om[2 * my_item.t]; pf.oy = om[2 * my_item.t + 1]; pf.m = om[2 * Kp + my_item.t];
+      }
 #pragma unroll
       for (int u = 0; u < kStageRounds; ++u) {
-        const int px = wave + u * kWaves;
-#pragma unroll
-        for (int v = 0; v < kStageChunks; ++v) {
-          const int ch = lane + v * kWave;
-          pf.go[u][v] = elem_t(0);
-          if (px < npx && ch < ng * D) pf.go[u][v] = go_row(px, hs)[ch];
-        }
+        pf.go[u] = elem_t(0);
+        if (wave + u * kWaves < npx && lane < ng * D) pf.go[u] = go_img[go_off[u] + (uint32_t)s_idx * go_strip];
       }
       return pf;
     };
@@ -156,7 +186,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
 
     int hs = ho_lo;
     int npx = min(rows_per_strip, ho_hi - hs) * nwx;
-    Prefetch pf = prefetch(hs, npx);
+    Prefetch pf = prefetch(0, npx);
     if (threadIdx.x < 2 * kMaxChunkGroups) s_count[threadIdx.x] = 0u;
 
     for (int s_idx = 0; hs < ho_hi; ++s_idx) {
@@ -165,34 +195,32 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
 
       // ---- park the strip's grad_out (this chunk's channels), normalised to [-1, 1]: a wave per pixel
       for (int px = wave, u = 0; px < npx; px += kWaves, ++u)
-        for (int ch = lane, v = 0; ch < ch_stride; ch += kWave, ++v) {
+        for (int ch = lane; ch < ch_stride; ch += kWave) {
           float g = 0.f;
-          if (ch < ng * D) g = (u < kStageRounds && v < kStageChunks) ? to_f(u == 0 ? pf.go[0][0] : pf.go[kStageRounds - 1][0])
-                                                                     : load_f(go_row(px, hs) + ch);
+          if (ch < ng * D) {
+            if (u < kStageRounds && ch < kWave) g = to_f(u == 0 ? pf.go[0] : pf.go[kStageRounds - 1]);
+            else {
+              const int r = px / nwx;
+              g = load_f(go_img + ((size_t)((hs + r) * p.Wo + wo_lo + (px - r * nwx)) * C + g0 * D + ch));
+            }
+          }
           s_go[px * ch_stride + ch] = ldexpf(g, -e_go);
         }
 
       // ---- phase A: one lane per (group, pixel, tap); a wave never mixes groups
-      const int n_wk = ng * ((npx * Kp + kWave - 1) / kWave);
       for (int wk = wave, round = 0; wk < n_wk; wk += kWaves, ++round) {
-        const Item it = item_of(wk, hs, npx);
+        const Item it = round == 0 ? my_item : item_of(wk);
+        const bool valid_item = it.in_range && it.px < npx;
         bool hit = false;
         f32x4 w = {0.f, 0.f, 0.f, 0.f};
         HitMeta meta = {0u, 0u};
-        if (it.valid) {
-          const float off_x = round == 0 ? to_f(pf.ox) : load_f(it.om + 2 * it.t);
-          const float off_y = round == 0 ? to_f(pf.oy) : load_f(it.om + 2 * it.t + 1);
-          int ti, tj;
-          if constexpr (KP > 0) {
-            tap_ij_3x3(KP, it.t, ti, tj);
-          } else {      // x index outer, y index inner, centre skipped when remove_center
-            int tt = it.t;
-            if (p.remove_center && tt >= (p.kw / 2) * p.kh + p.kh / 2) ++tt;
-            ti = tt / p.kh; tj = tt - ti * p.kh;
-          }
-          const float x_base = sub_rn((float)(cx0 + it.wo * p.sw), x_sub), y_base = sub_rn((float)(cy0 + it.ho * p.sh), y_sub);
-          const float x = add_rn(x_base, mul_rn(add_rn((float)(ti * p.dw), off_x), p.offset_scale));
-          const float y = add_rn(y_base, mul_rn(add_rn((float)(tj * p.dh), off_y), p.offset_scale));
+        if (valid_item) {
+          const elem_t *om = om_img + (it.om_off + (uint32_t)s_idx * om_strip);
+          const float off_x = round == 0 ? to_f(pf.ox) : load_f(om + 2 * it.t);
+          const float off_y = round == 0 ? to_f(pf.oy) : load_f(om + 2 * it.t + 1);
+          const float y_base = sub_rn((float)(cy0 + (hs + it.r) * p.sh), y_sub);
+          const float x = add_rn(it.x_base, mul_rn(add_rn((float)(it.ti * p.dw), off_x), p.offset_scale));
+          const float y = add_rn(y_base, mul_rn(add_rn((float)(it.tj * p.dh), off_y), p.offset_scale));
           const Tap tp = make_tap(y, x, p.H, p.W, 0u, 0u);
           const int ly = tp.y0 - ty0, lx = tp.x0 - tx0;
           const bool r0 = ly >= 0 && ly < th, r1 = ly + 1 >= 0 && ly + 1 < th;
@@ -201,11 +229,11 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
                                              ((uint32_t)(r1 && c0) << 2) | ((uint32_t)(r1 && c1) << 3));
           hit = valid != 0;
           if (hit) {
-            float m = round == 0 ? to_f(pf.m) : load_f(it.om + 2 * Kp + it.t);
+            float m = round == 0 ? to_f(pf.m) : load_f(om + 2 * Kp + it.t);
             if (p.softmax) {          // rare: normalise over this group's taps
-              float mx = load_f(it.om + 2 * Kp), sum = 0.f;
-              for (int k = 1; k < Kp; ++k) mx = fmaxf(mx, load_f(it.om + 2 * Kp + k));
-              for (int k = 0; k < Kp; ++k) sum += __expf(load_f(it.om + 2 * Kp + k) - mx);
+              float mx = load_f(om + 2 * Kp), sum = 0.f;
+              for (int k = 1; k < Kp; ++k) mx = fmaxf(mx, load_f(om + 2 * Kp + k));
+              for (int k = 0; k < Kp; ++k) sum += __expf(load_f(om + 2 * Kp + k) - mx);
               m = __expf(m - mx) / sum;
             }
             const float ms = ldexpf(m, p.fix_bits - e_m);
@@ -221,7 +249,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
             meta.cell3_px = cells[3] | ((uint32_t)it.px << kCellBits);
           }
         }
-        // append the wave's hits to its group's list: one LDS counter bump per wave
+      // append the wave's hits to its group's list: one LDS counter bump per wave
         const uint64_t mask = __builtin_amdgcn_ballot_w64(hit);
         if (mask != 0) {
           uint32_t base = 0;
@@ -240,7 +268,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       // next strip's loads fly while this strip's hits are applied; the other counter set is idle
       const int hs_next = hs + rows_per_strip;
       const int npx_next = hs_next < ho_hi ? min(rows_per_strip, ho_hi - hs_next) * nwx : 0;
-      if (npx_next > 0) pf = prefetch(hs_next, npx_next);
+      if (npx_next > 0) pf = prefetch(s_idx + 1, npx_next);
       if (threadIdx.x < kMaxChunkGroups) s_count[((s_idx + 1) & 1) * kMaxChunkGroups + threadIdx.x] = 0u;
 
       // ---- phase B: row r of each wave drains list r, 16 lanes = 16 channels (x CPL)
@@ -270,7 +298,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
           unsigned long long *dst = acc_lane + __umul24(cells[cn], (uint32_t)ch_stride);
 #pragma unroll
           for (int j = 0; j < CPL; ++j)
-            __hip_atomic_fetch_add(dst + kRow * j, to_fixed(gn[j] * wv[cn]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            __hip_atomic_fetch_add(dst + kRow * j, to_fixed<Tag::kBytes == 4>(gn[j] * wv[cn]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
       }
       hs = hs_next;
