@@ -10,7 +10,9 @@ divided by the step time, inputs resident in HBM.  Per-operator timings (HIP eve
 stream the kernels run on) for these shapes, the dense-prediction shapes and the
 Deformable-DETR attention shape are reported under "detail"; "roofline" describes the operator
 that takes the largest share of the step; "cpu_baseline" times the pure-PyTorch grid_sample
-formulation of the same operator (oracle/torch_core.py) on the host cores on a reduced batch.
+formulation of the same operator (oracle/torch_core.py) on the host cores on a reduced batch;
+"flash_intern_image_b" is the end-to-end classification forward (batch 128, fp16) with the share of
+its time spent inside the DCNv4 operator.
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W]
 """
@@ -58,6 +60,7 @@ def main():
     ap.add_argument("--op-iters", type=int, default=100, help="timed launches per operator in the detail table")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-detail", action="store_true", help="skip per-operator timings other than the step's own")
+    ap.add_argument("--no-model", action="store_true", help="skip the FlashInternImage-B end-to-end forward")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this operator has no cross-GPU communication and every box here "
@@ -159,6 +162,50 @@ def main():
                 time_op(lambda: ext.flash_deform_attn_backward(v, shapes, starts, sla, go, 64, K, 0, 0), args.op_iters), bb)
             del v, sla, go
 
+    # ------------------------------------------------------------------ FlashInternImage-B end to end (configs[4])
+    model_line = None
+    if not args.no_model:
+        from dcnv4_amd.models import flash_intern_image
+        model = flash_intern_image("b").to(dev).half().eval()
+        images = torch.randn(128, 3, 224, 224, device=dev).half()
+        spans = []                                    # (start, end) events around every DCNv4 operator call
+        real_forward = ext.dcnv4_forward
+
+        def timed_forward(*a):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            out = real_forward(*a)
+            e1.record()
+            spans.append((e0, e1))
+            return out
+
+        with torch.no_grad():
+            for _ in range(50):                       # protocol of the reference's throughput(): 50 warm-up, 30 timed
+                model(images)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(30):
+                model(images)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            ext.dcnv4_forward = timed_forward
+            try:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(5):
+                    model(images)
+                e1.record()
+                torch.cuda.synchronize()
+            finally:
+                ext.dcnv4_forward = real_forward
+            op_ms = sum(a.elapsed_time(b) for a, b in spans)
+            total_ms = e0.elapsed_time(e1)
+        model_line = {"model": "FlashInternImage-B, random init, eval forward, fp16, batch 128, 224x224, synthetic input",
+                      "img_per_s": round(30 * 128 / dt, 1), "ms_per_batch": round(dt / 30 * 1e3, 3),
+                      "dcnv4_calls_per_forward": len(spans) // 5,
+                      "dcnv4_kernel_share": round(op_ms / total_ms, 4)}
+        del model, images
+
     # ------------------------------------------------------------------ roofline of the dominant operator
     dom = max(step_ops, key=lambda d: d["ms"])
     dom_bytes = dom["MB"] * 1e6
@@ -167,7 +214,7 @@ def main():
         "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4), "traffic": None,
         "kernel": f'{dom["op"]} {dom["shape"]} {dom["dtype"]}', "ms": dom["ms"],
         "algorithmic_bytes": int(dom_bytes),
-        "note": "HIP events around whole operator calls (for backward: clear + scatter kernel + cast)",
+        "note": "HIP events around whole operator calls (backward = state reset + grad_offset_mask kernel + tiled grad_value kernel + fallback)",
     }
 
     # ------------------------------------------------------------------ CPU baseline (rank 0, bounded sample)
@@ -205,7 +252,7 @@ def main():
         "config": {"workload": "DCNv4 forward+backward, FlashInternImage-T stages (56x56 C64 G4, 28x28 C128 G8, "
                                "14x14 C256 G16, 7x7 C512 G32), batch 64, 3x3 s1 p1, fp16 and fp32 tensors, fp32 arithmetic",
                    "step_algorithmic_MB": round(step_bytes / 1e6, 1), "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2)},
-        "roofline": roofline, "cpu_baseline": cpu, "detail": detail,
+        "roofline": roofline, "cpu_baseline": cpu, "flash_intern_image_b": model_line, "detail": detail,
     }
     print(json.dumps(line))
 

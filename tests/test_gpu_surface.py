@@ -240,3 +240,36 @@ def test_forward_and_backward_replay_correctly_from_a_hip_graph():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(g_out, eager_out) and torch.equal(g_gv, eager_gv) and torch.equal(g_gom, eager_gom)
+
+
+def test_small_flash_intern_image_matches_the_same_network_on_the_torch_core(monkeypatch):
+    """A two-level FlashInternImage (DCNv4 layers on the HIP kernels) against the same weights evaluated on the
+    CPU with the operator swapped for the grid_sample formulation."""
+    from dcnv4_amd.models import FlashInternImage
+    from dcnv4_amd.modules import dcnv4 as dcnv4_module
+
+    torch.manual_seed(2)
+    kw = dict(channels=32, depths=(2, 2), groups=(2, 4), offset_scale=1.0, drop_path_rate=0.0, layer_scale=1e-1,
+              post_norm=True, dw_kernel_size=3, num_classes=10)
+    model = FlashInternImage(**kw).eval()
+    with torch.no_grad():
+        for m in model.modules():
+            if isinstance(m, dcnv4_module.DCNv4):
+                m.offset_mask.weight.normal_(0, 0.2)
+                m.offset_mask.bias.normal_(0, 0.5)
+    x = torch.randn(2, 3, 64, 64)
+
+    class CoreOnCpu:
+        @staticmethod
+        def apply(inp, om, kh, kw_, sh, sw, ph, pw, dh, dw, group, group_channels, offset_scale, im2col_step, remove_center):
+            return torch_core.dcnv4_core_torch(inp, om, kh, kw_, sh, sw, ph, pw, dh, dw, group, group_channels,
+                                               offset_scale, remove_center)
+
+    with torch.no_grad():
+        got = model.cuda()(x.cuda()).cpu()
+        feats = [f.cpu() for f in model.forward_features_seq_out(x.cuda())]
+        model.cpu()
+        monkeypatch.setattr(dcnv4_module, "DCNv4Function", CoreOnCpu)
+        want = model(x)
+    assert got.shape == (2, 10) and [tuple(f.shape) for f in feats] == [(2, 32, 16, 16), (2, 64, 8, 8)]
+    assert _rel_err(got, want) < 1e-3

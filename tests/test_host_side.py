@@ -116,3 +116,28 @@ def test_flash_deform_attn_module_keeps_the_reference_parameter_schema():
     bias = m.sampling_offsets.bias.view(8, 4, 4, 2)
     assert torch.allclose(bias[0, 0, :, 0], torch.tensor([1.0, 2.0, 3.0, 4.0])) and bias[0, 0, :, 1].abs().max() < 1e-6
     assert m.im2col_step == 64
+
+
+@pytest.mark.parametrize("variant,millions", [("t", 30), ("s", 50), ("b", 97), ("l", 223)])
+def test_flash_intern_image_parameter_counts_match_the_published_model_sizes(variant, millions):
+    # README.md:29-32 of the reference lists 30M / 50M / 97M / 223M parameters for T / S / B / L
+    from dcnv4_amd.models import flash_intern_image
+    m = flash_intern_image(variant)
+    n = sum(p.numel() for p in m.parameters())
+    assert abs(n / 1e6 - millions) < 0.6, n
+
+
+def test_flash_intern_image_state_dict_uses_the_reference_key_names():
+    from dcnv4_amd.models import flash_intern_image
+    keys = set(flash_intern_image("b").state_dict())
+    for k in ["patch_embed.conv1.weight", "patch_embed.norm1.0.running_mean", "patch_embed.norm2.0.weight",
+              "levels.0.blocks.0.gamma1", "levels.0.blocks.0.norm1.0.weight", "levels.0.blocks.0.dcn.offset_mask_dw.weight",
+              "levels.0.blocks.0.dcn.offset_mask.weight", "levels.0.blocks.0.dcn.value_proj.bias",
+              "levels.0.blocks.0.dcn.output_proj.weight", "levels.0.blocks.0.mlp.fc1.bias", "levels.0.blocks.0.mlp.fc2.weight",
+              "levels.0.downsample.conv.weight", "levels.0.downsample.norm.1.weight", "levels.2.blocks.20.norm2.0.bias",
+              "conv_head.0.weight", "conv_head.1.0.running_var", "head.weight", "head.bias"]:
+        assert k in keys, k
+    assert "levels.0.blocks.0.dcn.output_proj.bias" not in keys          # dcn_output_bias is False for B
+    assert "levels.3.downsample.conv.weight" not in keys and "levels.0.norm.0.weight" not in keys   # post_norm variant
+    t_keys = set(flash_intern_image("t").state_dict())
+    assert "levels.0.norm.0.weight" in t_keys and "levels.0.blocks.0.gamma1" not in t_keys
