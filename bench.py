@@ -61,6 +61,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-detail", action="store_true", help="skip per-operator timings other than the step's own")
     ap.add_argument("--no-model", action="store_true", help="skip the FlashInternImage-B end-to-end forward")
+    ap.add_argument("--only-op", default=None, metavar="OP:SHAPE:DTYPE",
+                    help="profiling aid: run just one operator of the step --steps times and exit, e.g. "
+                         "dcnv4_bwd:T-stage1:float32 (prints its HIP-event time); also copy:MB for a plain device copy")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this operator has no cross-GPU communication and every box here "
@@ -102,11 +105,32 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / iters      # ms per call
 
+    if args.only_op and args.only_op.startswith("copy:"):
+        # plain copy of known size: calibrates FETCH_SIZE / WRITE_SIZE counters and shows the HBM ceiling
+        n = int(float(args.only_op.split(":")[1]) * 1e6) // 4
+        src, dst = torch.randn(n, device=dev), torch.empty(n, device=dev)
+        ms = time_op(lambda: dst.copy_(src), args.steps, warm=args.warmup)
+        print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "read_MB": n * 4 / 1e6, "write_MB": n * 4 / 1e6,
+                          "GBps_read_plus_write": round(2 * n * 4 / (ms * 1e-3) / 1e9, 1)}))
+        return
+
     # ------------------------------------------------------------------ the step (configs[1])
     work = []
     for dtype, s in ((torch.float16, 2), (torch.float32, 4)):
         for name, B, H, W, C, G in CFG2:
             work.append((name, dtype, s, (B, H, W, C, G), dcn_inputs(B, H, W, C, G, dtype, 3.0)))
+
+    if args.only_op:
+        op, shape_name, dt_name = args.only_op.split(":")
+        for name, dtype, s, (B, H, W, C, G), t in work:
+            if name == shape_name and str(dtype) == "torch." + dt_name:
+                fn = (lambda: dcn_fwd(t, G, C)) if op == "dcnv4_fwd" else (lambda: dcn_bwd(t, G, C))
+                ms = time_op(fn, args.steps, warm=args.warmup)
+                nbytes = dcn_bytes(s, B, H, W, C, G)[0 if op == "dcnv4_fwd" else 1]
+                print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "algorithmic_MB": round(nbytes / 1e6, 2),
+                                  "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)}))
+                return
+        sys.exit(f"--only-op {args.only_op}: no such operator in the step")
 
     def step():
         for _, _, _, (B, H, W, C, G), t in work:

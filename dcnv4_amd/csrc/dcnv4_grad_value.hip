@@ -32,7 +32,7 @@ namespace dcn {
 namespace {
 
 constexpr int kValThreads = 1024;
-constexpr int kRow = 16;
+constexpr int kRow = 8;               // lanes that apply one hit record
 constexpr int kWaves = kValThreads / kWave;
 constexpr int kTrashPad = 64;
 constexpr int kMaxChunkGroups = 4;      // rows of a wave <-> groups of the chunk
@@ -104,6 +104,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   const int wo_hi = min(p.Wo, ceil_div_signed(tx0 + p.tile_w + reach - cx0, p.sw));
   const int nwx = wo_hi - wo_lo;
   const int lane = threadIdx.x & (kWave - 1), c = lane & (kRow - 1);
+  static_assert(kWave / kRow == 2 * kMaxChunkGroups, "a wave holds two rows per group of a full chunk");
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int row_in_wave = lane / kRow;
   const float x_sub = mul_rn((float)half_w, p.offset_scale), y_sub = mul_rn((float)half_h, p.offset_scale);
@@ -271,25 +272,37 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       if (npx_next > 0) pf = prefetch(s_idx + 1, npx_next);
       if (threadIdx.x < kMaxChunkGroups) s_count[((s_idx + 1) & 1) * kMaxChunkGroups + threadIdx.x] = 0u;
 
-      // ---- phase B: row r of each wave drains list r, 16 lanes = 16 channels (x CPL)
-      const uint32_t n_mine = row_in_wave < ng ? count[row_in_wave] : 0u;
+      // ---- phase B: a row of 8 lanes applies one hit record; lane c owns channels c, c+8, ... (CPL of them).
+      // The 8 rows of a wave are split evenly over the chunk's groups (two rows per group for a full
+      // chunk); the second row of a group walks its channels in the opposite order, so with 16 channels
+      // per group every ds_add_u64 instruction of the wave touches 64 distinct channels.
+      const int rows_per_group = (kWave / kRow) / p.ng_chunk;            // 2, 4 or 8
+      const int my_group = row_in_wave / rows_per_group, my_slot = row_in_wave - my_group * rows_per_group;
+      const bool group_live = my_group < ng;
+      const uint32_t n_mine = group_live ? count[my_group] : 0u;
       uint32_t n_max = count[0];
       for (int g = 1; g < ng; ++g) n_max = max(n_max, count[g]);
-      const int my_group = row_in_wave < ng ? row_in_wave : 0;      // idle rows only ever add zeros to the trash slots
-      unsigned long long *acc_lane = acc + my_group * D + c;
-      const float *go_lane = s_go + my_group * D + c;
-      for (uint32_t i = wave; i < n_max; i += kWaves) {
+      const int lane_group = group_live ? my_group : 0;                  // idle rows only ever add zeros to the trash slots
+      const bool flip = (my_slot & 1) != 0;
+      unsigned long long *acc_lane = acc + lane_group * D + c;
+      const float *go_lane = s_go + lane_group * D + c;
+      for (uint32_t i0 = wave * rows_per_group; i0 < n_max; i0 += kWaves * rows_per_group) {
+        const uint32_t i = i0 + my_slot;
         f32x4 w = {0.f, 0.f, 0.f, 0.f};
         HitMeta meta = {(uint32_t)n_cells | ((uint32_t)n_cells << kCellBits) | ((uint32_t)n_cells << (2 * kCellBits)),
                         (uint32_t)n_cells};
         if (i < n_mine) {
-          w = hit_w[row_in_wave * list_cap + i];
-          meta = hit_meta[row_in_wave * list_cap + i];
+          w = hit_w[lane_group * list_cap + i];
+          meta = hit_meta[lane_group * list_cap + i];
         }
         const int px = meta.cell3_px >> kCellBits;
         float gn[CPL];
+        int ch_off[CPL];
 #pragma unroll
-        for (int j = 0; j < CPL; ++j) gn[j] = (c + kRow * j < D) ? go_lane[px * ch_stride + kRow * j] : 0.f;
+        for (int j = 0; j < CPL; ++j) {
+          ch_off[j] = kRow * (flip ? CPL - 1 - j : j);
+          gn[j] = (c + ch_off[j] < D) ? go_lane[px * ch_stride + ch_off[j]] : 0.f;
+        }
         const uint32_t cells[4] = {meta.cells012 & 511u, (meta.cells012 >> kCellBits) & 511u,
                                    (meta.cells012 >> (2 * kCellBits)) & 511u, meta.cell3_px & 511u};
         const float wv[4] = {w.x, w.y, w.z, w.w};
@@ -298,7 +311,8 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
           unsigned long long *dst = acc_lane + __umul24(cells[cn], (uint32_t)ch_stride);
 #pragma unroll
           for (int j = 0; j < CPL; ++j)
-            __hip_atomic_fetch_add(dst + kRow * j, to_fixed<Tag::kBytes == 4>(gn[j] * wv[cn]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            __hip_atomic_fetch_add(dst + ch_off[j], to_fixed<Tag::kBytes == 4>(gn[j] * wv[cn]), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);
         }
       }
       hs = hs_next;
@@ -343,12 +357,13 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
     return hipGetLastError();
   };
-  const int cpl = (p.D + kRow - 1) / kRow;      // channels per lane: 1, 2 or 4 (3 rounds up to 4)
+  const int cpl = (p.D + kRow - 1) / kRow;      // channels per lane: 1, 2, 4 or 8 (odd counts round up)
 #define GV_CASE(KPV)                                                        \
   do {                                                                      \
     if (cpl == 1) return go(dcnv4_grad_value_kernel<Tag, KPV, 1>);          \
     if (cpl == 2) return go(dcnv4_grad_value_kernel<Tag, KPV, 2>);          \
-    return go(dcnv4_grad_value_kernel<Tag, KPV, 4>);                        \
+    if (cpl <= 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4>);          \
+    return go(dcnv4_grad_value_kernel<Tag, KPV, 8>);                        \
   } while (0)
   if (k3 && !p.remove_center) GV_CASE(9);
   if (k3 && p.remove_center) GV_CASE(8);
