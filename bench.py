@@ -52,6 +52,15 @@ def fda_bytes(s, B, N, Q, G, D, L, K):
     return s * (v + sla + out), s * (2 * v + 2 * sla + out)
 
 
+# HBM bytes moved per operator launch, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
+# `bench.py --only-op <key>`, each counter scaled by its reading for a plain copy of known size
+# (`--only-op copy:256`: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0, KiB).  The summaries are in profiles/.
+MEASURED_TRAFFIC_BYTES = {
+    "dcnv4_bwd:T-stage1:float32": 508.6e6,     # algorithmic 334.0e6: the tiled pass re-reads offset_mask and grad_out
+    "dcnv4_fwd:T-stage1:float16": 96.5e6,      # algorithmic 96.3e6
+}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -235,7 +244,8 @@ def main():
     dom_bytes = dom["MB"] * 1e6
     roofline = {
         "bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-        "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+        "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
+        "traffic": MEASURED_TRAFFIC_BYTES.get(f'{dom["op"]}:{dom["shape"]}:{dom["dtype"]}'),
         "kernel": f'{dom["op"]} {dom["shape"]} {dom["dtype"]}', "ms": dom["ms"],
         "algorithmic_bytes": int(dom_bytes),
         "note": "HIP events around whole operator calls (backward = state reset + grad_offset_mask kernel + tiled grad_value kernel + fallback)",

@@ -13,9 +13,10 @@
 //       A  tap-parallel: one lane per (pixel, group, kernel tap) recomputes the sampling position
 //          and, when a corner lands inside the tile, appends a hit record (four accumulator cells,
 //          four weights, pixel) to a per-group list in LDS; the strip's grad_out is parked in LDS;
-//       B  channel-parallel: a row of 16 lanes takes one hit record, lane c owns channel c (+16j),
+//       B  channel-parallel: a row of 8 lanes takes one hit record, lane c owns channels c, c+8, ...
 //          and adds its four corner contributions with 64-bit integer LDS atomics on fixed-point
-//          values.  Row r of every wave serves group r of the chunk, so with 16 channels per group
+//          values.  The 8 rows of a wave are dealt evenly to the groups of the chunk, and the second
+//          row of a group walks its channels in the opposite order, so with 16 channels per group
 //          one ds_add_u64 instruction touches 64 distinct channels: two conflict-free bank sweeps;
 //   * fixed point: contributions are normalised by the global maxima of |grad_out| and
 //     |modulation| (GradState, produced by the grad_offset_mask kernel that runs first) and carry
