@@ -8,6 +8,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 
 #include "../../include/dcnv4_gfx950.h"
 #include "common.hpp"
@@ -164,6 +165,53 @@ int plan_grad_value_tiles(DcnLaunch *L, int elem_bytes_of_launch) {
   if (L->Q >= (1 << 24) || (uint64_t)L->Q * (uint64_t)L->P_pad >= (1ull << 31) || (uint64_t)L->Q * (uint64_t)(L->G * L->D) >= (1ull << 31))
     return fail(DCNV4_ERR_RUNTIME, "one image of %d output pixels is too large for the tiled backward", L->Q);
   return DCNV4_OK;
+}
+
+// Tuning override: DCNV4_GFX950_GATHER=direct keeps the gathers on the global-memory kernels.
+bool tiled_gather_enabled() {
+  static const bool v = [] {
+    const char *e = getenv("DCNV4_GFX950_GATHER");
+    return !(e && strcmp(e, "direct") == 0);
+  }();
+  return v;
+}
+
+// Output tile, group chunk and input window of the LDS-tiled gather kernels.  Returns false (and
+// leaves gt_h = 0) when the shape does not suit them: group width not a power-of-two number of
+// 16-byte vectors, more than 32 channels per lane, or no tile whose window fits in LDS.
+constexpr int kTiledGatherThreads = 512;     // launch bound of the tiled gather kernels
+
+bool plan_gather_tiles(DcnLaunch *L, int s) {
+  L->gt_h = L->gt_w = L->gt_ng = L->gt_wh = L->gt_ww = 0;
+  L->gt_reach = reach_setting();
+  if (!tiled_gather_enabled() || L->softmax) return false;
+  const int lane_bytes = L->D * s;
+  if (lane_bytes % 16 != 0 || L->D > 32) return false;
+  const int nv = lane_bytes / 16;
+  if (nv != 1 && nv != 2 && nv != 4 && nv != 8) return false;
+  if (L->Kp > 64) return false;
+  const int Ho = L->Q / L->Wo, Wo = L->Wo, R = L->gt_reach;
+  auto even_split = [](int extent, int cap) { const int n = (extent + cap - 1) / cap; return (extent + n - 1) / n; };
+  // two workgroups per CU when the window allows it, so that one stages while the other computes
+  const size_t budgets[2] = {kMaxLdsPerWorkgroup / 2 - 512, kMaxLdsPerWorkgroup - 1024};
+  for (size_t budget : budgets) {
+    for (int cap_h = 16, cap_w = 16; cap_h >= 4 && cap_w >= 4;) {
+      L->gt_h = even_split(Ho, cap_h);
+      L->gt_w = even_split(Wo, cap_w);
+      L->gt_wh = std::min((L->gt_h - 1) * L->sh + 2 * R + 1, L->H + 2);
+      L->gt_ww = std::min((L->gt_w - 1) * L->sw + 2 * R + 1, L->W + 2);
+      const int px = L->gt_h * L->gt_w;
+      for (int ng = std::min(L->G, kTiledGatherThreads / px); ng >= 1; --ng) {
+        // 16-bit tensors: keep the offset_mask slices dword-aligned when the tap count is odd
+        if (s == 2 && ((ng * 3 * L->Kp) & 1) && ng > 1) continue;
+        L->gt_ng = ng;
+        if (dcnv4_tiled_gather_lds_bytes(*L, s) <= budget) return true;
+      }
+      if (cap_h >= cap_w) cap_h /= 2; else cap_w /= 2;
+    }
+  }
+  L->gt_h = L->gt_w = L->gt_ng = L->gt_wh = L->gt_ww = 0;
+  return false;
 }
 
 // ---------------------------------------------------------------- DCNv4
@@ -336,6 +384,7 @@ int dcnv4_gfx950_forward(const void *value, const void *offset_mask, void *outpu
     return rc;
   if (int rc = check_ptrs({value, offset_mask, output})) return rc;
   const int per = images_per_launch(pr, false);
+  const bool tiled = plan_gather_tiles(&pr.launch, pr.s);
   for (int b0 = 0; b0 < batch; b0 += per) {
     const int nb = std::min(per, batch - b0);
     DcnLaunch L = pr.launch;
@@ -344,8 +393,9 @@ int dcnv4_gfx950_forward(const void *value, const void *offset_mask, void *outpu
     L.out = at(output, b0 * pr.img_out_elems, pr.s);
     L.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
     L.n_pix = nb * L.Q;
-    if (hipError_t e = launch_dcnv4_forward(dtype, L, static_cast<hipStream_t>(stream)))
-      return hip_fail("dcnv4 forward launch", e);
+    const hipError_t e = tiled ? launch_dcnv4_forward_tiled(dtype, L, static_cast<hipStream_t>(stream))
+                               : launch_dcnv4_forward(dtype, L, static_cast<hipStream_t>(stream));
+    if (e) return hip_fail("dcnv4 forward launch", e);
   }
   return DCNV4_OK;
 }
@@ -384,6 +434,7 @@ int dcnv4_gfx950_backward(const void *value, const void *offset_mask, const void
     //    for corners beyond the reach / non-finite statistics (returns at once otherwise)
     DcnLaunch base = pr.launch;
     if (int rc = plan_grad_value_tiles(&base, pr.s)) return rc;
+    const bool gather_tiled = plan_gather_tiles(&base, pr.s);
     base.state = static_cast<GradState *>(workspace);
     hipLaunchKernelGGL(init_state_kernel, dim3(1), dim3(64), 0, st, base.state);
     if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);
@@ -401,7 +452,9 @@ int dcnv4_gfx950_backward(const void *value, const void *offset_mask, const void
         L.n_pix = nb * L.Q;
         L.n_img = nb;
         hipError_t e = hipSuccess;
-        if (pass == 0) {
+        if (pass == 0 && gather_tiled) {
+          e = launch_dcnv4_offset_mask_grad_tiled(dtype, L, st);
+        } else if (pass == 0) {
           // gathers want 16-byte lanes; the lane map chosen for scatter is only used by pass 2
           if (int rc = choose_lanes(group_channels, pr.s, 0, false, &L.lanes)) return rc;
           if (int rc = choose_block_pixels(&L, 0, true)) return rc;

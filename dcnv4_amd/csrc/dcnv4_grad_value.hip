@@ -96,7 +96,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   // output pixels this tile visits: reference point within `reach` of the tile (near_box)
   const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
   const int cy0 = half_h - p.ph, cx0 = half_w - p.pw, Ho = p.Q / p.Wo;
-  // every in-image corner lies within reach_needed of its reference point, so a smaller window than the
+  // every in-image corner that carries weight lies within reach_needed of its reference point, so a smaller window than the
   // planned cap loses nothing; beyond the cap the fallback kernel takes over
   const int reach = min(p.reach, (int)p.state->reach_needed);
   const int ho_lo = max(0, ceil_div_signed(ty0 - reach - cy0, p.sh));

@@ -185,7 +185,6 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
     float *gom = s_grad + lp * p.P_pad + g * 3 * Kp;
     float mx = 0.f, inv = 1.f;
     if (p.softmax) softmax_stats(om + 2 * Kp, Kp, mx, inv);
-    // reference point of this output pixel (centre tap, zero offset), for the reach rule
     // reference point of this output pixel (centre tap at zero offset) and the box the tiled scatter covers
     NearBox box = {0, 0, 0, 0};
     int p0y = 0, p0x = 0;
@@ -239,9 +238,11 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
       }
       if constexpr (MODE == kBwdOffsetMask) {
         mask_max = max(mask_max, __builtin_bit_cast(uint32_t, fabsf(m)));
-        if (t.valid != 0) {     // distance of the in-image part of the 2x2 corner block from the reference point
-          const int d = max(max(p0y - max(t.y0, 0), min(t.y0 + 1, p.H - 1) - p0y),
-                            max(p0x - max(t.x0, 0), min(t.x0 + 1, p.W - 1) - p0x));
+        if (t.valid != 0) {     // distance of the in-image part of the 2x2 corner block from the reference point;
+          // a far row or column whose bilinear weight is exactly zero (integer coordinate) adds nothing and is left out
+          const int y1 = t.y0 + (t.ly > 0.f ? 1 : 0), x1 = t.x0 + (t.lx > 0.f ? 1 : 0);
+          const int d = max(max(p0y - max(t.y0, 0), min(y1, p.H - 1) - p0y),
+                            max(p0x - max(t.x0, 0), min(x1, p.W - 1) - p0x));
           reach_needed = max(reach_needed, (uint32_t)max(d, 0));
         }
       }

@@ -1,0 +1,648 @@
+// DCNv4 forward and grad_offset_mask with the gather served from LDS.
+//
+// The reference's forward (DCNv4_op/src/cuda/dcnv4_im2col_cuda.cuh:142-244) fetches four vectors
+// per sampling point straight from global memory: 36 scattered 32-byte segments per (pixel,
+// group).  On MI355X that pattern is bound by the vector-memory address path, an order of
+// magnitude below what HBM delivers.  Sampling points stay close to their output pixel, so here
+//
+//   * a workgroup owns a tile of gt_h x gt_w output pixels of one image for gt_ng groups and
+//     copies the input window those pixels can reach (their reference points +- gt_reach input
+//     pixels, clipped to the image plus a one-pixel ring of zeros) into LDS with coalesced
+//     128-bit loads; cells outside the image come back as zeros from the buffer range check;
+//   * the workgroup's slice of offset_mask is parked in LDS next to it, in the tensor dtype;
+//   * one lane owns all D channels of one (pixel, group): the bilinear set-up is done once per
+//     sampling point instead of once per 16-byte channel chunk, no cross-lane traffic is
+//     needed, and the four corners are read from LDS with ds_read_b128;
+//   * a sampling point whose corners leave the window is remembered in a per-lane bit mask and
+//     served afterwards from global memory (the range-checked gather of dcnv4_kernels.hip), so
+//     any offset is handled; with offsets inside the window that code never runs.
+// The softmax variant of the modulation (never requested by the reference's Python side) stays on
+// the global-memory kernels.
+#include <type_traits>
+
+#include "common.hpp"
+#include "launch.hpp"
+
+#ifndef GT_PAD
+#define GT_PAD 16
+#endif
+
+namespace dcn {
+namespace {
+
+constexpr int kTiledThreads = 512;      // lanes per workgroup at most: leaves each wave 128+ registers
+
+// n / d for 0 <= n < 2^20 with inv = rcp(d) (one instruction, accurate to an ulp): the exact
+// quotient sits at least 0.5/d away from the next integer, far more than the error of the product.
+__device__ __forceinline__ float rcp(float d) { return __builtin_amdgcn_rcpf(d); }
+__device__ __forceinline__ int fdiv(int n, float inv) { return (int)(((float)n + 0.5f) * inv); }
+
+template <typename Tag>
+__device__ __forceinline__ float lds_elem(const typename RawWord<Tag::kBytes>::type *p, int i) {
+  float f[1];
+  Pack<Tag, 1>::decode(p[i], f);
+  return f[0];
+}
+
+// Geometry of one workgroup: its output tile, its group chunk and the input window it stages.
+struct TileGeom {
+  int b, g0, ng;           // image (within the launch), first group, groups in this chunk
+  int oy0, ox0, th, tw;    // output tile origin and extent inside the image
+  int wy0, wx0, wh, ww;    // input window origin (may be -1) and extent in cells
+};
+
+__device__ __forceinline__ TileGeom tile_geometry(const DcnLaunch &p) {
+  TileGeom t;
+  const int Ho = p.Q / p.Wo;
+  const int n_chunks = (p.G + p.gt_ng - 1) / p.gt_ng;
+  const int nty = (Ho + p.gt_h - 1) / p.gt_h, ntx = (p.Wo + p.gt_w - 1) / p.gt_w;
+  uint32_t id = xcd_contiguous_block(blockIdx.x, gridDim.x);
+  const int chunk = id % n_chunks; id /= n_chunks;
+  const int tx = id % ntx; id /= ntx;
+  const int ty = id % nty;
+  t.b = id / nty;
+  t.g0 = chunk * p.gt_ng;
+  t.ng = min(p.gt_ng, p.G - t.g0);
+  t.oy0 = ty * p.gt_h; t.ox0 = tx * p.gt_w;
+  t.th = min(p.gt_h, Ho - t.oy0); t.tw = min(p.gt_w, p.Wo - t.ox0);
+  // reference points (centre tap at zero offset) of the tile's first and last pixel
+  const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
+  const int yc0 = half_h - p.ph + t.oy0 * p.sh, yc1 = yc0 + (t.th - 1) * p.sh;
+  const int xc0 = half_w - p.pw + t.ox0 * p.sw, xc1 = xc0 + (t.tw - 1) * p.sw;
+  t.wy0 = max(yc0 - p.gt_reach, -1); t.wx0 = max(xc0 - p.gt_reach, -1);
+  t.wh = max(min(yc1 + p.gt_reach, p.H) - t.wy0 + 1, 0);
+  t.ww = max(min(xc1 + p.gt_reach, p.W) - t.wx0 + 1, 0);
+  return t;
+}
+
+// Fills the workgroup's LDS: the input window and this chunk's slice of offset_mask.
+//
+// Window: [wy0, wy0+wh) x [wx0, wx0+ww) of this chunk's channels, cell-major (cell = all channels
+// of the chunk for one input pixel, cell_stride bytes apart), followed by ww + 2 cells of zeros
+// that serve every corner of a sampling point that must contribute nothing.
+// offset_mask: tile pixel q, group gl of the chunk -> s_om[(q * gt_ng + gl) * 3 * Kp ...], in the
+// tensor dtype, untouched.
+//
+// The time of this phase is memory latency and address arithmetic, so: a lane keeps its place
+// inside a row (window row: cell and 16-byte piece; tile row: pixel and dword) and only the row
+// advances, by a uniform step; rows outside the image and idle lanes read through the dropped
+// offset of the buffer descriptor; and a lane issues a batch of loads before it stores any.
+template <typename Tag, int NV>
+__device__ __forceinline__ void stage_tile(const DcnLaunch &p, const TileGeom &t, char *s_win,
+                                           typename RawWord<Tag::kBytes>::type *s_om, int cell_stride) {
+  typedef typename RawWord<Tag::kBytes>::type elem_t;
+  constexpr int kBatch = 8;
+  const int bd = blockDim.x, tid = threadIdx.x;
+
+  // ---- window
+  {
+    const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
+    const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
+    const uint32_t img_base = (uint32_t)t.b * (uint32_t)(p.H * p.W) * pix_bytes + (uint32_t)(t.g0 * p.D) * Tag::kBytes;
+    const int ppc = t.ng * NV;                           // 16-byte pieces per cell
+    const int row_pieces = max(t.ww * ppc, 1);
+    const int rpp = max(bd / row_pieces, 1);             // window rows per pass
+    const int lanes_pp = min(bd, row_pieces);            // lanes of one row in one pass
+    const int col_passes = (row_pieces + bd - 1) / bd;   // > 1 only when a row is longer than the workgroup
+    const int r = fdiv(tid, rcp((float)row_pieces));    // row within the pass (0 when a row is longer)
+    for (int cp = 0; cp < col_passes; ++cp) {
+      const int rem = (col_passes == 1 ? tid - r * row_pieces : tid) + cp * lanes_pp;
+      const int wx = fdiv(rem, rcp((float)ppc)), piece = rem - wx * ppc;
+      const int x = t.wx0 + wx;
+      const bool lane_ok = (col_passes == 1 ? r < rpp : true) && rem < row_pieces;
+      const bool x_in = lane_ok && (unsigned)x < (unsigned)p.W;
+      const uint32_t g_lane = img_base + (uint32_t)x * pix_bytes + (uint32_t)piece * 16u;
+      const int l_lane = wx * cell_stride + piece * 16;
+      const int rows_step = col_passes == 1 ? rpp : 1;
+      for (int row0 = 0; row0 < t.wh; row0 += kBatch * rows_step) {
+        u32x4 raw[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          const int wy = row0 + u * rows_step + (col_passes == 1 ? r : 0), y = t.wy0 + wy;
+          const bool in = x_in && wy < t.wh && (unsigned)y < (unsigned)p.H;
+          raw[u] = buffer_load<16>(value, in ? g_lane + (uint32_t)(y * p.W) * pix_bytes : kDropOffset);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          const int wy = row0 + u * rows_step + (col_passes == 1 ? r : 0);
+          if (lane_ok && wy < t.wh) *reinterpret_cast<u32x4 *>(s_win + l_lane + wy * (t.ww * cell_stride)) = raw[u];
+        }
+      }
+    }
+    const int zero_base = t.wh * t.ww * cell_stride;
+    const int n_zero = (t.ww + 2) * cell_stride / 16;
+    for (int i = tid; i < n_zero; i += bd)
+      *reinterpret_cast<u32x4 *>(s_win + zero_base + i * 16) = u32x4{0u, 0u, 0u, 0u};
+  }
+
+  // ---- offset_mask slices
+  constexpr int EPW = 4 / Tag::kBytes;
+  const int run = t.ng * 3 * p.Kp, lds_row = p.gt_ng * 3 * p.Kp;          // elements per pixel: copied / LDS stride
+  const elem_t *om = reinterpret_cast<const elem_t *>(p.offset_mask) + ((size_t)t.b * p.Q + (size_t)t.oy0 * p.Wo + t.ox0) * p.P_pad +
+                     t.g0 * 3 * p.Kp;                                      // first element of the tile's slice
+  // whole dwords when every run starts and ends on a dword boundary (always for fp32)
+  const bool dwords = Tag::kBytes == 4 || (((p.P_pad | (t.g0 * 3 * p.Kp) | run | lds_row) & 1) == 0);
+  const int rw = run / EPW;                                               // dwords per pixel
+  int team_log2 = 0;
+  while ((1 << team_log2) < rw) ++team_log2;
+  if (dwords && (1 << team_log2) <= bd) {
+    // a power-of-two team of lanes per tile pixel; the tile's rows are row_bytes apart in memory
+    const uint32_t row_bytes = (uint32_t)p.Wo * p.P_pad * Tag::kBytes;
+    const __amdgpu_buffer_rsrc_t rows = make_rsrc(om, (uint32_t)(t.th - 1) * row_bytes + (uint32_t)((t.tw - 1) * p.P_pad + run) * Tag::kBytes);
+    uint32_t *s_om_w = reinterpret_cast<uint32_t *>(s_om);
+    const int ppp = bd >> team_log2;                                      // pixels per pass
+    const int pl = tid >> team_log2, j = tid & ((1 << team_log2) - 1);
+    for (int px0 = 0; px0 < t.tw; px0 += ppp) {
+      const int px = px0 + pl;
+      const bool live = px < t.tw && j < rw;
+      const uint32_t g_lane = live ? (uint32_t)(px * p.P_pad) * Tag::kBytes + 4u * j : kDropOffset;
+      const int l_lane = px * (lds_row / EPW) + j;
+      for (int py0 = 0; py0 < t.th; py0 += kBatch) {
+        uint32_t raw[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u)
+          raw[u] = buffer_load<4>(rows, py0 + u < t.th ? g_lane + (uint32_t)(py0 + u) * row_bytes : kDropOffset);
+        if (live) {
+#pragma unroll
+          for (int u = 0; u < kBatch; ++u)
+            if (py0 + u < t.th) s_om_w[l_lane + (py0 + u) * (p.gt_w * (lds_row / EPW))] = raw[u];
+        }
+      }
+    }
+  } else {            // odd alignments and very long rows: element by element
+    const int npx = p.gt_h * p.gt_w;
+    const float inv_run = rcp((float)run), inv_gtw = rcp((float)p.gt_w);
+    for (int idx = tid; idx < npx * run; idx += bd) {
+      const int q = fdiv(idx, inv_run), jj = idx - q * run;
+      const int py = fdiv(q, inv_gtw), px = q - py * p.gt_w;
+      if (py < t.th && px < t.tw) s_om[q * lds_row + jj] = om[((size_t)py * p.Wo + px) * p.P_pad + jj];
+    }
+  }
+}
+
+// Writes the gradient slices parked in LDS (layout of stage_tile) back to grad_offset_mask, and
+// zeros the padding tail of the rows when this workgroup owns the last group.
+template <typename Tag>
+__device__ __forceinline__ void unstage_tile_grads(const DcnLaunch &p, const TileGeom &t,
+                                                   const typename RawWord<Tag::kBytes>::type *s_om) {
+  typedef typename RawWord<Tag::kBytes>::type elem_t;
+  constexpr int EPW = 4 / Tag::kBytes;
+  const int bd = blockDim.x, tid = threadIdx.x;
+  const int run = t.ng * 3 * p.Kp, lds_row = p.gt_ng * 3 * p.Kp;
+  elem_t *gom = reinterpret_cast<elem_t *>(p.grad_offset_mask) + ((size_t)t.b * p.Q + (size_t)t.oy0 * p.Wo + t.ox0) * p.P_pad +
+                t.g0 * 3 * p.Kp;
+  const bool dwords = Tag::kBytes == 4 || (((p.P_pad | (t.g0 * 3 * p.Kp) | run | lds_row) & 1) == 0);
+  const int rw = run / EPW;
+  int team_log2 = 0;
+  while ((1 << team_log2) < rw) ++team_log2;
+  if (dwords && (1 << team_log2) <= bd) {
+    const uint32_t row_bytes = (uint32_t)p.Wo * p.P_pad * Tag::kBytes;
+    const __amdgpu_buffer_rsrc_t rows = make_rsrc(gom, (uint32_t)(t.th - 1) * row_bytes + (uint32_t)((t.tw - 1) * p.P_pad + run) * Tag::kBytes);
+    const uint32_t *s_om_w = reinterpret_cast<const uint32_t *>(s_om);
+    const int ppp = bd >> team_log2;
+    const int pl = tid >> team_log2, j = tid & ((1 << team_log2) - 1);
+    for (int px0 = 0; px0 < t.tw; px0 += ppp) {
+      const int px = px0 + pl;
+      if (px < t.tw && j < rw) {
+        const uint32_t g_lane = (uint32_t)(px * p.P_pad) * Tag::kBytes + 4u * j;
+        const int l_lane = px * (lds_row / EPW) + j;
+        for (int py = 0; py < t.th; ++py)
+          __builtin_amdgcn_raw_buffer_store_b32(s_om_w[l_lane + py * (p.gt_w * (lds_row / EPW))], rows,
+                                                g_lane + (uint32_t)py * row_bytes, 0, 0);
+      }
+    }
+  } else {
+    const int npx = p.gt_h * p.gt_w;
+    const float inv_run = rcp((float)run), inv_gtw = rcp((float)p.gt_w);
+    for (int idx = tid; idx < npx * run; idx += bd) {
+      const int q = fdiv(idx, inv_run), jj = idx - q * run;
+      const int py = fdiv(q, inv_gtw), px = q - py * p.gt_w;
+      if (py < t.th && px < t.tw) gom[((size_t)py * p.Wo + px) * p.P_pad + jj] = s_om[q * lds_row + jj];
+    }
+  }
+  const int tail = p.P_pad - p.G * 3 * p.Kp;
+  if (tail > 0 && t.g0 + t.ng == p.G) {
+    const float inv_tail = rcp((float)tail), inv_tw = rcp((float)t.tw);
+    for (int idx = tid; idx < t.th * t.tw * tail; idx += bd) {
+      const int q = fdiv(idx, inv_tail), jj = idx - q * tail;
+      const int py = fdiv(q, inv_tw), px = q - py * t.tw;
+      gom[((size_t)py * p.Wo + px) * p.P_pad + run + jj] = elem_t(0);
+    }
+  }
+}
+
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  for (int o = 32; o > 0; o >>= 1) v = max(v, (uint32_t)__shfl_xor((int)v, o, kWave));
+  return v;
+}
+
+// One sampling point against the staged window.
+struct WinTap {
+  float w[4];          // bilinear weights of the four corners (without the modulation)
+  float ly, lx;
+  int addr;            // LDS byte address of corner 0 for this lane's channels (the zero cells when !ok)
+  int ry, rx;          // corner 0 relative to the window origin
+  bool inside, ok;     // passes the reference's range test / and both corner rows and columns are staged
+};
+
+__device__ __forceinline__ WinTap window_tap(float y, float x, int H, int W, const TileGeom &t, int cell_stride,
+                                             int lane_bytes, int zero_base) {
+  WinTap r;
+  r.inside = (y > -1.f) && (x > -1.f) && (y < (float)H) && (x < (float)W);       // dcnv4_im2col_cuda.cuh:227
+  y = r.inside ? y : 0.f;
+  x = r.inside ? x : 0.f;
+  const float fy = floorf(y), fx = floorf(x);
+  const int ry = (int)fy - t.wy0, rx = (int)fx - t.wx0;
+  r.ry = ry; r.rx = rx;
+  r.ly = y - fy; r.lx = x - fx;
+  const float hy = 1.f - r.ly, hx = 1.f - r.lx;
+  r.w[0] = hy * hx; r.w[1] = hy * r.lx; r.w[2] = r.ly * hx; r.w[3] = r.ly * r.lx;
+  const bool near = (unsigned)ry < (unsigned)max(t.wh - 1, 0) && (unsigned)rx < (unsigned)max(t.ww - 1, 0);
+  r.ok = r.inside && near;
+  r.addr = r.ok ? __mul24(__mul24(ry, t.ww) + rx, cell_stride) + lane_bytes : zero_base;
+  return r;
+}
+
+template <typename Tag, int NV, int KP>
+__global__ void __launch_bounds__(kTiledThreads) dcnv4_forward_tiled_kernel(const DcnLaunch p) {
+  extern __shared__ u32x4 lds128[];
+  typedef typename RawWord<Tag::kBytes>::type elem_t;
+  constexpr int EPV = 16 / Tag::kBytes;           // elements per 16-byte vector
+  typedef Pack<Tag, EPV> pack;
+  const TileGeom t = tile_geometry(p);
+  const int Kp = p.Kp;
+  const int cell_stride = p.gt_ng * p.D * Tag::kBytes + GT_PAD;
+  char *s_win = reinterpret_cast<char *>(lds128);
+  elem_t *s_om = reinterpret_cast<elem_t *>(s_win + (size_t)(p.gt_wh * p.gt_ww + p.gt_ww + 2) * cell_stride);
+  stage_tile<Tag, NV>(p, t, s_win, s_om, cell_stride);
+  __syncthreads();
+
+  // lane -> (tile pixel, group of the chunk)
+  const int q = fdiv(threadIdx.x, rcp((float)p.gt_ng)), gl = threadIdx.x - q * p.gt_ng;
+  const int py = fdiv(q, rcp((float)p.gt_w)), px = q - py * p.gt_w;
+  if (q >= p.gt_h * p.gt_w || gl >= t.ng || py >= t.th || px >= t.tw) return;
+  const int ho = t.oy0 + py, wo = t.ox0 + px;
+  const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
+  const float x_base = sub_rn((float)(half_w - p.pw + wo * p.sw), mul_rn((float)half_w, p.offset_scale));
+  const float y_base = sub_rn((float)(half_h - p.ph + ho * p.sh), mul_rn((float)half_h, p.offset_scale));
+  const elem_t *om = s_om + threadIdx.x * 3 * Kp;
+  const int zero_base = t.wh * t.ww * cell_stride, row_bytes = t.ww * cell_stride;
+  const int lane_bytes = gl * p.D * Tag::kBytes;
+  float acc[NV][EPV];
+#pragma unroll
+  for (int v = 0; v < NV; ++v)
+#pragma unroll
+    for (int c = 0; c < EPV; ++c) acc[v][c] = 0.f;
+  typedef typename std::conditional<(KP > 0), uint32_t, uint64_t>::type mask_t;     // one bit per sampling point
+  mask_t far_mask = 0;
+
+  auto position = [&](int k, int i, int j, float &y, float &x, float &m) {
+    x = add_rn(x_base, mul_rn(add_rn((float)(i * p.dw), lds_elem<Tag>(om, 2 * k)), p.offset_scale));
+    y = add_rn(y_base, mul_rn(add_rn((float)(j * p.dh), lds_elem<Tag>(om, 2 * k + 1)), p.offset_scale));
+    m = lds_elem<Tag>(om, 2 * Kp + k);
+  };
+  // A sampling point in flight: its four modulated corner weights and its LDS reads.
+  struct Flight {
+    float w[4];
+    u32x4 raw[4][NV];
+  };
+  auto issue = [&](int k, int i, int j, Flight &fl) {
+    float y, x, m;
+    position(k, i, j, y, x, m);
+    const WinTap wt = window_tap(y, x, p.H, p.W, t, cell_stride, lane_bytes, zero_base);
+    far_mask |= (mask_t)(wt.inside && !wt.ok) << k;
+#pragma unroll
+    for (int cn = 0; cn < 4; ++cn) {
+      fl.w[cn] = m * wt.w[cn];
+      const char *src = s_win + wt.addr + (cn & 1) * cell_stride + (cn >> 1) * row_bytes;
+#pragma unroll
+      for (int v = 0; v < NV; ++v) fl.raw[cn][v] = *reinterpret_cast<const u32x4 *>(src + 16 * v);
+    }
+  };
+  auto retire = [&](const Flight &fl) {
+#pragma unroll
+    for (int cn = 0; cn < 4; ++cn) {
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        float f[EPV];
+        pack::decode(fl.raw[cn][v], f);
+#pragma unroll
+        for (int c = 0; c < EPV; ++c) acc[v][c] = fmaf(fl.w[cn], f[c], acc[v][c]);
+      }
+    }
+  };
+  // a sampling point whose corners lie outside the staged window: gather from memory instead
+  const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
+  const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
+  const uint32_t img_base = (uint32_t)t.b * (uint32_t)(p.H * p.W) * pix_bytes + (uint32_t)((t.g0 + gl) * p.D) * Tag::kBytes;
+  auto far_tap = [&](int k, int i, int j) {
+    float y, x, m;
+    position(k, i, j, y, x, m);
+    const Tap tp = make_tap(y, x, p.H, p.W, img_base, pix_bytes);
+#pragma unroll
+    for (int cn = 0; cn < 4; ++cn) {
+      const float w = m * tp.w[cn];
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        float f[EPV];
+        pack::decode(buffer_load<16>(value, tp.off[cn] + 16u * v), f);      // a dropped corner stays out of range
+#pragma unroll
+        for (int c = 0; c < EPV; ++c) acc[v][c] = fmaf(w, f[c], acc[v][c]);
+      }
+    }
+  };
+
+  if constexpr (KP > 0) {
+    // A real loop, one sampling point at a time: unrolled, the compiler front-loads all 72 LDS reads
+    // and spills, and keeping two points in flight by hand costs more in registers (occupancy) than
+    // the overlap returns; other waves cover the LDS latency.
+#pragma unroll 1
+    for (int k = 0; k < KP; ++k) {
+      int i, j;
+      tap_ij_3x3(KP, k, i, j);
+      Flight fl;
+      issue(k, i, j, fl);
+      retire(fl);
+    }
+    if (far_mask != 0) {
+      for (int k = 0; k < KP; ++k) {
+        if (!((far_mask >> k) & 1)) continue;
+        int i, j;
+        tap_ij_3x3(KP, k, i, j);
+        far_tap(k, i, j);
+      }
+    }
+  } else {
+    for (int pass = 0; pass < 2; ++pass) {
+      if (pass == 1 && far_mask == 0) break;
+      int k = 0;
+      for (int i = 0; i < p.kw; ++i)
+        for (int j = 0; j < p.kh; ++j) {
+          if (p.remove_center && i == p.kw / 2 && j == p.kh / 2) continue;
+          if (pass == 0) {
+            Flight fl;
+            issue(k, i, j, fl);
+            retire(fl);
+          } else if ((far_mask >> k) & 1) {
+            far_tap(k, i, j);
+          }
+          ++k;
+        }
+    }
+  }
+
+  char *dst = (char *)p.out + (((size_t)t.b * p.Q + (size_t)ho * p.Wo + wo) * (p.G * p.D) + (t.g0 + gl) * p.D) * Tag::kBytes;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) *reinterpret_cast<u32x4 *>(dst + 16 * v) = pack::encode(acc[v]);
+}
+
+// ------------------------------------------------------------------------------- backward
+// grad_offset_mask from the staged window (the part of dcnv4_col2im_cuda.cuh:280-350 and
+// common.h:188-211 that does not scatter): for every sampling point the four corner . grad_out
+// dot products give d/dx, d/dy and d/dmask.  One lane holds all D channels of its (pixel, group),
+// so nothing is reduced across lanes.  The gradients replace the lane's own offset_mask slice in
+// LDS (each slot is read before it is overwritten) and the slices go back to memory as rows;
+// the workgroup that owns the last groups also clears the padding tail of its rows.  The kernel
+// also folds the statistics the tiled grad_value kernel needs into GradState.
+template <typename Tag, int NV, int KP>
+__global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_kernel(const DcnLaunch p) {
+  extern __shared__ u32x4 lds128[];
+  typedef typename RawWord<Tag::kBytes>::type elem_t;
+  constexpr int EPV = 16 / Tag::kBytes;
+  typedef Pack<Tag, EPV> pack;
+  const TileGeom t = tile_geometry(p);
+  const int Kp = p.Kp;
+  const int cell_stride = p.gt_ng * p.D * Tag::kBytes + GT_PAD;
+  char *s_win = reinterpret_cast<char *>(lds128);
+  elem_t *s_om = reinterpret_cast<elem_t *>(s_win + (size_t)(p.gt_wh * p.gt_ww + p.gt_ww + 2) * cell_stride);
+  __shared__ uint32_t s_stat[3];
+  if (threadIdx.x < 3) s_stat[threadIdx.x] = 0u;
+
+  // lane -> (tile pixel, group of the chunk); its grad_out vector is requested before the staging
+  const int q = fdiv(threadIdx.x, rcp((float)p.gt_ng)), gl = threadIdx.x - q * p.gt_ng;
+  const int py = fdiv(q, rcp((float)p.gt_w)), px = q - py * p.gt_w;
+  const bool active = q < p.gt_h * p.gt_w && gl < t.ng && py < t.th && px < t.tw;
+  const int ho = t.oy0 + py, wo = t.ox0 + px;
+  u32x4 go_raw[NV];
+  {
+    const char *src = (const char *)p.grad_out +
+                      (((size_t)t.b * p.Q + (size_t)(active ? ho * p.Wo + wo : 0)) * (p.G * p.D) + (active ? t.g0 + gl : 0) * p.D) * Tag::kBytes;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) go_raw[v] = *reinterpret_cast<const u32x4 *>(src + 16 * v);
+  }
+  stage_tile<Tag, NV>(p, t, s_win, s_om, cell_stride);
+  __syncthreads();
+
+  uint32_t go_max = 0, mask_max = 0, reach_needed = 0;
+  if (active) {
+    float go[NV][EPV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      pack::decode(go_raw[v], go[v]);
+#pragma unroll
+      for (int c = 0; c < EPV; ++c) go_max = max(go_max, __builtin_bit_cast(uint32_t, fabsf(go[v][c])));
+    }
+    const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
+    const int p0y = half_h - p.ph + ho * p.sh, p0x = half_w - p.pw + wo * p.sw;      // reference point
+    const float x_base = sub_rn((float)p0x, mul_rn((float)half_w, p.offset_scale));
+    const float y_base = sub_rn((float)p0y, mul_rn((float)half_h, p.offset_scale));
+    elem_t *om = s_om + threadIdx.x * 3 * Kp;
+    const int zero_base = t.wh * t.ww * cell_stride, row_bytes = t.ww * cell_stride;
+    const int lane_bytes = gl * p.D * Tag::kBytes;
+    typedef typename std::conditional<(KP > 0), uint32_t, uint64_t>::type mask_t;
+    mask_t far_mask = 0;
+    auto put = [&](int k, float gx, float gy, float gz, float m) {
+      const float f0[1] = {gx * p.offset_scale * m}, f1[1] = {gy * p.offset_scale * m}, f2[1] = {gz};
+      om[2 * k] = Pack<Tag, 1>::encode(f0);
+      om[2 * k + 1] = Pack<Tag, 1>::encode(f1);
+      om[2 * Kp + k] = Pack<Tag, 1>::encode(f2);
+    };
+    auto combine = [&](int k, const float (&d)[4], float ly, float lx, const float (&w)[4], float m) {
+      const float hy = 1.f - ly, hx = 1.f - lx;
+      const float gx = hy * (d[1] - d[0]) + ly * (d[3] - d[2]);      // common.h:188-201
+      const float gy = hx * (d[2] - d[0]) + lx * (d[3] - d[1]);
+      const float gz = w[0] * d[0] + w[1] * d[1] + w[2] * d[2] + w[3] * d[3];
+      put(k, gx, gy, gz, m);
+    };
+    auto one_tap = [&](int k, int i, int j) {
+      const float x = add_rn(x_base, mul_rn(add_rn((float)(i * p.dw), lds_elem<Tag>(om, 2 * k)), p.offset_scale));
+      const float y = add_rn(y_base, mul_rn(add_rn((float)(j * p.dh), lds_elem<Tag>(om, 2 * k + 1)), p.offset_scale));
+      const float m = lds_elem<Tag>(om, 2 * Kp + k);
+      mask_max = max(mask_max, __builtin_bit_cast(uint32_t, fabsf(m)));
+      const WinTap wt = window_tap(y, x, p.H, p.W, t, cell_stride, lane_bytes, zero_base);
+      far_mask |= (mask_t)(wt.inside && !wt.ok) << k;
+      if (wt.inside) {      // distance of the weighted, in-image part of the 2x2 corner block from the reference point
+        const int y0 = wt.ry + t.wy0, x0 = wt.rx + t.wx0;
+        const int y1 = y0 + (wt.ly > 0.f ? 1 : 0), x1 = x0 + (wt.lx > 0.f ? 1 : 0);
+        const int d = max(max(p0y - max(y0, 0), min(y1, p.H - 1) - p0y), max(p0x - max(x0, 0), min(x1, p.W - 1) - p0x));
+        reach_needed = max(reach_needed, (uint32_t)max(d, 0));
+      }
+      u32x4 raw[4][NV];
+#pragma unroll
+      for (int cn = 0; cn < 4; ++cn) {
+        const char *src = s_win + wt.addr + (cn & 1) * cell_stride + (cn >> 1) * row_bytes;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) raw[cn][v] = *reinterpret_cast<const u32x4 *>(src + 16 * v);
+      }
+      float d[4];
+#pragma unroll
+      for (int cn = 0; cn < 4; ++cn) {
+        float acc = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+          float f[EPV];
+          pack::decode(raw[cn][v], f);
+#pragma unroll
+          for (int c = 0; c < EPV; ++c) acc = fmaf(f[c], go[v][c], acc);
+        }
+        d[cn] = acc;
+      }
+      combine(k, d, wt.ly, wt.lx, wt.w, m);      // all zeros for a point outside the image or the window
+    };
+    // a sampling point whose corners lie outside the staged window: gather from memory; its
+    // offsets are re-read from memory because the LDS slots already hold gradients
+    const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
+    const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
+    const uint32_t img_base = (uint32_t)t.b * (uint32_t)(p.H * p.W) * pix_bytes + (uint32_t)((t.g0 + gl) * p.D) * Tag::kBytes;
+    const elem_t *om_g = reinterpret_cast<const elem_t *>(p.offset_mask) +
+                         ((size_t)t.b * p.Q + (size_t)ho * p.Wo + wo) * p.P_pad + (t.g0 + gl) * 3 * Kp;
+    auto far_tap = [&](int k, int i, int j) {
+      const float x = add_rn(x_base, mul_rn(add_rn((float)(i * p.dw), lds_elem<Tag>(om_g, 2 * k)), p.offset_scale));
+      const float y = add_rn(y_base, mul_rn(add_rn((float)(j * p.dh), lds_elem<Tag>(om_g, 2 * k + 1)), p.offset_scale));
+      const float m = lds_elem<Tag>(om_g, 2 * Kp + k);
+      const Tap tp = make_tap(y, x, p.H, p.W, img_base, pix_bytes);
+      float d[4];
+#pragma unroll
+      for (int cn = 0; cn < 4; ++cn) {
+        float acc = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+          float f[EPV];
+          pack::decode(buffer_load<16>(value, tp.off[cn] + 16u * v), f);
+#pragma unroll
+          for (int c = 0; c < EPV; ++c) acc = fmaf(f[c], go[v][c], acc);
+        }
+        d[cn] = acc;
+      }
+      combine(k, d, tp.ly, tp.lx, tp.w, m);
+    };
+
+    if constexpr (KP > 0) {
+#pragma unroll 1
+      for (int k = 0; k < KP; ++k) {
+        int i, j;
+        tap_ij_3x3(KP, k, i, j);
+        one_tap(k, i, j);
+      }
+      if (far_mask != 0) {
+        for (int k = 0; k < KP; ++k) {
+          if (!((far_mask >> k) & 1)) continue;
+          int i, j;
+          tap_ij_3x3(KP, k, i, j);
+          far_tap(k, i, j);
+        }
+      }
+    } else {
+      for (int pass = 0; pass < 2; ++pass) {
+        if (pass == 1 && far_mask == 0) break;
+        int k = 0;
+        for (int i = 0; i < p.kw; ++i)
+          for (int j = 0; j < p.kh; ++j) {
+            if (p.remove_center && i == p.kw / 2 && j == p.kh / 2) continue;
+            if (pass == 0) one_tap(k, i, j);
+            else if ((far_mask >> k) & 1) far_tap(k, i, j);
+            ++k;
+          }
+      }
+    }
+  }
+
+  // statistics: fold in LDS, then touch the global words only when they would grow (same-address
+  // global atomics retire slowly)
+  go_max = wave_max_u32(go_max);
+  mask_max = wave_max_u32(mask_max);
+  reach_needed = wave_max_u32(reach_needed);
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    atomicMax(&s_stat[0], go_max);
+    atomicMax(&s_stat[1], mask_max);
+    atomicMax(&s_stat[2], reach_needed);
+  }
+  __syncthreads();
+  if (threadIdx.x < 3) {
+    uint32_t *dst = &p.state->go_max_bits + threadIdx.x;
+    const uint32_t mine = s_stat[threadIdx.x];
+    if (mine > __hip_atomic_load(dst, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(dst, mine);
+  }
+  unstage_tile_grads<Tag>(p, t, s_om);
+}
+
+template <typename Tag, int NV, bool BWD>
+hipError_t launch_nv(const DcnLaunch &p, hipStream_t stream, dim3 grid, dim3 block, size_t lds) {
+  const bool k3 = p.kh == 3 && p.kw == 3;
+  auto go = [&](auto kernel) -> hipError_t {
+    static bool raised = false;        // per kernel instantiation: dynamic LDS above 64 KB needs the attribute
+    if (!raised) {
+      if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLdsPerWorkgroup - 1024))   // leaves room for static LDS
+        return e;
+      raised = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
+    return hipGetLastError();
+  };
+  if constexpr (BWD) {
+    if (k3 && !p.remove_center) return go(dcnv4_offset_mask_grad_tiled_kernel<Tag, NV, 9>);
+    if (k3 && p.remove_center) return go(dcnv4_offset_mask_grad_tiled_kernel<Tag, NV, 8>);
+    return go(dcnv4_offset_mask_grad_tiled_kernel<Tag, NV, 0>);
+  } else {
+    if (k3 && !p.remove_center) return go(dcnv4_forward_tiled_kernel<Tag, NV, 9>);
+    if (k3 && p.remove_center) return go(dcnv4_forward_tiled_kernel<Tag, NV, 8>);
+    return go(dcnv4_forward_tiled_kernel<Tag, NV, 0>);
+  }
+}
+
+template <typename Tag, bool BWD>
+hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
+  const int Ho = p.Q / p.Wo;
+  const int n_chunks = (p.G + p.gt_ng - 1) / p.gt_ng;
+  const int nty = (Ho + p.gt_h - 1) / p.gt_h, ntx = (p.Wo + p.gt_w - 1) / p.gt_w;
+  const int n_img = p.n_pix / p.Q;
+  const dim3 grid((unsigned)(n_img * nty * ntx * n_chunks));
+  const dim3 block((unsigned)((p.gt_h * p.gt_w * p.gt_ng + kWave - 1) / kWave * kWave));
+  const size_t lds = dcnv4_tiled_gather_lds_bytes(p, Tag::kBytes);
+  switch (p.D * Tag::kBytes / 16) {
+    case 1: return launch_nv<Tag, 1, BWD>(p, stream, grid, block, lds);
+    case 2: return launch_nv<Tag, 2, BWD>(p, stream, grid, block, lds);
+    case 4: return launch_nv<Tag, 4, BWD>(p, stream, grid, block, lds);
+    case 8: return launch_nv<Tag, 8, BWD>(p, stream, grid, block, lds);
+  }
+  return hipErrorInvalidValue;
+}
+
+template <bool BWD>
+hipError_t launch_any(int dtype, const DcnLaunch &p, hipStream_t stream) {
+  switch (dtype) {
+    case F32::kCode: return launch_t<F32, BWD>(p, stream);
+    case F16::kCode: return launch_t<F16, BWD>(p, stream);
+    case BF16::kCode: return launch_t<BF16, BWD>(p, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+size_t dcnv4_tiled_gather_lds_bytes(const DcnLaunch &p, int elem_bytes) {
+  const size_t cell = (size_t)p.gt_ng * p.D * elem_bytes + GT_PAD;
+  return (size_t)(p.gt_wh * p.gt_ww + p.gt_ww + 2) * cell +                     // window + zero cells
+         (((size_t)p.gt_h * p.gt_w * p.gt_ng * 3 * p.Kp * elem_bytes + 15) & ~size_t(15));   // offset_mask slices
+}
+
+hipError_t launch_dcnv4_forward_tiled(int dtype, const DcnLaunch &p, hipStream_t stream) {
+  return launch_any<false>(dtype, p, stream);
+}
+
+hipError_t launch_dcnv4_offset_mask_grad_tiled(int dtype, const DcnLaunch &p, hipStream_t stream) {
+  return launch_any<true>(dtype, p, stream);
+}
+
+}  // namespace dcn

@@ -19,7 +19,7 @@ constexpr size_t kMaxLdsPerWorkgroup = 160 * 1024;  // gfx950
 struct GradState {
   uint32_t go_max_bits;    // max |grad_out| as IEEE bits (ordered like unsigned ints for x >= 0; NaN sorts last)
   uint32_t mask_max_bits;  // max |modulation| (after softmax when enabled)
-  uint32_t reach_needed;   // largest Chebyshev distance (pixels) of an in-image corner from its output pixel's reference point
+  uint32_t reach_needed;   // largest Chebyshev distance (pixels) of an in-image corner of non-zero weight from its output pixel's reference point
   uint32_t reserved;
 };
 
@@ -61,6 +61,11 @@ struct DcnLaunch {
   int ng_chunk;             // groups per workgroup (channel chunk = ng_chunk * D)
   int strip_pix;            // output pixels staged per strip
   int fix_bits;             // fractional bits of the 64-bit fixed-point accumulators
+  // LDS-tiled gather path (forward and grad_offset_mask); gt_h == 0: not planned
+  int gt_h, gt_w;           // output tile one workgroup owns
+  int gt_ng;                // groups per workgroup
+  int gt_wh, gt_ww;         // largest input window (rows, columns of cells) a tile stages
+  int gt_reach;             // input pixels around an output pixel's reference point that the window covers
 };
 
 // Flash deformable attention (reference: DCNv4_op/src/cuda/flash_deform_im2col_cuda.cuh:211-272)
@@ -85,6 +90,9 @@ hipError_t launch_dcnv4_forward(int dtype, const DcnLaunch &p, hipStream_t strea
 hipError_t launch_dcnv4_backward(int dtype, const DcnLaunch &p, int mode, hipStream_t stream);
 hipError_t launch_dcnv4_grad_value(int dtype, const DcnLaunch &p, hipStream_t stream);
 size_t dcnv4_grad_value_lds_bytes(const DcnLaunch &p);
+hipError_t launch_dcnv4_forward_tiled(int dtype, const DcnLaunch &p, hipStream_t stream);
+hipError_t launch_dcnv4_offset_mask_grad_tiled(int dtype, const DcnLaunch &p, hipStream_t stream);
+size_t dcnv4_tiled_gather_lds_bytes(const DcnLaunch &p, int elem_bytes);
 hipError_t launch_fda_forward(int dtype, const FdaLaunch &p, hipStream_t stream);
 hipError_t launch_fda_backward(int dtype, const FdaLaunch &p, hipStream_t stream);
 
