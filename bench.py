@@ -35,6 +35,9 @@ CFG2 = [("T-stage1", 64, 56, 56, 64, 4), ("T-stage2", 64, 28, 28, 128, 8),
         ("T-stage3", 64, 14, 14, 256, 16), ("T-stage4", 64, 7, 7, 512, 32)]
 CFG3 = [("L-dense1", 2, 256, 256, 160, 10), ("L-dense2", 2, 128, 128, 320, 20),
         ("L-dense3", 2, 64, 64, 640, 40), ("L-dense4", 2, 32, 32, 1280, 80)]
+# per-layer shapes of the FlashInternImage-B forward at batch 128 (offsets U(-3,3) here; the random-init model itself has zero offsets)
+CFG5 = [("B-stage1", 128, 56, 56, 112, 7), ("B-stage2", 128, 28, 28, 224, 14),
+        ("B-stage3", 128, 14, 14, 448, 28), ("B-stage4", 128, 7, 7, 896, 56)]
 CFG4_SHAPES = [(128, 128), (64, 64), (32, 32), (16, 16)]
 
 
@@ -123,23 +126,27 @@ def main():
                           "GBps_read_plus_write": round(2 * n * 4 / (ms * 1e-3) / 1e9, 1)}))
         return
 
+    if args.only_op:
+        op, shape_name, dt_name = args.only_op.split(":")
+        dtype = getattr(torch, dt_name)
+        for table, off in ((CFG2, 3.0), (CFG3, 4.0), (CFG5, 3.0)):
+            for name, B, H, W, C, G in table:
+                if name != shape_name:
+                    continue
+                t = dcn_inputs(B, H, W, C, G, dtype, off)
+                fn = (lambda: dcn_fwd(t, G, C)) if op == "dcnv4_fwd" else (lambda: dcn_bwd(t, G, C))
+                ms = time_op(fn, args.steps, warm=args.warmup)
+                nbytes = dcn_bytes(t[0].element_size(), B, H, W, C, G)[0 if op == "dcnv4_fwd" else 1]
+                print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "algorithmic_MB": round(nbytes / 1e6, 2),
+                                  "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)}))
+                return
+        sys.exit(f"--only-op {args.only_op}: no such DCNv4 shape")
+
     # ------------------------------------------------------------------ the step (configs[1])
     work = []
     for dtype, s in ((torch.float16, 2), (torch.float32, 4)):
         for name, B, H, W, C, G in CFG2:
             work.append((name, dtype, s, (B, H, W, C, G), dcn_inputs(B, H, W, C, G, dtype, 3.0)))
-
-    if args.only_op:
-        op, shape_name, dt_name = args.only_op.split(":")
-        for name, dtype, s, (B, H, W, C, G), t in work:
-            if name == shape_name and str(dtype) == "torch." + dt_name:
-                fn = (lambda: dcn_fwd(t, G, C)) if op == "dcnv4_fwd" else (lambda: dcn_bwd(t, G, C))
-                ms = time_op(fn, args.steps, warm=args.warmup)
-                nbytes = dcn_bytes(s, B, H, W, C, G)[0 if op == "dcnv4_fwd" else 1]
-                print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "algorithmic_MB": round(nbytes / 1e6, 2),
-                                  "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)}))
-                return
-        sys.exit(f"--only-op {args.only_op}: no such operator in the step")
 
     def step():
         for _, _, _, (B, H, W, C, G), t in work:
@@ -178,6 +185,10 @@ def main():
             fb, bb = dcn_bytes(2, B, H, W, C, G)
             add("dcnv4_fwd", name, torch.float16, time_op(lambda: dcn_fwd(t, G, C), args.op_iters), fb)
             add("dcnv4_bwd", name, torch.float16, time_op(lambda: dcn_bwd(t, G, C), args.op_iters), bb)
+            del t
+        for name, B, H, W, C, G in CFG5:
+            t = dcn_inputs(B, H, W, C, G, torch.float16, 3.0)
+            add("dcnv4_fwd", name, torch.float16, time_op(lambda: dcn_fwd(t, G, C), args.op_iters), dcn_bytes(2, B, H, W, C, G)[0])
             del t
         B, G, D, L, K = 4, 8, 32, 4, 4
         N = sum(h * w for h, w in CFG4_SHAPES)

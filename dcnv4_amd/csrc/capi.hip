@@ -123,14 +123,13 @@ constexpr int kTiledMaxGroupChannels = 64;
 
 bool tiled_grad_value(int D) { return D <= kTiledMaxGroupChannels; }
 
-// Tuning override for the cap on the reach of the tiled grad_value kernel (pixels).
+// Tuning override, read on every call: DCNV4_GFX950_REACH = distance (input pixels) from an output
+// pixel's reference point that the tiled kernels cover; sampling points beyond it take the
+// global-memory paths.  Default 5.
 int reach_setting() {
-  static const int v = [] {
-    const char *e = getenv("DCNV4_GFX950_REACH");
-    const int r = e ? atoi(e) : 5;
-    return r < 0 ? 0 : (r > 64 ? 64 : r);
-  }();
-  return v;
+  const char *e = getenv("DCNV4_GFX950_REACH");
+  const int r = e ? atoi(e) : 5;
+  return r < 0 ? 0 : (r > 64 ? 64 : r);
 }
 
 // Tile, channel chunk and strip of the tiled grad_value kernel such that its LDS footprint fits.
@@ -167,13 +166,11 @@ int plan_grad_value_tiles(DcnLaunch *L, int elem_bytes_of_launch) {
   return DCNV4_OK;
 }
 
-// Tuning override: DCNV4_GFX950_GATHER=direct keeps the gathers on the global-memory kernels.
+// Tuning override, read on every call: DCNV4_GFX950_GATHER=direct keeps the gathers on the
+// global-memory kernels.
 bool tiled_gather_enabled() {
-  static const bool v = [] {
-    const char *e = getenv("DCNV4_GFX950_GATHER");
-    return !(e && strcmp(e, "direct") == 0);
-  }();
-  return v;
+  const char *e = getenv("DCNV4_GFX950_GATHER");
+  return !(e && strcmp(e, "direct") == 0);
 }
 
 // Output tile, group chunk and input window of the LDS-tiled gather kernels.  Returns false (and

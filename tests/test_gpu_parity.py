@@ -68,6 +68,39 @@ def test_dcnv4_forward_and_backward_match_oracle(oracle, name, dtype):
     assert (gom[..., used:] == 0).all(), "padded tail of grad_offset_mask must be exactly zero"
 
 
+# The library picks between kernel families by shape; these settings force the other branches:
+# the global-memory gather kernels, and (tiny reach) the per-point fallbacks of the LDS-tiled
+# kernels plus the far-corner scatter of the backward.
+KERNEL_PATHS = {
+    "direct_gather": {"DCNV4_GFX950_GATHER": "direct"},
+    "reach1": {"DCNV4_GFX950_REACH": "1"},
+    "reach0": {"DCNV4_GFX950_REACH": "0"},
+    "reach9": {"DCNV4_GFX950_REACH": "9"},
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("path", list(KERNEL_PATHS))
+@pytest.mark.parametrize("name", ["cfg1_56x56_c64_g4", "g7_c112_scale_half", "remove_center", "stride2", "dilation2_pad2",
+                                  "kernel_5x5", "far_offsets_mostly_outside", "wide_g80"])
+def test_dcnv4_every_kernel_path_matches_oracle(oracle, monkeypatch, name, path, dtype):
+    for key, val in KERNEL_PATHS[path].items():
+        monkeypatch.setenv(key, val)
+    v, om, go, (geom, G, D, scale, rc) = _dcn_inputs(DCN_CASES[name], dtype, seed=zlib.crc32((name + path).encode()) % 1000)
+    print(f"case {name} path {path} dtype {dtype}", flush=True)
+    args = _oracle_args(geom, G, D, scale, rc)
+    want = oracle.dcnv4_forward(cabi.f64(v), cabi.f64(om), *args, coord_f32=True)
+    wgv, wgom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *args, coord_f32=True)
+    out = cabi.dcnv4_forward(v.cuda(), om.cuda(), geom, G, D, scale, rc)
+    gv, gom = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), geom, G, D, scale, rc)
+    torch.cuda.synchronize()
+    cabi.assert_close(out, want, *FWD_TOL[dtype], what="output")
+    cabi.assert_close(gv, wgv, *GRAD_TOL[dtype], what="grad_value")
+    cabi.assert_close(gom, wgom, *GRAD_TOL[dtype], what="grad_offset_mask")
+    used = G * 3 * (geom[0] * geom[1] - rc)
+    assert (gom[..., used:] == 0).all(), "padded tail of grad_offset_mask must be exactly zero"
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16], ids=["fp32", "fp16"])
 def test_dcnv4_softmax_flag_matches_oracle(oracle, dtype):
     v, om, go, (geom, G, D, scale, rc) = _dcn_inputs(DCN_CASES["remove_center"], dtype, seed=5)
