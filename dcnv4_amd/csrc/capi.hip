@@ -137,6 +137,12 @@ int plan_grad_value_tiles(DcnLaunch *L, int elem_bytes_of_launch) {
   const int D = L->D;
   L->reach = reach_setting();
   L->ng_chunk = std::max(1, std::min(L->G, kTiledMaxGroupChannels / std::max(D, 16)));   // <= 4
+  // 16-bit tensors: two 32-bit fixed-point sums per accumulator word when that leaves at least 18
+  // fractional bits.  A cell collects at most one corner per tap from the (2*reach+1)^2 output pixels
+  // around it, each of magnitude <= 2^fix_bits, and the sum must stay below 2^31.
+  const long long per_cell = (long long)(2 * L->reach + 1) * (2 * L->reach + 1) * L->Kp;
+  const int fix32 = 31 - ceil_log2((int)std::min<long long>(per_cell, 1 << 30));
+  L->pack32 = (elem_bytes_of_launch == 2 && D > 8 && fix32 >= 18) ? 1 : 0;
   // power-of-two tiles (the reach rule uses shifts); shrink until the LDS footprint fits
   L->tile_h_log2 = 4;
   L->tile_w_log2 = 4;
@@ -160,6 +166,7 @@ int plan_grad_value_tiles(DcnLaunch *L, int elem_bytes_of_launch) {
   const long long contributions = (long long)visited(L->tile_h, L->sh) * visited(L->tile_w, L->sw) * L->Kp;
   L->fix_bits = 62 - ceil_log2((int)std::min<long long>(contributions, 1 << 30));
   if (elem_bytes_of_launch == 2) L->fix_bits = std::min(L->fix_bits, 30);   // 32-bit conversion path for 16-bit tensors
+  if (L->pack32) L->fix_bits = std::min(fix32, 22);                         // the rounding trick of the packed path needs |term| < 2^22
   // the tiled kernel addresses one image's offset_mask and grad_out with 32-bit element offsets
   if (L->Q >= (1 << 24) || (uint64_t)L->Q * (uint64_t)L->P_pad >= (1ull << 31) || (uint64_t)L->Q * (uint64_t)(L->G * L->D) >= (1ull << 31))
     return fail(DCNV4_ERR_RUNTIME, "one image of %d output pixels is too large for the tiled backward", L->Q);

@@ -55,12 +55,31 @@ template <bool WIDE> __device__ __forceinline__ unsigned long long to_fixed(floa
   }
 }
 
+// round-to-nearest-even(a * b) for |a * b| < 2^22, two instructions: the product is formed inside an
+// fma whose addend pushes the integer part into the low mantissa bits.
+__device__ __forceinline__ int to_fixed32(float a, float b) {
+  return (int)(__builtin_bit_cast(uint32_t, fmaf(a, b, 12582912.f)) - 0x4B400000u);
+}
+
 struct HitMeta {
   uint32_t cells012;    // accumulator cell of corners 0,1,2 (9 bits each); n_cells = "nowhere" (weight 0)
   uint32_t cell3_px;    // cell of corner 3 | strip-local pixel << 9
 };
 
-template <typename Tag, int KP, int CPL>
+// channels per lane for a group of D channels: 1, 2, 4 or 8 (odd counts round up)
+__host__ __device__ inline int channels_per_lane(int D) {
+  const int c = (D + kRow - 1) / kRow;
+  return c <= 2 ? c : (c <= 4 ? 4 : 8);
+}
+
+// Accumulator words per cell.  PACK (16-bit tensors): one 64-bit word holds two 32-bit fixed-point
+// sums, the lane's channels c + 16k (low half) and c + 8 + 16k (high half); a group then takes
+// 4 * CPL words.  Otherwise one word per channel.
+__host__ __device__ inline int acc_words_per_cell(int ng_chunk, int D, bool pack) {
+  return pack ? ng_chunk * 4 * channels_per_lane(D) : ng_chunk * D;
+}
+
+template <typename Tag, int KP, int CPL, bool PACK>
 __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const DcnLaunch p) {
   extern __shared__ unsigned long long lds64[];
   const int Kp = p.Kp, D = p.D, C = p.G * p.D;
@@ -72,13 +91,15 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   const int ty = id % nty;
   const int b = id / nty;
   const int g0 = chunk * p.ng_chunk, ng = min(p.ng_chunk, p.G - g0);
-  const int ch_stride = p.ng_chunk * D;                 // accumulator channels per cell
+  const int ch_stride = p.ng_chunk * D;                 // channels of the chunk
+  const int acc_stride = PACK ? p.ng_chunk * 4 * CPL : ch_stride;       // accumulator words per cell
+  constexpr int kGroupWords = PACK ? 4 * CPL : 0;                       // PACK: words per group within a cell
   const int ty0 = ty << p.tile_h_log2, tx0 = tx << p.tile_w_log2;
   const int th = min(p.tile_h, p.H - ty0), tw = min(p.tile_w, p.W - tx0);
   const int n_cells = p.tile_h * p.tile_w;
   // the slots past the tile absorb the zero-valued adds of corners outside the tile, and of lanes
   // whose channel index runs past D (group widths that are not multiples of 16)
-  const int n_acc = ((n_cells + 1) * ch_stride + kTrashPad + 1) & ~1;      // even: keeps the lists 16-byte aligned
+  const int n_acc = ((n_cells + 1) * acc_stride + kTrashPad + 1) & ~1;     // even: keeps the lists 16-byte aligned
   const int list_cap = p.strip_pix * Kp;                // hit records per group list
   unsigned long long *acc = lds64;
   f32x4 *hit_w = reinterpret_cast<f32x4 *>(lds64 + n_acc);                       // [ng_chunk][list_cap]
@@ -285,7 +306,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       for (int g = 1; g < ng; ++g) n_max = max(n_max, count[g]);
       const int lane_group = group_live ? my_group : 0;                  // idle rows only ever add zeros to the trash slots
       const bool flip = (my_slot & 1) != 0;
-      unsigned long long *acc_lane = acc + lane_group * D + c;
+      unsigned long long *acc_lane = acc + (PACK ? lane_group * kGroupWords : lane_group * D) + c;
       const float *go_lane = s_go + lane_group * D + c;
       for (uint32_t i0 = wave * rows_per_group; i0 < n_max; i0 += kWaves * rows_per_group) {
         const uint32_t i = i0 + my_slot;
@@ -301,7 +322,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
         int ch_off[CPL];
 #pragma unroll
         for (int j = 0; j < CPL; ++j) {
-          ch_off[j] = kRow * (flip ? CPL - 1 - j : j);
+          ch_off[j] = kRow * ((flip && !PACK) ? CPL - 1 - j : j);
           gn[j] = (c + ch_off[j] < D) ? go_lane[px * ch_stride + ch_off[j]] : 0.f;
         }
         const uint32_t cells[4] = {meta.cells012 & 511u, (meta.cells012 >> kCellBits) & 511u,
@@ -309,11 +330,23 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
         const float wv[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
         for (int cn = 0; cn < 4; ++cn) {
-          unsigned long long *dst = acc_lane + __umul24(cells[cn], (uint32_t)ch_stride);
+          unsigned long long *dst = acc_lane + __umul24(cells[cn], (uint32_t)acc_stride);
+          if constexpr (PACK) {
+            // two channels per atomic: sum = hi * 2^32 + lo with both halves signed, so the low term is
+            // sign-extended into the high word before the add
 #pragma unroll
-          for (int j = 0; j < CPL; ++j)
-            __hip_atomic_fetch_add(dst + ch_off[j], to_fixed<Tag::kBytes == 4>(gn[j] * wv[cn]), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+            for (int j = 0; j < CPL; j += 2) {
+              const int lo = to_fixed32(gn[j], wv[cn]);
+              const int hi = j + 1 < CPL ? to_fixed32(gn[j + 1], wv[cn]) : 0;
+              const unsigned long long v = ((unsigned long long)(uint32_t)(hi + (lo >> 31)) << 32) | (uint32_t)lo;
+              __hip_atomic_fetch_add(dst + (j / 2) * kRow, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < CPL; ++j)
+              __hip_atomic_fetch_add(dst + ch_off[j], to_fixed<Tag::kBytes == 4>(gn[j] * wv[cn]), __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_WORKGROUP);
+          }
         }
       }
       hs = hs_next;
@@ -328,12 +361,20 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   const int n_ch = ng * D;
   for (int cell = wave; cell < th * tw; cell += kValThreads / kWave) {     // one cell per wave: contiguous channels
     const int ly = cell / tw, lx = cell - ly * tw;
-    const unsigned long long *src = acc + ((ly << p.tile_w_log2) + lx) * ch_stride;
+    const unsigned long long *src = acc + ((ly << p.tile_w_log2) + lx) * acc_stride;
     elem_t *dst = reinterpret_cast<elem_t *>(p.grad_value) + (((size_t)b * p.H + ty0 + ly) * p.W + tx0 + lx) * C + g0 * D;
     for (int ch = lane; ch < n_ch; ch += kWave) {
-      const unsigned long long a = src[ch];
-      const double v = ldexp((double)(int)(a >> 32) * 4294967296.0 + (double)(uint32_t)a, e_out);
-      const float f[1] = {(float)v};
+      float f[1];
+      if constexpr (PACK) {
+        const int g = ch / D, cg = ch - g * D, j = cg / kRow;
+        const unsigned long long a = src[g * kGroupWords + (j >> 1) * kRow + (cg & (kRow - 1))];
+        const int lo = (int)(uint32_t)a;
+        const int field = (j & 1) ? (int)(uint32_t)(a >> 32) + (lo < 0 ? 1 : 0) : lo;
+        f[0] = ldexpf((float)field, e_out);
+      } else {
+        const unsigned long long a = src[ch];
+        f[0] = (float)ldexp((double)(int)(a >> 32) * 4294967296.0 + (double)(uint32_t)a, e_out);
+      }
       dst[ch] = Pack<Tag, 1>::encode(f);
     }
   }
@@ -358,13 +399,19 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
     return hipGetLastError();
   };
-  const int cpl = (p.D + kRow - 1) / kRow;      // channels per lane: 1, 2, 4 or 8 (odd counts round up)
-#define GV_CASE(KPV)                                                        \
-  do {                                                                      \
-    if (cpl == 1) return go(dcnv4_grad_value_kernel<Tag, KPV, 1>);          \
-    if (cpl == 2) return go(dcnv4_grad_value_kernel<Tag, KPV, 2>);          \
-    if (cpl <= 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4>);          \
-    return go(dcnv4_grad_value_kernel<Tag, KPV, 8>);                        \
+  const int cpl = channels_per_lane(p.D);
+  constexpr bool kCanPack = Tag::kBytes == 2;
+#define GV_CASE(KPV)                                                                        \
+  do {                                                                                      \
+    if constexpr (kCanPack) {                                                               \
+      if (p.pack32 && cpl == 2) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, true>);      \
+      if (p.pack32 && cpl == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, true>);      \
+      if (p.pack32 && cpl == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, true>);      \
+    }                                                                                       \
+    if (cpl == 1) return go(dcnv4_grad_value_kernel<Tag, KPV, 1, false>);                   \
+    if (cpl == 2) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, false>);                   \
+    if (cpl == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, false>);                   \
+    return go(dcnv4_grad_value_kernel<Tag, KPV, 8, false>);                                 \
   } while (0)
   if (k3 && !p.remove_center) GV_CASE(9);
   if (k3 && p.remove_center) GV_CASE(8);
@@ -376,7 +423,8 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
 
 size_t dcnv4_grad_value_lds_bytes(const DcnLaunch &p) {
   const size_t ch_stride = (size_t)p.ng_chunk * p.D, list = (size_t)p.ng_chunk * p.strip_pix * p.Kp;
-  return ((((size_t)(p.tile_h * p.tile_w + 1) * ch_stride + kTrashPad + 1) & ~size_t(1)) * sizeof(unsigned long long)) +  // accumulators
+  const size_t acc_stride = acc_words_per_cell(p.ng_chunk, p.D, p.pack32 != 0);
+  return ((((size_t)(p.tile_h * p.tile_w + 1) * acc_stride + kTrashPad + 1) & ~size_t(1)) * sizeof(unsigned long long)) +  // accumulators
          list * (sizeof(f32x4) + sizeof(HitMeta)) +                                                    // hit lists
          (size_t)p.strip_pix * ch_stride * sizeof(float) + 2 * kMaxChunkGroups * sizeof(uint32_t);     // grad_out, two counter sets
 }

@@ -60,7 +60,8 @@ struct DcnLaunch {
   int reach;                // cap on the reach the tiled scatter covers; it uses min(reach, GradState::reach_needed)
   int ng_chunk;             // groups per workgroup (channel chunk = ng_chunk * D)
   int strip_pix;            // output pixels staged per strip
-  int fix_bits;             // fractional bits of the 64-bit fixed-point accumulators
+  int fix_bits;             // fractional bits of the fixed-point accumulators
+  int pack32;               // 16-bit tensors: two 32-bit sums per accumulator word instead of one 64-bit sum
   // LDS-tiled gather path (forward and grad_offset_mask); gt_h == 0: not planned
   int gt_h, gt_w;           // output tile one workgroup owns
   int gt_ng;                // groups per workgroup
