@@ -126,9 +126,31 @@ def main():
                           "GBps_read_plus_write": round(2 * n * 4 / (ms * 1e-3) / 1e9, 1)}))
         return
 
+    def fda_inputs(dtype):
+        B, G, D, L, K = 4, 8, 32, 4, 4
+        N = sum(h * w for h, w in CFG4_SHAPES)
+        shapes = torch.tensor(CFG4_SHAPES, dtype=torch.int64, device=dev)
+        sizes = [h * w for h, w in CFG4_SHAPES]
+        starts = torch.tensor([sum(sizes[:i]) for i in range(L)], dtype=torch.int64, device=dev)
+        v = torch.randn(B, N, G, D, device=dev).to(dtype)
+        sla = torch.cat([torch.rand(B, N, G, L * K * 2, device=dev), torch.randn(B, N, G, L * K, device=dev)], -1).to(dtype)
+        go = torch.randn(B, N, G * D, device=dev).to(dtype)
+        return (B, N, G, D, L, K), shapes, starts, v, sla, go
+
     if args.only_op:
         op, shape_name, dt_name = args.only_op.split(":")
         dtype = getattr(torch, dt_name)
+        if op.startswith("flash_deform_attn"):
+            (B, N, G, D, L, K), shapes, starts, v, sla, go = fda_inputs(dtype)
+            if op.endswith("fwd"):
+                fn = lambda: ext.flash_deform_attn_forward(v, shapes, starts, sla, 64, K, 0, 0)
+            else:
+                fn = lambda: ext.flash_deform_attn_backward(v, shapes, starts, sla, go, 64, K, 0, 0)
+            ms = time_op(fn, args.steps, warm=args.warmup)
+            nbytes = fda_bytes(v.element_size(), B, N, N, G, D, L, K)[0 if op.endswith("fwd") else 1]
+            print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "algorithmic_MB": round(nbytes / 1e6, 2),
+                              "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)}))
+            return
         for table, off in ((CFG2, 3.0), (CFG3, 4.0), (CFG5, 3.0)):
             for name, B, H, W, C, G in table:
                 if name != shape_name:
@@ -190,15 +212,8 @@ def main():
             t = dcn_inputs(B, H, W, C, G, torch.float16, 3.0)
             add("dcnv4_fwd", name, torch.float16, time_op(lambda: dcn_fwd(t, G, C), args.op_iters), dcn_bytes(2, B, H, W, C, G)[0])
             del t
-        B, G, D, L, K = 4, 8, 32, 4, 4
-        N = sum(h * w for h, w in CFG4_SHAPES)
-        shapes = torch.tensor(CFG4_SHAPES, dtype=torch.int64, device=dev)
-        sizes = [h * w for h, w in CFG4_SHAPES]
-        starts = torch.tensor([sum(sizes[:i]) for i in range(L)], dtype=torch.int64, device=dev)
         for dtype, s in ((torch.float16, 2), (torch.float32, 4)):
-            v = torch.randn(B, N, G, D, device=dev).to(dtype)
-            sla = torch.cat([torch.rand(B, N, G, L * K * 2, device=dev), torch.randn(B, N, G, L * K, device=dev)], -1).to(dtype)
-            go = torch.randn(B, N, G * D, device=dev).to(dtype)
+            (B, N, G, D, L, K), shapes, starts, v, sla, go = fda_inputs(dtype)
             fb, bb = fda_bytes(s, B, N, N, G, D, L, K)
             add("flash_deform_attn_fwd", "DETR-enc 4lvl Q=21760", dtype,
                 time_op(lambda: ext.flash_deform_attn_forward(v, shapes, starts, sla, 64, K, 0, 0), args.op_iters), fb)

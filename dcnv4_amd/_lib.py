@@ -10,7 +10,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libdcnv4_gfx950.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 OK, ERR_INVALID_ARGUMENT, ERR_RUNTIME = 0, 1, 2
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 
@@ -24,7 +24,7 @@ SIGNATURES = {
     "dcnv4_gfx950_backward_workspace_bytes": (_sz, [_i] * 6),
     "dcnv4_gfx950_backward": (_i, [_vp] * 6 + [_sz, _i] + [_i] * 13 + [_f] + [_i] * 6 + [_vp]),
     "flash_deform_attn_gfx950_forward": (_i, [_vp] * 5 + [_i] * 11 + [_vp]),
-    "flash_deform_attn_gfx950_backward_workspace_bytes": (_sz, [_i] * 5),
+    "flash_deform_attn_gfx950_backward_workspace_bytes": (_sz, [_i] * 8),
     "flash_deform_attn_gfx950_backward": (_i, [_vp] * 8 + [_sz] + [_i] * 11 + [_vp]),
 }
 

@@ -132,6 +132,18 @@ int reach_setting() {
   return r < 0 ? 0 : (r > 64 ? 64 : r);
 }
 
+// Flash attention backward: head widths the tiled grad_value kernel handles (8 lanes x up to 4 channels,
+// whole 8-channel blocks), with point counts that fit its 32-bit point ids.
+bool fda_tiled_shape(int D, int L, int Q, int K) {
+  return D % 8 == 0 && D <= 32 && L >= 1 && K >= 1 && (long long)Q * K < (1ll << 31);
+}
+
+// Tuning override, read on every call: DCNV4_GFX950_FDA_SCATTER=atomic keeps the fp32 atomic scatter.
+bool fda_tiled_enabled() {
+  const char *e = getenv("DCNV4_GFX950_FDA_SCATTER");
+  return !(e && strcmp(e, "atomic") == 0);
+}
+
 // Tile, channel chunk and strip of the tiled grad_value kernel such that its LDS footprint fits.
 int plan_grad_value_tiles(DcnLaunch *L, int elem_bytes_of_launch) {
   const int D = L->D;
@@ -303,7 +315,7 @@ struct FdaProblem {
   size_t img_elems, img_row_elems, img_out_elems;
 };
 
-int fda_prepare(FdaProblem *pr, bool backward, int dtype, int batch, int N, int G, int D, int L, int Q, int K,
+int fda_prepare(FdaProblem *pr, bool backward, bool scatter, int dtype, int batch, int N, int G, int D, int L, int Q, int K,
                 int im2col_step, int d_stride, int block_thread) {
   const int s = elem_bytes(dtype);
   if (s == 0) return fail(DCNV4_ERR_RUNTIME, "unsupported dtype code %d (fp32, fp16, bf16 only)", dtype);
@@ -319,7 +331,7 @@ int fda_prepare(FdaProblem *pr, bool backward, int dtype, int batch, int N, int 
 
   FdaLaunch &F = pr->launch;
   F = FdaLaunch{};
-  if (int rc = choose_lanes(D, s, d_stride, backward, &F.lanes)) return rc;
+  if (int rc = choose_lanes(D, s, d_stride, scatter, &F.lanes)) return rc;
   const int width = 1 << F.lanes.tpgp_log2;
   if (backward && width > kWave)
     return fail(DCNV4_ERR_INVALID_ARGUMENT, "backward needs head_channels/%d <= 64 lanes per head, got %d",
@@ -500,7 +512,7 @@ int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_s
                                      int head_channels, int num_levels, int num_query, int num_points,
                                      int im2col_step, int d_stride, int block_thread, void *stream) {
   FdaProblem pr;
-  if (int rc = fda_prepare(&pr, false, dtype, batch, spatial_size, num_heads, head_channels, num_levels, num_query,
+  if (int rc = fda_prepare(&pr, false, false, dtype, batch, spatial_size, num_heads, head_channels, num_levels, num_query,
                            num_points, im2col_step, d_stride, block_thread))
     return rc;
   if (int rc = check_ptrs({value, sampling_loc_attn, output})) return rc;
@@ -523,9 +535,14 @@ int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_s
 }
 
 size_t flash_deform_attn_gfx950_backward_workspace_bytes(int dtype, int batch, int spatial_size, int num_heads,
-                                                         int head_channels) {
-  if (elem_bytes(dtype) != 2 || batch <= 0 || spatial_size <= 0 || num_heads <= 0 || head_channels <= 0) return 0;
-  return round16((size_t)batch * spatial_size * num_heads * head_channels * sizeof(float));
+                                                         int head_channels, int num_levels, int num_query,
+                                                         int num_points) {
+  if (elem_bytes(dtype) == 0 || batch <= 0 || spatial_size <= 0 || num_heads <= 0 || head_channels <= 0) return 0;
+  size_t need = 0;
+  if (elem_bytes(dtype) == 2) need = round16((size_t)batch * spatial_size * num_heads * head_channels * sizeof(float));
+  if (fda_tiled_shape(head_channels, num_levels, num_query, num_points))
+    need = std::max(need, kStateBytes + 2 * round16((size_t)batch * num_heads * num_levels * num_query * num_points * sizeof(uint32_t)));
+  return need;
 }
 
 int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_shapes,
@@ -536,22 +553,65 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
                                       int num_query, int num_points, int im2col_step, int d_stride,
                                       int block_thread, void *stream) {
   FdaProblem pr;
-  if (int rc = fda_prepare(&pr, true, dtype, batch, spatial_size, num_heads, head_channels, num_levels, num_query,
+  const bool tiled = fda_tiled_shape(head_channels, num_levels, num_query, num_points) && fda_tiled_enabled();
+  // the tiled path gathers only: 16-byte lanes; the atomic path wants one channel per lane
+  if (int rc = fda_prepare(&pr, true, !tiled, dtype, batch, spatial_size, num_heads, head_channels, num_levels, num_query,
                            num_points, im2col_step, d_stride, block_thread))
     return rc;
   if (int rc = check_ptrs({value, sampling_loc_attn, grad_output, grad_value, grad_sampling_loc_attn})) return rc;
   if (spatial_shapes == nullptr || level_start_index == nullptr) return fail(DCNV4_ERR_RUNTIME, "null level tensors");
-  const size_t need =
-      flash_deform_attn_gfx950_backward_workspace_bytes(dtype, batch, spatial_size, num_heads, head_channels);
+  const size_t need = flash_deform_attn_gfx950_backward_workspace_bytes(dtype, batch, spatial_size, num_heads, head_channels,
+                                                                        num_levels, num_query, num_points);
   if (need > 0) {
     if (workspace == nullptr || !aligned16(workspace) || workspace_bytes < need)
       return fail(DCNV4_ERR_RUNTIME, "workspace of %zu bytes needed, got %zu at %p", need, workspace_bytes, workspace);
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   const size_t total = (size_t)batch * pr.img_elems;
-  float *acc = need > 0 ? static_cast<float *>(workspace) : static_cast<float *>(grad_value);
-  if (hipError_t e = clear_async(acc, total, st)) return hip_fail("clear launch", e);
   const int per = images_per_launch(pr, true);
+
+  if (tiled) {
+    // pass 0: grad_sampling_loc_attn, keys and max |grad_out|; pass 1: tiled grad_value; pass 2: fallback
+    FdaLaunch base = pr.launch;
+    base.state = static_cast<GradState *>(workspace);
+    const size_t key_bytes = round16((size_t)batch * num_heads * num_levels * num_query * num_points * sizeof(uint32_t));
+    uint32_t *keys = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + kStateBytes);
+    float *probs = reinterpret_cast<float *>(static_cast<char *>(workspace) + kStateBytes + key_bytes);
+    // every term is grad_out * (probability * bilinear weight <= 1); at most Q * K of them meet in one cell
+    base.fix_bits = 62 - ceil_log2((int)std::min<long long>((long long)num_query * num_points, 1 << 30));
+    if (pr.s == 2) base.fix_bits = std::min(base.fix_bits, 30);
+    hipLaunchKernelGGL(init_state_kernel, dim3(1), dim3(64), 0, st, base.state);
+    if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);
+    const size_t img_keys = (size_t)num_heads * num_levels * num_query * num_points;
+    for (int pass = 0; pass < 3; ++pass) {
+      for (int b0 = 0; b0 < batch; b0 += per) {
+        const int nb = std::min(per, batch - b0);
+        FdaLaunch F = base;
+        F.value = at(value, b0 * pr.img_elems, pr.s);
+        F.sla = at(sampling_loc_attn, b0 * pr.img_row_elems, pr.s);
+        F.grad_out = at(grad_output, b0 * pr.img_out_elems, pr.s);
+        F.grad_value = at(grad_value, b0 * pr.img_elems, pr.s);
+        F.grad_sla = at(grad_sampling_loc_attn, b0 * pr.img_row_elems, pr.s);
+        F.keys = keys + b0 * img_keys;
+        F.probs = probs + b0 * img_keys;
+        F.shapes = spatial_shapes;
+        F.level_start = level_start_index;
+        F.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
+        F.n_row = nb * F.Q;
+        F.n_img = nb;
+        hipError_t e = hipSuccess;
+        if (pass == 0) e = launch_fda_backward(dtype, F, kFdaNoScatter, st);
+        else if (pass == 1) e = launch_fda_grad_value(dtype, F, st);
+        else e = launch_fda_backward(dtype, F, kFdaFallback, st);
+        if (e) return hip_fail("flash_deform_attn backward launch", e);
+      }
+    }
+    return DCNV4_OK;
+  }
+
+  const bool widen = pr.s == 2;
+  float *acc = widen ? static_cast<float *>(workspace) : static_cast<float *>(grad_value);
+  if (hipError_t e = clear_async(acc, total, st)) return hip_fail("clear launch", e);
   for (int b0 = 0; b0 < batch; b0 += per) {
     const int nb = std::min(per, batch - b0);
     FdaLaunch F = pr.launch;
@@ -564,9 +624,9 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
     F.level_start = level_start_index;
     F.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
     F.n_row = nb * F.Q;
-    if (hipError_t e = launch_fda_backward(dtype, F, st)) return hip_fail("flash_deform_attn backward launch", e);
+    if (hipError_t e = launch_fda_backward(dtype, F, kFdaFull, st)) return hip_fail("flash_deform_attn backward launch", e);
   }
-  if (need > 0)
+  if (widen)
     if (hipError_t e = narrow_async(dtype, acc, grad_value, total, st)) return hip_fail("cast launch", e);
   return DCNV4_OK;
 }

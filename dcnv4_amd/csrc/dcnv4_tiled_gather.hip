@@ -231,11 +231,6 @@ __device__ __forceinline__ void unstage_tile_grads(const DcnLaunch &p, const Til
   }
 }
 
-__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-  for (int o = 32; o > 0; o >>= 1) v = max(v, (uint32_t)__shfl_xor((int)v, o, kWave));
-  return v;
-}
-
 // One sampling point against the staged window.
 struct WinTap {
   float w[4];          // bilinear weights of the four corners (without the modulation)

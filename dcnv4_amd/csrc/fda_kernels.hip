@@ -91,10 +91,20 @@ __global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLau
 }
 
 // ------------------------------------------------------------------------------- backward
-template <typename Tag, int CPT, int KT>
+// One kernel body, three roles (FdaBackwardMode):
+//   kFdaFull       grad_sampling_loc_attn, and grad_value scattered with fp32 buffer atomics into a
+//                  cleared fp32 image (any head width)
+//   kFdaNoScatter  grad_sampling_loc_attn, plus what the tiled grad_value kernel needs: one key per
+//                  sampling point and the maximum of |grad_out|
+//   kFdaFallback   exits at once unless max |grad_out| is not finite; then it scatters with atomics in
+//                  the tensor dtype into grad_value, which the tiled kernel has left zeroed
+template <typename Tag, int CPT, int KT, int MODE>
 __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLaunch p) {
   extern __shared__ float lds[];
   typedef Pack<Tag, CPT> pack;
+  if constexpr (MODE == kFdaFallback) {
+    if (p.state->go_max_bits < 0x7f800000u) return;
+  }
   const int LK = p.L * p.K, row_len = 3 * LK;
   const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
   const int row0 = (int)blk * p.nq_block;
@@ -111,6 +121,7 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
   const int items = (nrow * p.G) << tpgp_log2;
   const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
   const int K = KT > 0 ? KT : p.K;
+  uint32_t go_max = 0;
 
   for (int it = threadIdx.x; it < items; it += blockDim.x) {
     const int chunk = it & (width - 1);
@@ -134,6 +145,11 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
       }
     }
     float dot_rg = 0.f;
+    if constexpr (MODE == kFdaNoScatter) {
+#pragma unroll
+      for (int c = 0; c < CPT; ++c) go_max = max(go_max, __builtin_bit_cast(uint32_t, fabsf(go[c])));
+    }
+    const int b_local = (row0 + lr) / p.Q, q = (row0 + lr) - b_local * p.Q;
 
     for (int l = 0; l < p.L; ++l) {
       const Level lv = load_level(p, l);
@@ -149,6 +165,28 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
 #pragma unroll
           for (int cn = 0; cn < 4; ++cn) tp.off[cn] = kDropOffset;
         }
+        if constexpr (MODE == kFdaNoScatter) {
+          if (chunk == 0) {
+            uint32_t key = kFdaKeyOutside;
+            if (tp.valid != 0)
+              key = (tp.y0 + 1 >= kFdaKeyFieldMax || tp.x0 + 1 >= kFdaKeyFieldMax) ? kFdaKeySaturated
+                                                                                  : ((uint32_t)(tp.y0 + 1) << 16) | (uint32_t)(tp.x0 + 1);
+            const size_t slot = ((((size_t)b_local * p.G + g) * p.L + l) * p.Q + q) * K + k;
+            p.keys[slot] = key;
+            p.probs[slot] = pr;
+          }
+        }
+        if constexpr (MODE == kFdaFallback) {
+#pragma unroll
+          for (int cn = 0; cn < 4; ++cn) {
+            if (!(tp.valid & (1u << cn)) || !active) continue;
+            const float w = pr * tp.w[cn];
+            const size_t e0 = ((((size_t)b * p.N + lv.start + (size_t)(tp.y0 + (cn >> 1)) * lv.W + tp.x0 + (cn & 1)) * p.G + g) * p.D) + chunk * CPT;
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) atomic_add_element<Tag>(p.grad_value, e0 + c, go[c] * w);
+          }
+          continue;
+        }
         typename pack::raw_t raw[4];
 #pragma unroll
         for (int cn = 0; cn < 4; ++cn) raw[cn] = buffer_load<pack::kBytes>(value, tp.off[cn]);
@@ -161,11 +199,13 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
 #pragma unroll
           for (int c = 0; c < CPT; ++c) d = fmaf(v[c], go[c], d);
           dots[cn] = d;
-          const float w = pr * tp.w[cn];
-          const uint32_t aoff = (tp.off[cn] == kDropOffset) ? kDropOffset : tp.off[cn] * (4 / Tag::kBytes);
+          if constexpr (MODE == kFdaFull) {
+            const float w = pr * tp.w[cn];
+            const uint32_t aoff = (tp.off[cn] == kDropOffset) ? kDropOffset : tp.off[cn] * (4 / Tag::kBytes);
 #pragma unroll
-          for (int c = 0; c < CPT; ++c)
-            __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(go[c] * w, gacc, aoff + 4 * c, 0, 0);
+            for (int c = 0; c < CPT; ++c)
+              __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(go[c] * w, gacc, aoff + 4 * c, 0, 0);
+          }
         }
         const float hy = 1.f - tp.ly, hx = 1.f - tp.lx;
         float gx = hy * (dots[1] - dots[0]) + tp.ly * (dots[3] - dots[2]);
@@ -182,22 +222,36 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
         dot_rg = fmaf(pr, gz, dot_rg);
       }
     }
-    if (chunk == 0) {
+    if (MODE != kFdaFallback && chunk == 0) {
       for (int t = 0; t < LK; ++t) {
         const float pr = __expf(s[2 * LK + t] - mx) * inv;
         gs[2 * LK + t] = pr * (gs[2 * LK + t] - dot_rg);
       }
     }
   }
+  if constexpr (MODE == kFdaFallback) return;
+  if constexpr (MODE == kFdaNoScatter) {
+    // fold the statistic in LDS first: same-address global atomics retire slowly
+    __shared__ uint32_t s_stat;
+    if (threadIdx.x == 0) s_stat = 0u;
+    __syncthreads();
+    go_max = wave_max_u32(go_max);
+    if ((threadIdx.x & (kWave - 1)) == 0) atomicMax(&s_stat, go_max);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      uint32_t *dst = &p.state->go_max_bits;
+      if (s_stat > __hip_atomic_load(dst, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(dst, s_stat);
+    }
+  }
   __syncthreads();
   unstage_rows_from_lds<Tag>((char *)p.grad_sla + (size_t)row0 * p.G * row_len * Tag::kBytes, s_grad, span, vec16);
 }
 
-template <typename Tag, int CPT, bool BWD>
+template <typename Tag, int CPT, int MODE>      // MODE -1: forward
 hipError_t launch_k(const FdaLaunch &p, hipStream_t stream, dim3 grid, dim3 block, size_t lds) {
 #define FDA_LAUNCH(KT)                                                                                     \
   do {                                                                                                     \
-    if (BWD) hipLaunchKernelGGL((fda_backward_kernel<Tag, CPT, KT>), grid, block, lds, stream, p);         \
+    if constexpr (MODE >= 0) hipLaunchKernelGGL((fda_backward_kernel<Tag, CPT, KT, MODE>), grid, block, lds, stream, p); \
     else hipLaunchKernelGGL((fda_forward_kernel<Tag, CPT, KT>), grid, block, lds, stream, p);              \
   } while (0)
   if (p.K == 4) FDA_LAUNCH(4);
@@ -207,13 +261,13 @@ hipError_t launch_k(const FdaLaunch &p, hipStream_t stream, dim3 grid, dim3 bloc
   return hipGetLastError();
 }
 
-template <typename Tag, bool BWD>
+template <typename Tag, int MODE>
 hipError_t launch_by_cpt(const FdaLaunch &p, hipStream_t stream) {
   const dim3 grid((p.n_row + p.nq_block - 1) / p.nq_block), block(kBlockThreads);
-  const size_t lds = BWD ? fda_backward_lds_bytes(p) : fda_forward_lds_bytes(p);
+  const size_t lds = MODE >= 0 ? fda_backward_lds_bytes(p) : fda_forward_lds_bytes(p);
 #define FDA_CASE(N)                                                                       \
   case N:                                                                                 \
-    if constexpr (N * Tag::kBytes <= 16) return launch_k<Tag, N, BWD>(p, stream, grid, block, lds); \
+    if constexpr (N * Tag::kBytes <= 16) return launch_k<Tag, N, MODE>(p, stream, grid, block, lds); \
     break;
   switch (p.lanes.cpt) {
     FDA_CASE(1) FDA_CASE(2) FDA_CASE(4) FDA_CASE(8)
@@ -222,11 +276,11 @@ hipError_t launch_by_cpt(const FdaLaunch &p, hipStream_t stream) {
   return hipErrorInvalidValue;
 }
 
-template <bool BWD> hipError_t launch_by_dtype(int dtype, const FdaLaunch &p, hipStream_t stream) {
+template <int MODE> hipError_t launch_by_dtype(int dtype, const FdaLaunch &p, hipStream_t stream) {
   switch (dtype) {
-    case F32::kCode: return launch_by_cpt<F32, BWD>(p, stream);
-    case F16::kCode: return launch_by_cpt<F16, BWD>(p, stream);
-    case BF16::kCode: return launch_by_cpt<BF16, BWD>(p, stream);
+    case F32::kCode: return launch_by_cpt<F32, MODE>(p, stream);
+    case F16::kCode: return launch_by_cpt<F16, MODE>(p, stream);
+    case BF16::kCode: return launch_by_cpt<BF16, MODE>(p, stream);
   }
   return hipErrorInvalidValue;
 }
@@ -239,10 +293,15 @@ size_t fda_forward_lds_bytes(const FdaLaunch &p) {
 size_t fda_backward_lds_bytes(const FdaLaunch &p) { return 2 * fda_forward_lds_bytes(p); }
 
 hipError_t launch_fda_forward(int dtype, const FdaLaunch &p, hipStream_t stream) {
-  return launch_by_dtype<false>(dtype, p, stream);
+  return launch_by_dtype<-1>(dtype, p, stream);
 }
-hipError_t launch_fda_backward(int dtype, const FdaLaunch &p, hipStream_t stream) {
-  return launch_by_dtype<true>(dtype, p, stream);
+hipError_t launch_fda_backward(int dtype, const FdaLaunch &p, int mode, hipStream_t stream) {
+  switch (mode) {
+    case kFdaFull: return launch_by_dtype<kFdaFull>(dtype, p, stream);
+    case kFdaNoScatter: return launch_by_dtype<kFdaNoScatter>(dtype, p, stream);
+    case kFdaFallback: return launch_by_dtype<kFdaFallback>(dtype, p, stream);
+  }
+  return hipErrorInvalidValue;
 }
 
 }  // namespace dcn

@@ -84,7 +84,38 @@ struct FdaLaunch {
   int Q, N, G, D, L, K;
   int nq_block;             // queries per workgroup
   LaneMap lanes;
+  // tiled grad_value path
+  void *grad_value;         // [n_img, N, G, D] in the tensor dtype
+  GradState *state;         // go_max_bits only
+  uint32_t *keys;           // [n_img, G, L, Q, K] one key per sampling point
+  float *probs;             // same layout: softmax probability of the point
+  int n_img;
+  int fix_bits;             // fractional bits of the fixed-point accumulators
 };
+
+// Key of a sampling point: (y0 + 1) << 16 | (x0 + 1) for the integer position (y0, x0) of its first
+// corner, y0 in [-1, H-1]; two reserved values for a point outside its level and for a level too
+// large for 16-bit fields (the consumer then recomputes the position).
+constexpr uint32_t kFdaKeyOutside = 0xfffeffffu;
+constexpr uint32_t kFdaKeySaturated = 0xffffffffu;
+constexpr int kFdaKeyFieldMax = 0xfff0;
+
+enum FdaBackwardMode {
+  kFdaFull = 0,        // grad_sampling_loc_attn + fp32 atomic scatter of grad_value (any head width)
+  kFdaNoScatter = 1,   // grad_sampling_loc_attn + keys + max |grad_out|, no scatter
+  kFdaFallback = 2,    // scatter with atomics in the tensor dtype, only when max |grad_out| is not finite
+};
+
+// Accumulator channels per cell (head width rounded up to 8, 16, 32 or 64) and cells per tile of the
+// tiled flash-attention grad_value kernel.
+__host__ __device__ inline int fda_padded_channels(int D) {
+  const int c = (D + 7) / 8;
+  return (c <= 2 ? c : (c <= 4 ? 4 : 8)) * 8;
+}
+__host__ __device__ inline int fda_tile_cells(int D) {
+  const int cells = 8192 / fda_padded_channels(D);
+  return cells < 256 ? cells : 256;
+}
 
 // Each returns hipSuccess or the launch error.  dtype: 0 fp32, 1 fp16, 2 bf16.
 hipError_t launch_dcnv4_forward(int dtype, const DcnLaunch &p, hipStream_t stream);
@@ -95,7 +126,9 @@ hipError_t launch_dcnv4_forward_tiled(int dtype, const DcnLaunch &p, hipStream_t
 hipError_t launch_dcnv4_offset_mask_grad_tiled(int dtype, const DcnLaunch &p, hipStream_t stream);
 size_t dcnv4_tiled_gather_lds_bytes(const DcnLaunch &p, int elem_bytes);
 hipError_t launch_fda_forward(int dtype, const FdaLaunch &p, hipStream_t stream);
-hipError_t launch_fda_backward(int dtype, const FdaLaunch &p, hipStream_t stream);
+hipError_t launch_fda_backward(int dtype, const FdaLaunch &p, int mode, hipStream_t stream);
+hipError_t launch_fda_grad_value(int dtype, const FdaLaunch &p, hipStream_t stream);
+size_t fda_grad_value_lds_bytes(const FdaLaunch &p);
 
 size_t dcnv4_forward_lds_bytes(const DcnLaunch &p);
 size_t dcnv4_backward_lds_bytes(const DcnLaunch &p);

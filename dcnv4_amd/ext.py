@@ -141,7 +141,8 @@ def flash_deform_attn_backward(value, spatial_shapes, level_start_index, samplin
     with torch.cuda.device(value.device):
         grad_value = torch.empty_like(value)
         grad_sla = torch.empty_like(sampling_loc_attn)
-        ws_bytes = _L.flash_deform_attn_gfx950_backward_workspace_bytes(code, batch, spatial_size, num_heads, channels)
+        ws_bytes = _L.flash_deform_attn_gfx950_backward_workspace_bytes(code, batch, spatial_size, num_heads, channels,
+                                                                        num_levels, num_query, int(K))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=value.device) if ws_bytes else None
         _lib.check(_L.flash_deform_attn_gfx950_backward(
             value.data_ptr(), spatial_shapes.data_ptr(), level_start_index.data_ptr(), sampling_loc_attn.data_ptr(),

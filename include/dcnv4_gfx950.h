@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define DCNV4_GFX950_ABI_VERSION 1
+#define DCNV4_GFX950_ABI_VERSION 2
 
 #define DCNV4_DTYPE_F32 0
 #define DCNV4_DTYPE_F16 1
@@ -106,8 +106,17 @@ int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_s
                                      int num_points, int im2col_step, int d_stride,
                                      int block_thread, void *stream);
 
+/*
+ * Bytes of device scratch flash_deform_attn_gfx950_backward needs for this problem (16-byte aligned;
+ * contents need no initialisation).  Head widths that are multiples of 8 up to 32 take 8 bytes
+ * per sampling point (a key and a probability) plus a small state block; other widths take an fp32 image of value for 16-bit
+ * tensors.  The reference allocates its fp32 gradient buffers itself
+ * (DCNv4_op/src/cuda/flash_deform_attn_cuda.cu:127-133).
+ */
 size_t flash_deform_attn_gfx950_backward_workspace_bytes(int dtype, int batch, int spatial_size,
-                                                         int num_heads, int head_channels);
+                                                         int num_heads, int head_channels,
+                                                         int num_levels, int num_query,
+                                                         int num_points);
 
 /*
  * Flash deformable attention backward.  Replaces flash_deform_attn_backward /

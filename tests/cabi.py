@@ -60,7 +60,7 @@ def fda_backward(value, shapes, starts, sla, go, K, im2col_step=64, d_stride=0, 
     Q = sla.shape[1]
     gv = torch.full_like(value, float("nan"))
     gs = torch.full_like(sla, float("nan"))
-    nbytes = L.flash_deform_attn_gfx950_backward_workspace_bytes(CODES[value.dtype], B, N, G, D)
+    nbytes = L.flash_deform_attn_gfx950_backward_workspace_bytes(CODES[value.dtype], B, N, G, D, shapes.shape[0], Q, K)
     ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=value.device)
     rc_ = L.flash_deform_attn_gfx950_backward(value.data_ptr(), shapes.data_ptr(), starts.data_ptr(), sla.data_ptr(),
                                               go.data_ptr(), gv.data_ptr(), gs.data_ptr(), ws.data_ptr(), nbytes,

@@ -195,6 +195,58 @@ def test_flash_deform_attn_forward_and_backward_match_oracle(oracle, name, dtype
     cabi.assert_close(gs, wgs, *GRAD_TOL[dtype], what="grad_sampling_loc_attn")
 
 
+FDA_PATH_CASES = {
+    # head width 24 pads to 32 accumulator channels in the tiled grad_value kernel
+    "d24_three_levels": (2, [(12, 20), (6, 10), (3, 5)], 3, 24, 4, 90, (-0.2, 1.2)),
+    # 6000 queries x 8 points on a 3x3 level: every tile collects far more points than one batch, the list is flushed repeatedly
+    "crowded_small_level": (1, [(3, 3), (20, 17)], 2, 16, 8, 6000, (0.0, 1.0)),
+    # a level wider than the 16-bit fields of a key: the scan recomputes those positions
+    "level_wider_than_a_key": (1, [(1, 65530), (2, 3)], 1, 8, 4, 300, (0.0, 1.0)),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("scatter", ["tiled", "atomic"])
+@pytest.mark.parametrize("name", ["detr_small_4lvl_k4", "five_levels", "k8_one_level"] + list(FDA_PATH_CASES))
+def test_flash_deform_attn_backward_paths_match_oracle(oracle, monkeypatch, name, scatter, dtype):
+    if scatter == "atomic":
+        monkeypatch.setenv("DCNV4_GFX950_FDA_SCATTER", "atomic")
+    if name == "level_wider_than_a_key" and dtype != torch.float32:
+        pytest.skip("location gradients scale with the level width (65530) and overflow the 16-bit types")
+    B, shapes, G, D, K, Q, (lo, hi) = {**FDA_CASES, **FDA_PATH_CASES}[name]
+    print(f"case {name} scatter {scatter} dtype {dtype}", flush=True)
+    v, shp, st, sla, go = make_fda_inputs(B, shapes, G, D, K, Q, seed=zlib.crc32((name + scatter).encode()) % 1000, dtype=dtype,
+                                          loc_lo=lo, loc_hi=hi)
+    wgv, wgs = oracle.flash_deform_attn_backward(cabi.f64(v), shp.numpy(), st.numpy(), cabi.f64(sla), cabi.f64(go), K, coord_f32=True)
+    gv, gs = cabi.fda_backward(v.cuda(), shp.cuda(), st.cuda(), sla.cuda(), go.cuda(), K)
+    torch.cuda.synchronize()
+    rtol, atol = GRAD_TOL[dtype]
+    if name == "crowded_small_level":       # thousands of terms per cell: the tolerance scales with the sum's magnitude
+        atol = atol * float(np.abs(wgv).max())
+    cabi.assert_close(gv, wgv, rtol, atol, what="grad_value")
+    cabi.assert_close(gs, wgs, *GRAD_TOL[dtype], what="grad_sampling_loc_attn")
+
+
+def test_flash_deform_attn_backward_is_bit_reproducible_and_handles_non_finite_grad_out(oracle):
+    B, shapes, G, D, K, Q, (lo, hi) = FDA_CASES["detr_small_4lvl_k4"]
+    v, shp, st, sla, go = make_fda_inputs(B, shapes, G, D, K, Q, seed=4, dtype=torch.float16, loc_lo=lo, loc_hi=hi)
+    args = (v.cuda(), shp.cuda(), st.cuda(), sla.cuda())
+    first = cabi.fda_backward(*args, go.cuda(), K)
+    for _ in range(3):
+        again = cabi.fda_backward(*args, go.cuda(), K)
+        assert torch.equal(first[0], again[0]) and torch.equal(first[1], again[1])
+    # NaN / Inf in grad_out: the fixed-point path steps aside, the result still matches the oracle's pattern
+    go32 = go.float()
+    go32[0, 3, 5] = float("nan")
+    go32[1, 7, 40] = float("inf")
+    wgv, _ = oracle.flash_deform_attn_backward(cabi.f64(v), shp.numpy(), st.numpy(), cabi.f64(sla), cabi.f64(go32.half()), K, coord_f32=True)
+    gv, _ = cabi.fda_backward(*args, go32.half().cuda(), K)
+    gv = cabi.f64(gv)
+    assert np.array_equal(np.isnan(gv), np.isnan(wgv))
+    ok = np.isfinite(wgv)
+    np.testing.assert_allclose(gv[ok], wgv[ok], rtol=2e-2, atol=2e-2)
+
+
 def test_c_abi_rejects_bad_arguments():
     from dcnv4_amd import _lib
     v = torch.zeros(2, 4, 4, 16, device="cuda")
