@@ -541,7 +541,8 @@ size_t flash_deform_attn_gfx950_backward_workspace_bytes(int dtype, int batch, i
   size_t need = 0;
   if (elem_bytes(dtype) == 2) need = round16((size_t)batch * spatial_size * num_heads * head_channels * sizeof(float));
   if (fda_tiled_shape(head_channels, num_levels, num_query, num_points))
-    need = std::max(need, kStateBytes + 2 * round16((size_t)batch * num_heads * num_levels * num_query * num_points * sizeof(uint32_t)));
+    need = std::max(need, kStateBytes + round16((size_t)batch * num_heads * num_levels * fda_key_stride(num_query, num_points) * 2) +
+                              round16((size_t)batch * num_heads * num_levels * fda_key_stride(num_query, num_points) * 4));
   return need;
 }
 
@@ -553,7 +554,11 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
                                       int num_query, int num_points, int im2col_step, int d_stride,
                                       int block_thread, void *stream) {
   FdaProblem pr;
-  const bool tiled = fda_tiled_shape(head_channels, num_levels, num_query, num_points) && fda_tiled_enabled();
+  // the tiled grad_value kernel addresses one image's sampling_loc_attn and grad_out with 32-bit byte offsets
+  const unsigned long long row_bytes = (unsigned long long)std::max(num_heads, 1) *
+                                       std::max(3 * num_levels * num_points, head_channels) * 4ull;
+  const bool tiled = fda_tiled_shape(head_channels, num_levels, num_query, num_points) && fda_tiled_enabled() &&
+                     (unsigned long long)num_query * row_bytes < (1ull << 31);
   // the tiled path gathers only: 16-byte lanes; the atomic path wants one channel per lane
   if (int rc = fda_prepare(&pr, true, !tiled, dtype, batch, spatial_size, num_heads, head_channels, num_levels, num_query,
                            num_points, im2col_step, d_stride, block_thread))
@@ -574,15 +579,15 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
     // pass 0: grad_sampling_loc_attn, keys and max |grad_out|; pass 1: tiled grad_value; pass 2: fallback
     FdaLaunch base = pr.launch;
     base.state = static_cast<GradState *>(workspace);
-    const size_t key_bytes = round16((size_t)batch * num_heads * num_levels * num_query * num_points * sizeof(uint32_t));
-    uint32_t *keys = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + kStateBytes);
+    const size_t img_keys = (size_t)num_heads * num_levels * fda_key_stride(num_query, num_points);
+    const size_t key_bytes = round16((size_t)batch * img_keys * sizeof(uint16_t));
+    uint16_t *keys = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + kStateBytes);
     float *probs = reinterpret_cast<float *>(static_cast<char *>(workspace) + kStateBytes + key_bytes);
     // every term is grad_out * (probability * bilinear weight <= 1); at most Q * K of them meet in one cell
     base.fix_bits = 62 - ceil_log2((int)std::min<long long>((long long)num_query * num_points, 1 << 30));
     if (pr.s == 2) base.fix_bits = std::min(base.fix_bits, 30);
     hipLaunchKernelGGL(init_state_kernel, dim3(1), dim3(64), 0, st, base.state);
     if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);
-    const size_t img_keys = (size_t)num_heads * num_levels * num_query * num_points;
     for (int pass = 0; pass < 3; ++pass) {
       for (int b0 = 0; b0 < batch; b0 += per) {
         const int nb = std::min(per, batch - b0);

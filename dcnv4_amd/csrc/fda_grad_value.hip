@@ -6,10 +6,10 @@
 // window around the query to exploit; instead a workgroup OWNS a tile of one level of one
 // (image, head) and finds its contributions by scanning:
 //
-//   * the grad_sampling_loc_attn kernel, which runs first, leaves one 32-bit key (integer position of
+//   * the grad_sampling_loc_attn kernel, which runs first, leaves one 16-bit key (integer position of
 //     the first corner, or "outside") and the softmax probability per sampling point, both laid out
 //     [image][head][level][query][point], and the maximum of |grad_out| in GradState;
-//   * scan: the workgroup streams the keys of its (image, head, level) - coalesced dwords, a handful
+//   * scan: the workgroup streams the keys of its (image, head, level) - coalesced dwords of two keys, a handful
 //     of instructions per point - and appends the points whose 2x2 corner block touches its tile
 //     to a list in LDS;
 //   * apply, in batches of 256 listed points: one lane per point recomputes the position from
@@ -34,10 +34,10 @@ namespace {
 constexpr int kThreads = 1024;
 constexpr int kRowLanes = 8;                 // lanes that apply one listed point
 constexpr int kBatch = 256;                  // listed points applied between two barriers
-constexpr int kScanPerLane = 16;             // keys per lane and scan step (one memory latency per step)
-constexpr int kRoundKeys = 4;                // keys per lane tested between two looks at the list's fill
+constexpr int kScanPerLane = 16;             // dwords (two keys each) per lane and scan step: one memory latency per step
+constexpr int kRoundKeys = 4;                // dwords per lane tested between two looks at the list's fill
 constexpr int kScanStep = kThreads * kScanPerLane;
-constexpr int kListCap = 3 * kRoundKeys * kThreads;      // flushed when another round might not fit
+constexpr int kListCap = 3 * kRoundKeys * kThreads;      // flushed when another round (2 * kRoundKeys points per lane) might not fit
 constexpr int kCellBitsF = 9;
 
 struct LevelPlan {
@@ -134,7 +134,9 @@ __global__ void __launch_bounds__(kThreads) fda_grad_value_kernel(const FdaLaunc
     for (int i = tid; i < n_acc; i += kThreads) acc[i] = 0ull;
     __syncthreads();
 
-    const uint32_t *keys = p.keys + ((size_t)(b * p.G + g) * p.L + l) * QK;
+    const size_t QKp = fda_key_stride(p.Q, p.K);
+    const uint32_t *keys = reinterpret_cast<const uint32_t *>(p.keys + ((size_t)(b * p.G + g) * p.L + l) * QKp);      // two keys per dword
+    const int n_words = (int)(QKp / 2);
     const size_t sla_bg = ((size_t)b * p.Q * p.G + g) * 3 * LK;       // + q * G * 3LK
     const size_t go_bg = ((size_t)b * p.Q * p.G + g) * D;             // + q * G * D
 
@@ -151,48 +153,52 @@ __global__ void __launch_bounds__(kThreads) fda_grad_value_kernel(const FdaLaunc
     // ---- apply the first `n` listed points, in batches.  What a batch needs from memory (position,
     // probability, grad_out rows) is requested one batch ahead, so the loads fly while the previous
     // batch is applied.
-    const float *probs = p.probs + ((size_t)(b * p.G + g) * p.L + l) * QK;
+    const float *probs = p.probs + ((size_t)(b * p.G + g) * p.L + l) * QKp;
     constexpr int kParts = DP / 4;                           // 4-channel pieces of a grad_out row
     constexpr int kGoLoads = kBatch * kParts / kThreads;     // pieces per lane and batch (DP = 32: 2)
     static_assert(kBatch * kParts % kThreads == 0 || kBatch * kParts < kThreads, "grad_out pieces divide over the lanes");
     constexpr int kGoPerLane = kGoLoads > 0 ? kGoLoads : 1;
+    // Everything is requested through range-checked buffer loads of raw words: no branches around
+    // the loads, so they all fly together, and nothing is converted before it is needed.
+    typedef typename RawWord<2 * Tag::kBytes>::type xy_t;      // (x, y) of a point are adjacent
+    typedef typename RawWord<4 * Tag::kBytes>::type go4_t;     // 4 channels of grad_out
+    const __amdgpu_buffer_rsrc_t sla_rs = make_rsrc(reinterpret_cast<const elem_t *>(p.sla) + sla_bg,
+                                                    (uint32_t)((size_t)p.Q * p.G * 3 * LK * Tag::kBytes));
+    const __amdgpu_buffer_rsrc_t go_rs = make_rsrc(reinterpret_cast<const elem_t *>(p.grad_out) + go_bg,
+                                                   (uint32_t)((size_t)p.Q * p.G * D * Tag::kBytes));
+    const __amdgpu_buffer_rsrc_t pr_rs = make_rsrc(probs, (uint32_t)QK * 4u);
     struct Ahead {
-      float x, y, pr;                  // lanes < batch size: their point
-      float go[kGoPerLane][4];
+      xy_t xy;                         // lanes < batch size: their point
+      uint32_t pr;
+      go4_t go[kGoPerLane];
     };
     auto fetch = [&](uint32_t b0, int nb) {
       Ahead a;
-      a.x = a.y = a.pr = 0.f;
-      if (tid < nb) {
-        const uint32_t pt = s_list[b0 + tid];
+      {
+        const uint32_t pt = s_list[b0 + min(tid, max(nb - 1, 0))];
         const uint32_t q = pt / (uint32_t)p.K;
         const int t = l * p.K + (int)(pt - q * p.K);
-        const size_t row = sla_bg + (size_t)q * p.G * 3 * LK;
-        a.x = elem_at<Tag>(p.sla, row + 2 * t);
-        a.y = elem_at<Tag>(p.sla, row + 2 * t + 1);
-        a.pr = probs[pt];
+        const bool live = tid < nb;
+        a.xy = buffer_load<2 * Tag::kBytes>(sla_rs, live ? (q * (uint32_t)(p.G * 3 * LK) + 2u * t) * Tag::kBytes : kDropOffset);
+        a.pr = buffer_load<4>(pr_rs, live ? pt * 4u : kDropOffset);
       }
 #pragma unroll
       for (int u = 0; u < kGoPerLane; ++u) {
         const int i = tid + u * kThreads, h = i / kParts, part = i - h * kParts;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) a.go[u][j] = 0.f;
-        if (h < nb && i < kBatch * kParts) {
-          const uint32_t q = s_list[b0 + h] / (uint32_t)p.K;
-          const size_t src = go_bg + (size_t)q * p.G * D + 4 * part;
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            if (4 * part + j < D) a.go[u][j] = elem_at<Tag>(p.grad_out, src + j);
-        }
+        const bool live = h < nb && i < kBatch * kParts && 4 * part < D;
+        const uint32_t q = s_list[b0 + min(h, max(nb - 1, 0))] / (uint32_t)p.K;
+        a.go[u] = buffer_load<4 * Tag::kBytes>(go_rs, live ? (q * (uint32_t)(p.G * D) + 4u * part) * Tag::kBytes : kDropOffset);
       }
       return a;
     };
     auto park = [&](const Ahead &a, int nb) {
       if (tid < nb) {          // one lane per point: corner weights and accumulator cells
-        const float x = sub_rn(mul_rn(a.x, (float)lp.W), 0.5f);       // flash_deform_im2col_cuda.cuh:188-189
-        const float y = sub_rn(mul_rn(a.y, (float)lp.H), 0.5f);
+        float xy[2];
+        Pack<Tag, 2>::decode(a.xy, xy);
+        const float x = sub_rn(mul_rn(xy[0], (float)lp.W), 0.5f);       // flash_deform_im2col_cuda.cuh:188-189
+        const float y = sub_rn(mul_rn(xy[1], (float)lp.H), 0.5f);
         const Tap tp = make_tap(y, x, lp.H, lp.W, 0u, 0u);
-        const float ps = ldexpf(a.pr, p.fix_bits);
+        const float ps = ldexpf(__builtin_bit_cast(float, a.pr), p.fix_bits);
         const int ly = tp.y0 - ty0, lx = tp.x0 - tx0;
         uint32_t cells[4];
         float w[4];
@@ -207,11 +213,14 @@ __global__ void __launch_bounds__(kThreads) fda_grad_value_kernel(const FdaLaunc
         rec_meta[tid] = u32x2{cells[0] | (cells[1] << kCellBitsF) | (cells[2] << (2 * kCellBitsF)), cells[3]};
       }
 #pragma unroll
-      for (int u = 0; u < kGoPerLane; ++u) {      // grad_out rows, normalised to [-1, 1]
+      for (int u = 0; u < kGoPerLane; ++u) {      // grad_out rows, normalised to [-1, 1] (zeros past the head width)
         const int i = tid + u * kThreads, h = i / kParts, part = i - h * kParts;
-        if (h < nb && i < kBatch * kParts)
+        if (h < nb && i < kBatch * kParts) {
+          float g4[4];
+          Pack<Tag, 4>::decode(a.go[u], g4);
           *reinterpret_cast<f32x4 *>(s_go + h * DP + 4 * part) =
-              f32x4{ldexpf(a.go[u][0], -e_go), ldexpf(a.go[u][1], -e_go), ldexpf(a.go[u][2], -e_go), ldexpf(a.go[u][3], -e_go)};
+              f32x4{ldexpf(g4[0], -e_go), ldexpf(g4[1], -e_go), ldexpf(g4[2], -e_go), ldexpf(g4[3], -e_go)};
+        }
       }
     };
     auto apply_list = [&](uint32_t n) {
@@ -252,54 +261,66 @@ __global__ void __launch_bounds__(kThreads) fda_grad_value_kernel(const FdaLaunc
 
     // ---- scan the keys of (image, head, level); flush the list whenever another step might overflow it
     if (finite && gmax != 0u) {
-      // A step = kScanPerLane keys per lane, loaded in one go (and one step ahead) so that the memory
-      // latency is paid once per step; the step is then tested in rounds of kRoundKeys keys per lane,
-      // few enough that the list can always take a whole round.
+      // A step = kScanPerLane dwords (two keys each) per lane, loaded in one go (and one step ahead) so that
+      // the memory latency is paid once per step; the step is then tested in rounds of kRoundKeys dwords per
+      // lane, few enough that the list can always take a whole round.
       auto load_keys = [&](int base, uint32_t (&key)[kScanPerLane]) {
 #pragma unroll
         for (int u = 0; u < kScanPerLane; ++u) {
           const int i = base + u * kThreads + tid;
-          key[u] = i < QK ? keys[i] : kFdaKeyOutside;
+          key[u] = keys[min(i, n_words - 1)];             // points past the end are masked when tested
         }
       };
       uint32_t key[kScanPerLane], key_next[kScanPerLane];
       load_keys(0, key_next);
-      for (int base = 0; base < QK; base += kScanStep) {
+      for (int base = 0; base < n_words; base += kScanStep) {
 #pragma unroll
         for (int u = 0; u < kScanPerLane; ++u) key[u] = key_next[u];
-        if (base + kScanStep < QK) load_keys(base + kScanStep, key_next);      // in flight while this step is tested
+        if (base + kScanStep < n_words) load_keys(base + kScanStep, key_next);      // in flight while this step is tested
         // a real loop (the flush below must not be replicated per round): each round tests key[0..kRoundKeys)
         // and then shifts the rest of the step's keys down
 #pragma unroll 1
         for (int r = 0; r < kScanPerLane / kRoundKeys; ++r) {
+          // test the round's points first, then reserve list slots for all of them with one LDS atomic per wave
+          uint64_t masks[2 * kRoundKeys];
+          uint32_t total = 0;
 #pragma unroll
-          for (int uu = 0; uu < kRoundKeys; ++uu) {
-            const int u = uu;
-            const uint32_t pt = (uint32_t)(base + (r * kRoundKeys + uu) * kThreads + tid);
+          for (int uu = 0; uu < 2 * kRoundKeys; ++uu) {
+            const uint32_t k16 = (key[uu >> 1] >> (16 * (uu & 1))) & 0xffffu;
+            const uint32_t pt = 2u * (uint32_t)(base + (r * kRoundKeys + (uu >> 1)) * kThreads + tid) + (uu & 1);
             bool hit = false;
-            if (key[u] == kFdaKeySaturated) {                   // level wider than the key can hold: exact test
+            if (pt >= (uint32_t)QK) {
+            } else if (k16 == kFdaKeySaturated) {                   // position beyond the key's fields: exact test
               float y, x;
               uint32_t q;
               position(pt, y, x, q);
               const Tap tp = make_tap(y, x, lp.H, lp.W, 0u, 0u);
               hit = tp.valid != 0 && tp.y0 + 1 >= ty0 && tp.y0 < ty0 + th && tp.x0 + 1 >= tx0 && tp.x0 < tx0 + tw;
-            } else if (key[u] != kFdaKeyOutside) {
-              // key = (y0 + 1) << 16 | (x0 + 1); the corner block {x0, x0 + 1} meets [tx0, tx0 + tw) iff 0 <= x0 + 1 - tx0 <= tw
-              hit = (uint32_t)((int)(key[u] & 0xffffu) - tx0) <= (uint32_t)tw && (uint32_t)((int)(key[u] >> 16) - ty0) <= (uint32_t)th;
+            } else if (k16 != kFdaKeyOutside) {
+              // key = (y0 + 1) << 8 | (x0 + 1); the corner block {x0, x0 + 1} meets [tx0, tx0 + tw) iff 0 <= x0 + 1 - tx0 <= tw
+              hit = (uint32_t)((int)(k16 & 0xffu) - tx0) <= (uint32_t)tw && (uint32_t)((int)(k16 >> 8) - ty0) <= (uint32_t)th;
             }
-            const uint64_t mask = __builtin_amdgcn_ballot_w64(hit);
-            if (mask != 0) {
-              uint32_t slot0 = 0;
-              if (lane == 0) slot0 = atomicAdd(&s_count, (uint32_t)__builtin_popcountll(mask));
-              slot0 = __builtin_amdgcn_readfirstlane(slot0);
-              if (hit)
+            masks[uu] = __builtin_amdgcn_ballot_w64(hit);
+            total += (uint32_t)__builtin_popcountll(masks[uu]);
+          }
+          if (total != 0) {
+            uint32_t slot0 = 0;
+            if (lane == 0) slot0 = atomicAdd(&s_count, total);
+            slot0 = __builtin_amdgcn_readfirstlane(slot0);
+#pragma unroll
+            for (int uu = 0; uu < 2 * kRoundKeys; ++uu) {
+              const uint64_t mask = masks[uu];
+              if ((mask >> lane) & 1) {
+                const uint32_t pt = 2u * (uint32_t)(base + (r * kRoundKeys + (uu >> 1)) * kThreads + tid) + (uu & 1);
                 s_list[slot0 + __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u))] = pt;
+              }
+              slot0 += (uint32_t)__builtin_popcountll(mask);
             }
           }
           __syncthreads();
           const uint32_t n = s_count;
-          const bool last = base + kScanStep >= QK && r == kScanPerLane / kRoundKeys - 1;
-          if (n > (uint32_t)(kListCap - kRoundKeys * kThreads) || last) {
+          const bool last = base + kScanStep >= n_words && r == kScanPerLane / kRoundKeys - 1;
+          if (n > (uint32_t)(kListCap - 2 * kRoundKeys * kThreads) || last) {
             __syncthreads();                // everyone has read the count
             if (tid == 0) s_count = 0u;
             apply_list(n);                  // ends with a barrier

@@ -170,9 +170,9 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
             uint32_t key = kFdaKeyOutside;
             if (tp.valid != 0)
               key = (tp.y0 + 1 >= kFdaKeyFieldMax || tp.x0 + 1 >= kFdaKeyFieldMax) ? kFdaKeySaturated
-                                                                                  : ((uint32_t)(tp.y0 + 1) << 16) | (uint32_t)(tp.x0 + 1);
-            const size_t slot = ((((size_t)b_local * p.G + g) * p.L + l) * p.Q + q) * K + k;
-            p.keys[slot] = key;
+                                                                                  : ((uint32_t)(tp.y0 + 1) << 8) | (uint32_t)(tp.x0 + 1);
+            const size_t slot = (((size_t)b_local * p.G + g) * p.L + l) * fda_key_stride(p.Q, K) + (size_t)q * K + k;
+            p.keys[slot] = (uint16_t)key;
             p.probs[slot] = pr;
           }
         }

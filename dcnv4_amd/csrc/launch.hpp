@@ -87,18 +87,19 @@ struct FdaLaunch {
   // tiled grad_value path
   void *grad_value;         // [n_img, N, G, D] in the tensor dtype
   GradState *state;         // go_max_bits only
-  uint32_t *keys;           // [n_img, G, L, Q, K] one key per sampling point
+  uint16_t *keys;           // [n_img, G, L, QKp] one key per sampling point (QKp = Q*K rounded up to even)
   float *probs;             // same layout: softmax probability of the point
   int n_img;
   int fix_bits;             // fractional bits of the fixed-point accumulators
 };
 
-// Key of a sampling point: (y0 + 1) << 16 | (x0 + 1) for the integer position (y0, x0) of its first
-// corner, y0 in [-1, H-1]; two reserved values for a point outside its level and for a level too
-// large for 16-bit fields (the consumer then recomputes the position).
-constexpr uint32_t kFdaKeyOutside = 0xfffeffffu;
-constexpr uint32_t kFdaKeySaturated = 0xffffffffu;
-constexpr int kFdaKeyFieldMax = 0xfff0;
+// Key of a sampling point: (y0 + 1) << 8 | (x0 + 1) for the integer position (y0, x0) of its first
+// corner, y0 in [-1, H-1]; two reserved values for a point outside its level and for a position that
+// does not fit the 8-bit fields (the consumer then recomputes it from sampling_loc_attn).
+constexpr uint32_t kFdaKeyOutside = 0xfeffu;
+constexpr uint32_t kFdaKeySaturated = 0xffffu;
+constexpr int kFdaKeyFieldMax = 0xfe;
+__host__ __device__ inline size_t fda_key_stride(int Q, int K) { return ((size_t)Q * K + 1) & ~size_t(1); }
 
 enum FdaBackwardMode {
   kFdaFull = 0,        // grad_sampling_loc_attn + fp32 atomic scatter of grad_value (any head width)
