@@ -12,6 +12,8 @@
 // Backward: coordinate / modulation partials are summed over the lanes of a (pixel, group) with
 // DPP, parked in LDS and written back as whole rows (padding tail included, so the gradient
 // tensor needs no separate clearing); the value gradient is scattered with fp32 buffer atomics.
+#include <algorithm>
+
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -129,11 +131,18 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
     scatter_all = gmax >= 0x7f800000u || mmax >= 0x7f800000u;
     if (!scatter_all && p.state->reach_needed <= (uint32_t)p.reach) return;
   }
-  const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
-  const int pix0 = (int)blk * p.npix_block;
-  const int npix = min(p.npix_block, p.n_pix - pix0);
+  // The fallback role is launched with a small grid (its usual job is to find out that there is nothing
+  // to do) and strides over the pixel blocks; the other roles own exactly one block.
+  const uint32_t n_blocks = (uint32_t)((p.n_pix + p.npix_block - 1) / p.npix_block);
+  uint32_t block_index = blockIdx.x;
+  int pix0 = 0, npix = 0;
   const bool vec16 = (p.P_pad * Tag::kBytes) % 16 == 0;
   float *s_om = lds, *s_grad = lds + p.npix_block * p.P_pad;
+  uint32_t go_max = 0, mask_max = 0, reach_needed = 0;
+  for (;;) {
+  const uint32_t blk = MODE == kBwdFallback ? block_index : xcd_contiguous_block(block_index, gridDim.x);
+  pix0 = (int)blk * p.npix_block;
+  npix = min(p.npix_block, p.n_pix - pix0);
   stage_rows_to_lds<Tag>(s_om, (const char *)p.offset_mask + (size_t)pix0 * p.P_pad * Tag::kBytes,
                          npix * p.P_pad, vec16);
   if constexpr (MODE != kBwdFallback)
@@ -148,7 +157,6 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
   const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
   const int Kp = p.Kp;
   const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
-  uint32_t go_max = 0, mask_max = 0, reach_needed = 0;
 
   for (int it = threadIdx.x; it < items; it += blockDim.x) {
     const int chunk = it & (width - 1);
@@ -283,7 +291,11 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
       }
     }
   }
-  if constexpr (MODE == kBwdFallback) return;
+  if constexpr (MODE != kBwdFallback) break;
+  block_index += gridDim.x;
+  if (block_index >= n_blocks) return;
+  __syncthreads();        // the staged rows are replaced next
+  }
   if constexpr (MODE == kBwdOffsetMask) {
     // Same-address atomics retire slowly at the memory side: fold the workgroup's statistics in
     // LDS first and only touch the global word when it would actually grow.
@@ -331,7 +343,8 @@ hipError_t launch_bwd_k(const DcnLaunch &p, hipStream_t stream, dim3 grid, dim3 
 // MODE < 0 selects the forward kernel.
 template <typename Tag, int MODE>
 hipError_t launch_by_cpt(const DcnLaunch &p, hipStream_t stream) {
-  const dim3 grid((p.n_pix + p.npix_block - 1) / p.npix_block), block(kBlockThreads);
+  const unsigned n_blocks = (unsigned)((p.n_pix + p.npix_block - 1) / p.npix_block);
+  const dim3 grid(MODE == kBwdFallback ? std::min(n_blocks, 1024u) : n_blocks), block(kBlockThreads);
   const size_t lds = MODE >= 0 ? dcnv4_backward_lds_bytes(p) : dcnv4_forward_lds_bytes(p);
 #define DCN_CASE(N)                                                              \
   case N:                                                                        \
