@@ -199,6 +199,7 @@ constexpr int kTiledGatherThreads = 512;     // launch bound of the tiled gather
 
 bool plan_gather_tiles(DcnLaunch *L, int s) {
   L->gt_h = L->gt_w = L->gt_ng = L->gt_wh = L->gt_ww = 0;
+  L->gt_lpg = 1;
   L->gt_reach = reach_setting();
   if (!tiled_gather_enabled() || L->softmax) return false;
   const int lane_bytes = L->D * s;
@@ -206,6 +207,7 @@ bool plan_gather_tiles(DcnLaunch *L, int s) {
   const int nv = lane_bytes / 16;
   if (nv != 1 && nv != 2 && nv != 4 && nv != 8) return false;
   if (L->Kp > 64) return false;
+  L->gt_lpg = nv >= 4 ? 2 : 1;      // wide groups: two lanes each, for twice the waves per workgroup
   const int Ho = L->Q / L->Wo, Wo = L->Wo, R = L->gt_reach;
   auto even_split = [](int extent, int cap) { const int n = (extent + cap - 1) / cap; return (extent + n - 1) / n; };
   // two workgroups per CU when the window allows it, so that one stages while the other computes
@@ -217,7 +219,7 @@ bool plan_gather_tiles(DcnLaunch *L, int s) {
       L->gt_wh = std::min((L->gt_h - 1) * L->sh + 2 * R + 1, L->H + 2);
       L->gt_ww = std::min((L->gt_w - 1) * L->sw + 2 * R + 1, L->W + 2);
       const int px = L->gt_h * L->gt_w;
-      for (int ng = std::min(L->G, kTiledGatherThreads / px); ng >= 1; --ng) {
+      for (int ng = std::min(L->G, kTiledGatherThreads / (px * L->gt_lpg)); ng >= 1; --ng) {
         // 16-bit tensors: keep the offset_mask slices dword-aligned when the tap count is odd
         if (s == 2 && ((ng * 3 * L->Kp) & 1) && ng > 1) continue;
         L->gt_ng = ng;

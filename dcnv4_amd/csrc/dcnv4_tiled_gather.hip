@@ -10,9 +10,10 @@
 //     pixels, clipped to the image plus a one-pixel ring of zeros) into LDS with coalesced
 //     128-bit loads; cells outside the image come back as zeros from the buffer range check;
 //   * the workgroup's slice of offset_mask is parked in LDS next to it, in the tensor dtype;
-//   * one lane owns all D channels of one (pixel, group): the bilinear set-up is done once per
-//     sampling point instead of once per 16-byte channel chunk, no cross-lane traffic is
-//     needed, and the four corners are read from LDS with ds_read_b128;
+//   * one lane owns all D channels of one (pixel, group) - or half of them when a group is 64 bytes
+//     or wider, which doubles the waves that hide LDS latency: the bilinear set-up is done once
+//     (twice) per sampling point instead of once per 16-byte channel chunk, at most one DPP add
+//     crosses lanes, and the four corners are read from LDS with ds_read_b128;
 //   * a sampling point whose corners leave the window is remembered in a per-lane bit mask and
 //     served afterwards from global memory (the range-checked gather of dcnv4_kernels.hip), so
 //     any offset is handled; with offsets inside the window that code never runs.
@@ -99,7 +100,7 @@ __device__ __forceinline__ void stage_tile(const DcnLaunch &p, const TileGeom &t
     const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
     const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
     const uint32_t img_base = (uint32_t)t.b * (uint32_t)(p.H * p.W) * pix_bytes + (uint32_t)(t.g0 * p.D) * Tag::kBytes;
-    const int ppc = t.ng * NV;                           // 16-byte pieces per cell
+    const int ppc = t.ng * (p.D * Tag::kBytes / 16);     // 16-byte pieces per cell
     const int row_pieces = max(t.ww * ppc, 1);
     const int rpp = max(bd / row_pieces, 1);             // window rows per pass
     const int lanes_pp = min(bd, row_pieces);            // lanes of one row in one pass
@@ -272,17 +273,19 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_forward_tiled_kernel(cons
   stage_tile<Tag, NV>(p, t, s_win, s_om, cell_stride);
   __syncthreads();
 
-  // lane -> (tile pixel, group of the chunk)
-  const int q = fdiv(threadIdx.x, rcp((float)p.gt_ng)), gl = threadIdx.x - q * p.gt_ng;
+  // lane -> (tile pixel, group of the chunk, part): gt_lpg (1 or 2) adjacent lanes share one (pixel, group),
+  // each with NV of its 16-byte vectors
+  const int part = threadIdx.x & (p.gt_lpg - 1), unit = threadIdx.x >> (p.gt_lpg - 1);
+  const int q = fdiv(unit, rcp((float)p.gt_ng)), gl = unit - q * p.gt_ng;
   const int py = fdiv(q, rcp((float)p.gt_w)), px = q - py * p.gt_w;
   if (q >= p.gt_h * p.gt_w || gl >= t.ng || py >= t.th || px >= t.tw) return;
   const int ho = t.oy0 + py, wo = t.ox0 + px;
   const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
   const float x_base = sub_rn((float)(half_w - p.pw + wo * p.sw), mul_rn((float)half_w, p.offset_scale));
   const float y_base = sub_rn((float)(half_h - p.ph + ho * p.sh), mul_rn((float)half_h, p.offset_scale));
-  const elem_t *om = s_om + threadIdx.x * 3 * Kp;
+  const elem_t *om = s_om + unit * 3 * Kp;
   const int zero_base = t.wh * t.ww * cell_stride, row_bytes = t.ww * cell_stride;
-  const int lane_bytes = gl * p.D * Tag::kBytes;
+  const int lane_bytes = gl * p.D * Tag::kBytes + part * NV * 16;
   float acc[NV][EPV];
 #pragma unroll
   for (int v = 0; v < NV; ++v)
@@ -329,7 +332,7 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_forward_tiled_kernel(cons
   // a sampling point whose corners lie outside the staged window: gather from memory instead
   const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
   const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
-  const uint32_t img_base = (uint32_t)t.b * (uint32_t)(p.H * p.W) * pix_bytes + (uint32_t)((t.g0 + gl) * p.D) * Tag::kBytes;
+  const uint32_t img_base = (uint32_t)t.b * (uint32_t)(p.H * p.W) * pix_bytes + (uint32_t)((t.g0 + gl) * p.D) * Tag::kBytes + (uint32_t)(part * NV * 16);
   auto far_tap = [&](int k, int i, int j) {
     float y, x, m;
     position(k, i, j, y, x, m);
@@ -386,7 +389,7 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_forward_tiled_kernel(cons
     }
   }
 
-  char *dst = (char *)p.out + (((size_t)t.b * p.Q + (size_t)ho * p.Wo + wo) * (p.G * p.D) + (t.g0 + gl) * p.D) * Tag::kBytes;
+  char *dst = (char *)p.out + (((size_t)t.b * p.Q + (size_t)ho * p.Wo + wo) * (p.G * p.D) + (t.g0 + gl) * p.D) * Tag::kBytes + part * NV * 16;
 #pragma unroll
   for (int v = 0; v < NV; ++v) *reinterpret_cast<u32x4 *>(dst + 16 * v) = pack::encode(acc[v]);
 }
@@ -414,14 +417,16 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
   if (threadIdx.x < 3) s_stat[threadIdx.x] = 0u;
 
   // lane -> (tile pixel, group of the chunk); its grad_out vector is requested before the staging
-  const int q = fdiv(threadIdx.x, rcp((float)p.gt_ng)), gl = threadIdx.x - q * p.gt_ng;
+  const int part = threadIdx.x & (p.gt_lpg - 1), unit = threadIdx.x >> (p.gt_lpg - 1);
+  const int q = fdiv(unit, rcp((float)p.gt_ng)), gl = unit - q * p.gt_ng;
   const int py = fdiv(q, rcp((float)p.gt_w)), px = q - py * p.gt_w;
   const bool active = q < p.gt_h * p.gt_w && gl < t.ng && py < t.th && px < t.tw;
   const int ho = t.oy0 + py, wo = t.ox0 + px;
   u32x4 go_raw[NV];
   {
     const char *src = (const char *)p.grad_out +
-                      (((size_t)t.b * p.Q + (size_t)(active ? ho * p.Wo + wo : 0)) * (p.G * p.D) + (active ? t.g0 + gl : 0) * p.D) * Tag::kBytes;
+                      (((size_t)t.b * p.Q + (size_t)(active ? ho * p.Wo + wo : 0)) * (p.G * p.D) + (active ? t.g0 + gl : 0) * p.D) * Tag::kBytes +
+                      part * NV * 16;
 #pragma unroll
     for (int v = 0; v < NV; ++v) go_raw[v] = *reinterpret_cast<const u32x4 *>(src + 16 * v);
   }
@@ -441,12 +446,14 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
     const int p0y = half_h - p.ph + ho * p.sh, p0x = half_w - p.pw + wo * p.sw;      // reference point
     const float x_base = sub_rn((float)p0x, mul_rn((float)half_w, p.offset_scale));
     const float y_base = sub_rn((float)p0y, mul_rn((float)half_h, p.offset_scale));
-    elem_t *om = s_om + threadIdx.x * 3 * Kp;
+    elem_t *om = s_om + unit * 3 * Kp;
     const int zero_base = t.wh * t.ww * cell_stride, row_bytes = t.ww * cell_stride;
-    const int lane_bytes = gl * p.D * Tag::kBytes;
+    const int lane_bytes = gl * p.D * Tag::kBytes + part * NV * 16;
+    const bool pair = p.gt_lpg == 2;       // the two lanes of a (pixel, group) add their halves of each dot product
     typedef typename std::conditional<(KP > 0), uint32_t, uint64_t>::type mask_t;
     mask_t far_mask = 0;
     auto put = [&](int k, float gx, float gy, float gz, float m) {
+      if (part != 0) return;
       const float f0[1] = {gx * p.offset_scale * m}, f1[1] = {gy * p.offset_scale * m}, f2[1] = {gz};
       om[2 * k] = Pack<Tag, 1>::encode(f0);
       om[2 * k + 1] = Pack<Tag, 1>::encode(f1);
@@ -490,7 +497,7 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
 #pragma unroll
           for (int c = 0; c < EPV; ++c) acc = fmaf(f[c], go[v][c], acc);
         }
-        d[cn] = acc;
+        d[cn] = pair ? acc + dpp_quad_xor1(acc) : acc;
       }
       combine(k, d, wt.ly, wt.lx, wt.w, m);      // all zeros for a point outside the image or the window
     };
@@ -498,7 +505,7 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
     // offsets are re-read from memory because the LDS slots already hold gradients
     const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
     const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
-    const uint32_t img_base = (uint32_t)t.b * (uint32_t)(p.H * p.W) * pix_bytes + (uint32_t)((t.g0 + gl) * p.D) * Tag::kBytes;
+    const uint32_t img_base = (uint32_t)t.b * (uint32_t)(p.H * p.W) * pix_bytes + (uint32_t)((t.g0 + gl) * p.D) * Tag::kBytes + (uint32_t)(part * NV * 16);
     const elem_t *om_g = reinterpret_cast<const elem_t *>(p.offset_mask) +
                          ((size_t)t.b * p.Q + (size_t)ho * p.Wo + wo) * p.P_pad + (t.g0 + gl) * 3 * Kp;
     auto far_tap = [&](int k, int i, int j) {
@@ -517,7 +524,7 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
 #pragma unroll
           for (int c = 0; c < EPV; ++c) acc = fmaf(f[c], go[v][c], acc);
         }
-        d[cn] = acc;
+        d[cn] = pair ? acc + dpp_quad_xor1(acc) : acc;
       }
       combine(k, d, tp.ly, tp.lx, tp.w, m);
     };
@@ -603,9 +610,9 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
   const int nty = (Ho + p.gt_h - 1) / p.gt_h, ntx = (p.Wo + p.gt_w - 1) / p.gt_w;
   const int n_img = p.n_pix / p.Q;
   const dim3 grid((unsigned)(n_img * nty * ntx * n_chunks));
-  const dim3 block((unsigned)((p.gt_h * p.gt_w * p.gt_ng + kWave - 1) / kWave * kWave));
+  const dim3 block((unsigned)((p.gt_h * p.gt_w * p.gt_ng * p.gt_lpg + kWave - 1) / kWave * kWave));
   const size_t lds = dcnv4_tiled_gather_lds_bytes(p, Tag::kBytes);
-  switch (p.D * Tag::kBytes / 16) {
+  switch (p.D * Tag::kBytes / 16 / p.gt_lpg) {      // 16-byte vectors per lane
     case 1: return launch_nv<Tag, 1, BWD>(p, stream, grid, block, lds);
     case 2: return launch_nv<Tag, 2, BWD>(p, stream, grid, block, lds);
     case 4: return launch_nv<Tag, 4, BWD>(p, stream, grid, block, lds);

@@ -65,6 +65,7 @@ struct DcnLaunch {
   // LDS-tiled gather path (forward and grad_offset_mask); gt_h == 0: not planned
   int gt_h, gt_w;           // output tile one workgroup owns
   int gt_ng;                // groups per workgroup
+  int gt_lpg;               // lanes per (pixel, group): 1, or 2 when a group is 64 bytes or wider
   int gt_wh, gt_ww;         // largest input window (rows, columns of cells) a tile stages
   int gt_reach;             // input pixels around an output pixel's reference point that the window covers
 };
