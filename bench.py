@@ -60,6 +60,7 @@ def fda_bytes(s, B, N, Q, G, D, L, K):
 # (`--only-op copy:256`: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0, KiB).  The summaries are in profiles/.
 MEASURED_TRAFFIC_BYTES = {
     "dcnv4_bwd:T-stage1:float32": 508.6e6,     # algorithmic 334.0e6: the tiled pass re-reads offset_mask and grad_out
+    "dcnv4_bwd:T-stage1:float16": 238.0e6,     # algorithmic 167.0e6
     "dcnv4_fwd:T-stage1:float16": 96.5e6,      # algorithmic 96.3e6
 }
 
@@ -274,7 +275,7 @@ def main():
         "traffic": MEASURED_TRAFFIC_BYTES.get(f'{dom["op"]}:{dom["shape"]}:{dom["dtype"]}'),
         "kernel": f'{dom["op"]} {dom["shape"]} {dom["dtype"]}', "ms": dom["ms"],
         "algorithmic_bytes": int(dom_bytes),
-        "note": "HIP events around whole operator calls (backward = state reset + grad_offset_mask kernel + tiled grad_value kernel + fallback)",
+        "note": "HIP events around whole operator calls (backward = state reset + grad_offset_mask kernel + tiled grad_value kernel + fallback); traffic = rocprofv3 FETCH_SIZE/WRITE_SIZE per call, scaled by a copy of known size (profiles/)",
     }
 
     # ------------------------------------------------------------------ CPU baseline (rank 0, bounded sample)
