@@ -1,3 +1,3 @@
-from .flash_intern_image import FlashInternImage, flash_intern_image
+from .flash_intern_image import FlashInternImage, FlashInternImageBackbone, flash_intern_image
 
-__all__ = ["FlashInternImage", "flash_intern_image"]
+__all__ = ["FlashInternImage", "FlashInternImageBackbone", "flash_intern_image"]

@@ -224,6 +224,35 @@ class FlashInternImage(nn.Module):
         return self.head(self.forward_features(x))
 
 
+class FlashInternImageBackbone(FlashInternImage):
+    """Dense-prediction backbone: the same stem and levels without the classification head; ``forward`` returns
+    the NCHW feature map of every level in ``out_indices``, taken before that level's downsample, for inputs of
+    any (non-square) size.  Follows detection/mmdet_custom/models/backbones/flash_intern_image.py:596-608,750-763
+    (the segmentation backbone is the same code); checkpoint loading and layer-wise learning-rate tables belong to
+    the mmdet/mmseg side and are not reproduced."""
+
+    def __init__(self, out_indices=(0, 1, 2, 3), **kwargs):
+        kwargs.setdefault("num_classes", 0)
+        super().__init__(**kwargs)
+        self.out_indices = tuple(out_indices)
+        del self.conv_head, self.head, self.avgpool
+
+    def forward_features(self, x):
+        raise NotImplementedError("the backbone has no classification head; call forward()")
+
+    def forward(self, x):
+        x = self.patch_embed(x)
+        N, H, W, C = x.shape
+        x = x.view(N, H * W, C)
+        shape, outs = (H, W), []
+        for level_idx, level in enumerate(self.levels):
+            h, w = shape
+            x, before, shape = level(x, shape, return_wo_downsample=True)
+            if level_idx in self.out_indices:
+                outs.append(before.reshape(N, h, w, -1).permute(0, 3, 1, 2))
+        return outs
+
+
 # classification/configs/flash_intern_image_{t,s,b}_1k_224.yaml, flash_intern_image_l_22kto1k_384.yaml
 _VARIANTS = {
     "t": dict(channels=64, depths=(4, 4, 18, 4), groups=(4, 8, 16, 32), offset_scale=1.0, drop_path_rate=0.1),

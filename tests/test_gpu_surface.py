@@ -273,3 +273,37 @@ def test_small_flash_intern_image_matches_the_same_network_on_the_torch_core(mon
         want = model(x)
     assert got.shape == (2, 10) and [tuple(f.shape) for f in feats] == [(2, 32, 16, 16), (2, 64, 8, 8)]
     assert _rel_err(got, want) < 1e-3
+
+
+def test_dense_prediction_backbone_returns_per_level_maps_for_a_non_square_input(monkeypatch):
+    """FlashInternImageBackbone (detection / segmentation use): list of NCHW maps for the requested levels, on a
+    non-square input, equal to the same weights evaluated with the operator on the CPU grid_sample formulation."""
+    from dcnv4_amd.models import FlashInternImageBackbone
+    from dcnv4_amd.modules import dcnv4 as dcnv4_module
+
+    torch.manual_seed(5)
+    model = FlashInternImageBackbone(out_indices=(1, 2, 3), channels=16, depths=(1, 1, 1, 1), groups=(1, 2, 4, 8),
+                                     offset_scale=1.0, drop_path_rate=0.0, layer_scale=1e-1, post_norm=True,
+                                     dw_kernel_size=3).eval()
+    assert not any(k.startswith(("conv_head", "head")) for k in model.state_dict())
+    with torch.no_grad():
+        for m in model.modules():
+            if isinstance(m, dcnv4_module.DCNv4):
+                m.offset_mask.weight.normal_(0, 0.2)
+                m.offset_mask.bias.normal_(0, 0.5)
+    x = torch.randn(2, 3, 64, 96)
+
+    class CoreOnCpu:
+        @staticmethod
+        def apply(inp, om, kh, kw_, sh, sw, ph, pw, dh, dw, group, group_channels, offset_scale, im2col_step, remove_center):
+            return torch_core.dcnv4_core_torch(inp, om, kh, kw_, sh, sw, ph, pw, dh, dw, group, group_channels,
+                                               offset_scale, remove_center)
+
+    with torch.no_grad():
+        got = [f.cpu() for f in model.cuda()(x.cuda())]
+        model.cpu()
+        monkeypatch.setattr(dcnv4_module, "DCNv4Function", CoreOnCpu)
+        want = model(x)
+    assert [tuple(f.shape) for f in got] == [(2, 32, 8, 12), (2, 64, 4, 6), (2, 128, 2, 3)]
+    for g, w in zip(got, want):
+        assert _rel_err(g, w) < 1e-3
