@@ -80,7 +80,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this operator has no cross-GPU communication and every box here "
-                 "has a single MI355X; run with --gpus 1 (data-parallel scaling is a batch split, see DESIGN.md).")
+                 "has a single MI355X; run with --gpus 1 (data-parallel scaling is a plain batch split: the operator exchanges nothing between images).")
 
     import torch
     if not torch.cuda.is_available():
