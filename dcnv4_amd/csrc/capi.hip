@@ -536,6 +536,32 @@ int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_s
   return DCNV4_OK;
 }
 
+// Scratch of the tiled attention backward, in this order: GradState, keys, probabilities, tile table, sorted
+// point lists.  The last two are sized for the images of one launch and reused by the next.
+struct FdaScratch {
+  size_t keys, probs, table, regions, total;     // byte offsets, total bytes
+  int n_chunks, tile_stride, per;
+};
+
+FdaScratch fda_scratch(int batch, int N, int G, int D, int L, int Q, int K) {
+  FdaScratch sc;
+  const uint64_t per_img = (uint64_t)N * G * D * 4;
+  uint64_t per = std::max<uint64_t>(1, kMaxSpanBytes / per_img);
+  per = std::min<uint64_t>(per, 0x7fffffffull / (uint64_t)Q);
+  sc.per = (int)std::min<uint64_t>(per, (uint64_t)batch);
+  const size_t points = (size_t)G * L * fda_key_stride(Q, K);          // per image
+  sc.n_chunks = (int)(((size_t)Q * K + kFdaChunkPoints - 1) / kFdaChunkPoints);
+  // a level of H x W cells is cut into tiles of min(8, ceil(dim / 8)) cells per side: at most N/8 + 64 tiles
+  sc.tile_stride = (int)std::min<size_t>(kFdaMaxTilesPerLevel, (size_t)N / 8 + 64);
+  const size_t segs = (size_t)sc.per * G * L * sc.n_chunks;
+  sc.keys = kStateBytes;
+  sc.probs = sc.keys + round16((size_t)batch * points * sizeof(uint16_t));
+  sc.table = sc.probs + round16((size_t)batch * points * sizeof(float));
+  sc.regions = sc.table + round16(segs * sc.tile_stride * sizeof(uint32_t));
+  sc.total = sc.regions + round16(segs * 4 * kFdaChunkPoints * sizeof(uint32_t));
+  return sc;
+}
+
 size_t flash_deform_attn_gfx950_backward_workspace_bytes(int dtype, int batch, int spatial_size, int num_heads,
                                                          int head_channels, int num_levels, int num_query,
                                                          int num_points) {
@@ -543,8 +569,7 @@ size_t flash_deform_attn_gfx950_backward_workspace_bytes(int dtype, int batch, i
   size_t need = 0;
   if (elem_bytes(dtype) == 2) need = round16((size_t)batch * spatial_size * num_heads * head_channels * sizeof(float));
   if (fda_tiled_shape(head_channels, num_levels, num_query, num_points))
-    need = std::max(need, kStateBytes + round16((size_t)batch * num_heads * num_levels * fda_key_stride(num_query, num_points) * 2) +
-                              round16((size_t)batch * num_heads * num_levels * fda_key_stride(num_query, num_points) * 4));
+    need = std::max(need, fda_scratch(batch, spatial_size, num_heads, head_channels, num_levels, num_query, num_points).total);
   return need;
 }
 
@@ -575,16 +600,21 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   const size_t total = (size_t)batch * pr.img_elems;
-  const int per = images_per_launch(pr, true);
+  const int per = images_per_launch(pr, true);      // equals FdaScratch::per
 
   if (tiled) {
     // pass 0: grad_sampling_loc_attn, keys and max |grad_out|; pass 1: tiled grad_value; pass 2: fallback
     FdaLaunch base = pr.launch;
     base.state = static_cast<GradState *>(workspace);
+    const FdaScratch sc = fda_scratch(batch, spatial_size, num_heads, head_channels, num_levels, num_query, num_points);
     const size_t img_keys = (size_t)num_heads * num_levels * fda_key_stride(num_query, num_points);
-    const size_t key_bytes = round16((size_t)batch * img_keys * sizeof(uint16_t));
-    uint16_t *keys = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + kStateBytes);
-    float *probs = reinterpret_cast<float *>(static_cast<char *>(workspace) + kStateBytes + key_bytes);
+    char *ws = static_cast<char *>(workspace);
+    uint16_t *keys = reinterpret_cast<uint16_t *>(ws + sc.keys);
+    float *probs = reinterpret_cast<float *>(ws + sc.probs);
+    base.table = reinterpret_cast<uint32_t *>(ws + sc.table);
+    base.regions = reinterpret_cast<uint32_t *>(ws + sc.regions);
+    base.n_chunks = sc.n_chunks;
+    base.tile_stride = sc.tile_stride;
     // every term is grad_out * (probability * bilinear weight <= 1); at most Q * K of them meet in one cell
     base.fix_bits = 62 - ceil_log2((int)std::min<long long>((long long)num_query * num_points, 1 << 30));
     if (pr.s == 2) base.fix_bits = std::min(base.fix_bits, 30);

@@ -3,27 +3,35 @@
 // The reference scatters 4 * L * K * D fp32 atomicAdds per (query, head)
 // (DCNv4_op/src/cuda/flash_deform_col2im_cuda.cuh:240-270 through common.h:153-184).  Sampling
 // locations are free to land anywhere in their level, so unlike the DCNv4 operator there is no
-// window around the query to exploit; instead a workgroup OWNS a tile of one level of one
-// (image, head) and finds its contributions by scanning:
+// window around the query to exploit.  Instead the sampling points are first BINNED by the tile
+// of their level they touch, and then a workgroup that OWNS a tile adds them up in LDS:
 //
 //   * the grad_sampling_loc_attn kernel, which runs first, leaves one 16-bit key (integer position of
 //     the first corner, or "outside") and the softmax probability per sampling point, both laid out
 //     [image][head][level][query][point], and the maximum of |grad_out| in GradState;
-//   * scan: the workgroup streams the keys of its (image, head, level) - coalesced dwords of two keys, a handful
-//     of instructions per point - and appends the points whose 2x2 corner block touches its tile
-//     to a list in LDS;
-//   * apply, in batches of 256 listed points: one lane per point recomputes the position from
-//     sampling_loc_attn and, with the softmax probability the first kernel left beside the key,
-//     the four corner weights; grad_out rows of the batch are parked in LDS (both requested one
-//     batch ahead, so the loads fly while the previous batch is applied); a row of 8 lanes per point adds the
-//     contributions to the tile's accumulators with 64-bit integer LDS atomics on fixed-point
-//     values (normalised by max |grad_out|; probability * bilinear weight <= 1), so the result
-//     does not depend on the order of arrival and is bit-reproducible;
+//   * fda_bin_points_kernel: one workgroup per chunk of 8192 points of one (image, head, level)
+//     counting-sorts the chunk by tile in LDS (a point whose 2x2 corner block straddles tiles is
+//     listed under each of them) and writes the sorted point ids to the chunk's region of the
+//     workspace plus one (offset, count) word per tile to a table - no global atomics, no host
+//     round trip, every chunk independent;
+//   * fda_grad_value_kernel: persistent workgroups walk (tile, image, head) items, smallest level
+//     first.  An item collects its tile's slices of all chunk lists into LDS and applies them in
+//     batches: one lane per point rebuilds the position from sampling_loc_attn and, with the stored
+//     probability, the four corner weights; grad_out rows of the batch are parked in LDS (both
+//     requested one batch ahead, so the loads fly while the previous batch is applied); then a
+//     row of 8 lanes per point adds the contributions to the tile's accumulators with 64-bit integer
+//     LDS atomics on fixed-point values (normalised by max |grad_out|; probability * bilinear weight
+//     <= 1), so the result does not depend on the order of arrival and is bit-reproducible;
 //   * the finished tile is written to grad_value with plain stores in the tensor dtype.
 //
-// Workgroups are persistent and walk the (tile, image, head) items with a stride, smallest levels
-// first: those tiles collect the most points each.  Levels, tile shapes and the item count are
-// derived on the device from the spatial_shapes tensor; the host never reads it.
+// Tiles are at most 8x8 cells and every level is cut into up to 64 of them or more, so items stay
+// small (several workgroups share a CU and hide each other's latencies) and comparable in size.
+// Levels and tile shapes are derived on the device from the spatial_shapes tensor; the host never
+// reads it.  A level with more tiles than the binning kernel's LDS histogram holds raises a flag in
+// GradState: grad_value is then left zeroed for the atomic fallback kernel, like for non-finite
+// statistics.
+#include <algorithm>
+
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -31,20 +39,30 @@ namespace dcn {
 
 namespace {
 
-constexpr int kThreads = 1024;
+constexpr int kBinThreads = 1024;
+constexpr int kBinWordsPerLane = kFdaChunkPoints / 2 / kBinThreads;      // dwords of two keys per lane: 4
+constexpr int kApplyThreads = 512;
 constexpr int kRowLanes = 8;                 // lanes that apply one listed point
-constexpr int kBatch = 256;                  // listed points applied between two barriers
-constexpr int kScanPerLane = 16;             // dwords (two keys each) per lane and scan step: one memory latency per step
-constexpr int kRoundKeys = 4;                // dwords per lane tested between two looks at the list's fill
-constexpr int kScanStep = kThreads * kScanPerLane;
-constexpr int kListCap = 3 * kRoundKeys * kThreads;      // flushed when another round (2 * kRoundKeys points per lane) might not fit
-constexpr int kCellBitsF = 9;
+constexpr int kBatch = 128;                  // listed points applied between two barriers
+constexpr int kListCap = 1024;               // listed points held in LDS at a time
+constexpr int kTabCap = 256;                 // chunk table entries held in LDS at a time
+constexpr int kCellBitsF = 7;                // tiles have at most 64 cells; cell 64.. = trash
+constexpr int kTileCells = 64;
 
 struct LevelPlan {
   int H, W, start;
-  int th, tw, nty, ntx;      // tile shape and tile grid
-  int first_item_rank;       // rank of this level's first tile in the walk (smallest level first)
+  int th, tw, nty, ntx;      // tile shape (1..8 each) and tile grid
 };
+
+__device__ __forceinline__ LevelPlan level_plan(const FdaLaunch &p, int l) {
+  LevelPlan lp;
+  lp.H = (int)p.shapes[2 * l]; lp.W = (int)p.shapes[2 * l + 1]; lp.start = (int)p.level_start[l];
+  lp.th = max(1, min(8, (lp.H + 7) / 8));
+  lp.tw = max(1, min(8, (lp.W + 7) / 8));
+  lp.nty = lp.H > 0 ? (lp.H + lp.th - 1) / lp.th : 0;
+  lp.ntx = lp.W > 0 ? (lp.W + lp.tw - 1) / lp.tw : 0;
+  return lp;
+}
 
 // float -> two's-complement 64-bit integer, see dcnv4_grad_value.hip
 template <bool WIDE> __device__ __forceinline__ unsigned long long to_fixed64(float t) {
@@ -67,99 +85,192 @@ __device__ __forceinline__ float elem_at(const void *base, size_t i) {
   return f[0];
 }
 
+// n / d for small non-negative n and 1 <= d <= 8
+__device__ __forceinline__ int div_small(int n, float inv) { return (int)(((float)n + 0.5f) * inv); }
+
+// ------------------------------------------------------------------------------- binning
+// The tiles a sampling point touches: the tile of the first in-level row and column of its corner
+// block, and whether the block continues into the next tile column / row.
+struct Touch {
+  uint32_t t00;        // 0xffffffff = none
+  uint32_t dx, dy;
+};
+
+template <typename Tag>
+__global__ void __launch_bounds__(kBinThreads) fda_bin_points_kernel(const FdaLaunch p) {
+  __shared__ uint32_t s_hist[kFdaMaxTilesPerLevel];       // counts, then running cursors
+  __shared__ uint32_t s_wave_sum[kBinThreads / kWave];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int QK = p.Q * p.K, LK = p.L * p.K;
+  const int chunk = blockIdx.x % p.n_chunks, seg = blockIdx.x / p.n_chunks;       // seg = (image * G + head) * L + level
+  const int l = seg % p.L, bg = seg / p.L;
+  const int b = bg / p.G, g = bg - b * p.G;
+  const LevelPlan lp = level_plan(p, l);
+  const int n_tiles = lp.nty * lp.ntx;
+  if (n_tiles > p.tile_stride || n_tiles > kFdaMaxTilesPerLevel) {
+    if (tid == 0) atomicOr(&p.state->reserved, 1u);       // the fallback kernel takes over
+    return;
+  }
+  for (int i = tid; i < n_tiles; i += kBinThreads) s_hist[i] = 0u;
+  __syncthreads();
+
+  const size_t QKp = fda_key_stride(p.Q, p.K);
+  const uint32_t *keys = reinterpret_cast<const uint32_t *>(p.keys + (size_t)seg * QKp);
+  const int n_words = (int)(QKp / 2);
+  const float inv_th = 1.f / (float)lp.th, inv_tw = 1.f / (float)lp.tw;
+  const size_t sla_bg = ((size_t)b * p.Q * p.G + g) * 3 * LK;
+
+  auto touch_of = [&](uint32_t k16, uint32_t pt) {
+    Touch t;
+    t.t00 = 0xffffffffu; t.dx = t.dy = 0u;
+    if (pt >= (uint32_t)QK || k16 == kFdaKeyOutside) return t;
+    int y1 = (int)(k16 >> 8), x1 = (int)(k16 & 0xffu);             // y0 + 1, x0 + 1
+    if (k16 == kFdaKeySaturated) {                                // position beyond the key's fields: recompute it
+      const uint32_t q = pt / (uint32_t)p.K;
+      const int tt = l * p.K + (int)(pt - q * p.K);
+      const size_t row = sla_bg + (size_t)q * p.G * 3 * LK;
+      const float x = sub_rn(mul_rn(elem_at<Tag>(p.sla, row + 2 * tt), (float)lp.W), 0.5f);
+      const float y = sub_rn(mul_rn(elem_at<Tag>(p.sla, row + 2 * tt + 1), (float)lp.H), 0.5f);
+      const Tap tp = make_tap(y, x, lp.H, lp.W, 0u, 0u);
+      if (tp.valid == 0) return t;
+      y1 = tp.y0 + 1; x1 = tp.x0 + 1;
+    }
+    // rows y1 - 1 and y1 of the block, where they exist
+    const int ty_lo = div_small(y1 >= 1 ? y1 - 1 : y1, inv_th), ty_hi = y1 <= lp.H - 1 ? div_small(y1, inv_th) : ty_lo;
+    const int tx_lo = div_small(x1 >= 1 ? x1 - 1 : x1, inv_tw), tx_hi = x1 <= lp.W - 1 ? div_small(x1, inv_tw) : tx_lo;
+    t.t00 = (uint32_t)(ty_lo * lp.ntx + tx_lo);
+    t.dx = (uint32_t)(tx_hi != tx_lo);
+    t.dy = (uint32_t)(ty_hi != ty_lo);
+    return t;
+  };
+
+  // ---- pass 1: count
+  Touch touch[2 * kBinWordsPerLane];
+#pragma unroll
+  for (int u = 0; u < kBinWordsPerLane; ++u) {
+    const int w = chunk * (kFdaChunkPoints / 2) + u * kBinThreads + tid;
+    const uint32_t word = keys[min(w, n_words - 1)];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const Touch t = touch_of((word >> (16 * h)) & 0xffffu, w < n_words ? 2u * (uint32_t)w + h : 0xffffffffu);
+      touch[2 * u + h] = t;
+      if (t.t00 != 0xffffffffu) {
+        atomicAdd(&s_hist[t.t00], 1u);
+        if (t.dx) atomicAdd(&s_hist[t.t00 + 1], 1u);
+        if (t.dy) atomicAdd(&s_hist[t.t00 + lp.ntx], 1u);
+        if (t.dx && t.dy) atomicAdd(&s_hist[t.t00 + lp.ntx + 1], 1u);
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- exclusive prefix over the tiles (8 consecutive tiles per lane), table row out
+  constexpr int kPer = kFdaMaxTilesPerLevel / kBinThreads;      // 8
+  uint32_t cnt[kPer], sum = 0;
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int i = tid * kPer + j;
+    cnt[j] = i < n_tiles ? s_hist[i] : 0u;
+    sum += cnt[j];
+  }
+  uint32_t incl = sum;
+  for (int o = 1; o < kWave; o <<= 1) {
+    const uint32_t v = (uint32_t)__shfl_up((int)incl, o, kWave);
+    if (lane >= o) incl += v;
+  }
+  if (lane == kWave - 1) s_wave_sum[wave] = incl;
+  __syncthreads();
+  uint32_t before = incl - sum;
+  for (int w = 0; w < wave; ++w) before += s_wave_sum[w];
+  uint32_t *table = p.table + (size_t)blockIdx.x * p.tile_stride;
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int i = tid * kPer + j;
+    if (i < n_tiles) {
+      table[i] = before | (cnt[j] << 16);                 // offset <= 32767 and count <= 32768 for 8192 points
+      s_hist[i] = before;                                 // now the running cursor of the tile
+    }
+    before += cnt[j];
+  }
+  __syncthreads();
+
+  // ---- pass 2: place
+  uint32_t *region = p.regions + (size_t)blockIdx.x * (4 * kFdaChunkPoints);
+#pragma unroll
+  for (int u = 0; u < kBinWordsPerLane; ++u) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const Touch t = touch[2 * u + h];
+      if (t.t00 == 0xffffffffu) continue;
+      const uint32_t pt = 2u * (uint32_t)(chunk * (kFdaChunkPoints / 2) + u * kBinThreads + tid) + h;
+      region[atomicAdd(&s_hist[t.t00], 1u)] = pt;
+      if (t.dx) region[atomicAdd(&s_hist[t.t00 + 1], 1u)] = pt;
+      if (t.dy) region[atomicAdd(&s_hist[t.t00 + lp.ntx], 1u)] = pt;
+      if (t.dx && t.dy) region[atomicAdd(&s_hist[t.t00 + lp.ntx + 1], 1u)] = pt;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------- accumulation
 template <typename Tag, int CPL>
-__global__ void __launch_bounds__(kThreads) fda_grad_value_kernel(const FdaLaunch p) {
+__global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const FdaLaunch p) {
   extern __shared__ unsigned long long lds64[];
   typedef typename RawWord<Tag::kBytes>::type elem_t;
   constexpr int DP = CPL * kRowLanes;                         // accumulator channels per cell (D rounded up)
   const int D = p.D, LK = p.L * p.K, QK = p.Q * p.K;
-  const int cells_max = fda_tile_cells(D);
-  unsigned long long *acc = lds64;                            // [(cells_max + 1) * DP], last cell = trash
-  const int n_acc = (cells_max + 1) * DP;
+  unsigned long long *acc = lds64;                            // [(kTileCells + 1) * DP], last cell = trash
+  constexpr int n_acc = (kTileCells + 1) * DP;
   f32x4 *rec_w = reinterpret_cast<f32x4 *>(lds64 + n_acc);    // [kBatch]
-  u32x2 *rec_meta = reinterpret_cast<u32x2 *>(rec_w + kBatch);   // [kBatch] cells 0,1,2 | cell 3
+  u32x2 *rec_meta = reinterpret_cast<u32x2 *>(rec_w + kBatch);   // [kBatch] four 7-bit cells
   float *s_go = reinterpret_cast<float *>(rec_meta + kBatch); // [kBatch][DP]
   uint32_t *s_list = reinterpret_cast<uint32_t *>(s_go + kBatch * DP);   // [kListCap]
+  uint32_t *s_tab = s_list + kListCap;                        // [kTabCap] (offset | count << 16) of the item's tile per chunk
+  uint32_t *s_pre = s_tab + kTabCap;                          // [kTabCap + 1] exclusive prefix of the counts
   __shared__ LevelPlan s_plan[kMaxLevels];
-  __shared__ int s_items;
-  __shared__ uint32_t s_count;
+  __shared__ int s_first[kMaxLevels + 1];                     // rank of each level's first tile in the walk
 
-  const int tid = threadIdx.x, lane = tid & (kWave - 1);
+  const int tid = threadIdx.x;
   if (tid == 0) {
-    // walk order: last level first
-    int rank = 0;
+    int rank = 0;                                             // walk order: last level first
     for (int l = p.L - 1; l >= 0; --l) {
-      LevelPlan lp;
-      lp.H = (int)p.shapes[2 * l]; lp.W = (int)p.shapes[2 * l + 1]; lp.start = (int)p.level_start[l];
-      lp.tw = max(1, min(lp.W, 16));
-      lp.th = max(1, min(lp.H, cells_max / lp.tw));
-      auto tiles = [&]() { return ((lp.H + lp.th - 1) / lp.th) * ((lp.W + lp.tw - 1) / lp.tw); };
-      while (tiles() < 16 && lp.th * lp.tw > 16) {           // small levels: more, smaller tiles
-        if (lp.th >= lp.tw) lp.th = (lp.th + 1) / 2; else lp.tw = (lp.tw + 1) / 2;
-      }
-      lp.nty = (lp.H + lp.th - 1) / lp.th; lp.ntx = (lp.W + lp.tw - 1) / lp.tw;
-      lp.first_item_rank = rank;
-      rank += (lp.H > 0 && lp.W > 0) ? lp.nty * lp.ntx : 0;
-      s_plan[l] = lp;
+      s_plan[l] = level_plan(p, l);
+      s_first[l] = rank;
+      rank += s_plan[l].nty * s_plan[l].ntx;
     }
-    s_items = rank;
-    s_count = 0u;
+    s_first[p.L] = rank;                                      // total
   }
   __syncthreads();
-  const int n_tiles = s_items;
+  const int n_tiles = s_first[p.L];
   const int BG = p.n_img * p.G;
 
   const uint32_t gmax = p.state->go_max_bits;
-  const bool finite = gmax < 0x7f800000u;
+  const bool usable = gmax < 0x7f800000u && gmax != 0u && p.state->reserved == 0u;
   const int e_go = (int)(gmax >> 23) - 126;                  // 2^e_go > max |grad_out|
   const int e_out = e_go - p.fix_bits;
+  const size_t QKp = fda_key_stride(p.Q, p.K);
 
   for (int item = blockIdx.x; item < n_tiles * BG; item += gridDim.x) {
     const int rank = item / BG, bg = item - rank * BG;
     const int b = bg / p.G, g = bg - b * p.G;
     int l = 0;
-    for (int i = 0; i < p.L; ++i)
-      if (s_plan[i].first_item_rank <= rank && (s_plan[i].H > 0 && s_plan[i].W > 0)) {
-        // levels were ranked from the last one down: the matching level is the smallest index whose first rank <= rank
-        l = i;
-        break;
-      }
+    for (int i = 0; i < p.L; ++i)       // first ranks fall with the level index: the first level whose rank fits
+      if (s_first[i] <= rank && s_plan[i].nty * s_plan[i].ntx > 0) { l = i; break; }
     const LevelPlan lp = s_plan[l];
-    const int t_in = rank - lp.first_item_rank;
+    const int t_in = rank - s_first[l];
     const int ty = t_in / lp.ntx, tx = t_in - ty * lp.ntx;
     const int ty0 = ty * lp.th, tx0 = tx * lp.tw;
     const int th = min(lp.th, lp.H - ty0), tw = min(lp.tw, lp.W - tx0);
-    const int n_cells = th * tw;                             // <= cells_max; cell n_cells.. = trash
+    const int n_cells = th * tw;                             // <= 64; cell n_cells.. = trash
+    const int seg = bg * p.L + l;
 
-    for (int i = tid; i < n_acc; i += kThreads) acc[i] = 0ull;
-    __syncthreads();
+    for (int i = tid; i < n_acc; i += kApplyThreads) acc[i] = 0ull;
 
-    const size_t QKp = fda_key_stride(p.Q, p.K);
-    const uint32_t *keys = reinterpret_cast<const uint32_t *>(p.keys + ((size_t)(b * p.G + g) * p.L + l) * QKp);      // two keys per dword
-    const int n_words = (int)(QKp / 2);
+    const float *probs = p.probs + (size_t)seg * QKp;
     const size_t sla_bg = ((size_t)b * p.Q * p.G + g) * 3 * LK;       // + q * G * 3LK
     const size_t go_bg = ((size_t)b * p.Q * p.G + g) * D;             // + q * G * D
 
-    // exact position of point `pt` of this level, from sampling_loc_attn (dcnv4 convention: x first)
-    auto position = [&](uint32_t pt, float &y, float &x, uint32_t &q) {
-      q = pt / (uint32_t)p.K;
-      const int k = (int)(pt - q * p.K);
-      const size_t row = sla_bg + (size_t)q * p.G * 3 * LK;
-      const int t = l * p.K + k;
-      x = sub_rn(mul_rn(elem_at<Tag>(p.sla, row + 2 * t), (float)lp.W), 0.5f);       // flash_deform_im2col_cuda.cuh:188-189
-      y = sub_rn(mul_rn(elem_at<Tag>(p.sla, row + 2 * t + 1), (float)lp.H), 0.5f);
-    };
-
-    // ---- apply the first `n` listed points, in batches.  What a batch needs from memory (position,
-    // probability, grad_out rows) is requested one batch ahead, so the loads fly while the previous
-    // batch is applied.
-    const float *probs = p.probs + ((size_t)(b * p.G + g) * p.L + l) * QKp;
-    constexpr int kParts = DP / 4;                           // 4-channel pieces of a grad_out row
-    constexpr int kGoLoads = kBatch * kParts / kThreads;     // pieces per lane and batch (DP = 32: 2)
-    static_assert(kBatch * kParts % kThreads == 0 || kBatch * kParts < kThreads, "grad_out pieces divide over the lanes");
-    constexpr int kGoPerLane = kGoLoads > 0 ? kGoLoads : 1;
-    // Everything is requested through range-checked buffer loads of raw words: no branches around
-    // the loads, so they all fly together, and nothing is converted before it is needed.
+    // Everything a batch needs is requested through range-checked buffer loads of raw words: no branches
+    // around the loads, so they all fly together, and nothing is converted before it is needed.
     typedef typename RawWord<2 * Tag::kBytes>::type xy_t;      // (x, y) of a point are adjacent
     typedef typename RawWord<4 * Tag::kBytes>::type go4_t;     // 4 channels of grad_out
     const __amdgpu_buffer_rsrc_t sla_rs = make_rsrc(reinterpret_cast<const elem_t *>(p.sla) + sla_bg,
@@ -167,6 +278,9 @@ __global__ void __launch_bounds__(kThreads) fda_grad_value_kernel(const FdaLaunc
     const __amdgpu_buffer_rsrc_t go_rs = make_rsrc(reinterpret_cast<const elem_t *>(p.grad_out) + go_bg,
                                                    (uint32_t)((size_t)p.Q * p.G * D * Tag::kBytes));
     const __amdgpu_buffer_rsrc_t pr_rs = make_rsrc(probs, (uint32_t)QK * 4u);
+    constexpr int kParts = DP / 4;                           // 4-channel pieces of a grad_out row
+    constexpr int kGoLoads = kBatch * kParts / kApplyThreads;
+    constexpr int kGoPerLane = kGoLoads > 0 ? kGoLoads : 1;
     struct Ahead {
       xy_t xy;                         // lanes < batch size: their point
       uint32_t pr;
@@ -184,7 +298,7 @@ __global__ void __launch_bounds__(kThreads) fda_grad_value_kernel(const FdaLaunc
       }
 #pragma unroll
       for (int u = 0; u < kGoPerLane; ++u) {
-        const int i = tid + u * kThreads, h = i / kParts, part = i - h * kParts;
+        const int i = tid + u * kApplyThreads, h = i / kParts, part = i - h * kParts;
         const bool live = h < nb && i < kBatch * kParts && 4 * part < D;
         const uint32_t q = s_list[b0 + min(h, max(nb - 1, 0))] / (uint32_t)p.K;
         a.go[u] = buffer_load<4 * Tag::kBytes>(go_rs, live ? (q * (uint32_t)(p.G * D) + 4u * part) * Tag::kBytes : kDropOffset);
@@ -210,11 +324,11 @@ __global__ void __launch_bounds__(kThreads) fda_grad_value_kernel(const FdaLaunc
           w[cn] = ok ? ps * tp.w[cn] : 0.f;
         }
         rec_w[tid] = f32x4{w[0], w[1], w[2], w[3]};
-        rec_meta[tid] = u32x2{cells[0] | (cells[1] << kCellBitsF) | (cells[2] << (2 * kCellBitsF)), cells[3]};
+        rec_meta[tid] = u32x2{cells[0] | (cells[1] << kCellBitsF) | (cells[2] << (2 * kCellBitsF)) | (cells[3] << (3 * kCellBitsF)), 0u};
       }
 #pragma unroll
       for (int u = 0; u < kGoPerLane; ++u) {      // grad_out rows, normalised to [-1, 1] (zeros past the head width)
-        const int i = tid + u * kThreads, h = i / kParts, part = i - h * kParts;
+        const int i = tid + u * kApplyThreads, h = i / kParts, part = i - h * kParts;
         if (h < nb && i < kBatch * kParts) {
           float g4[4];
           Pack<Tag, 4>::decode(a.go[u], g4);
@@ -223,6 +337,7 @@ __global__ void __launch_bounds__(kThreads) fda_grad_value_kernel(const FdaLaunc
         }
       }
     };
+    // applies the first n entries of s_list; called by every lane, ends past a barrier
     auto apply_list = [&](uint32_t n) {
       if (n == 0) return;
       Ahead ahead = fetch(0, (int)min((uint32_t)kBatch, n));
@@ -234,10 +349,11 @@ __global__ void __launch_bounds__(kThreads) fda_grad_value_kernel(const FdaLaunc
         // a row of 8 lanes per point; row r starts its channel blocks at (r mod CPL), so the rows of one
         // instruction spread over the banks
         const int row_in_block = tid / kRowLanes, c = tid & (kRowLanes - 1);
-        for (int h = row_in_block; h < nb; h += kThreads / kRowLanes) {
+        for (int h = row_in_block; h < nb; h += kApplyThreads / kRowLanes) {
           const f32x4 w = rec_w[h];
-          const u32x2 meta = rec_meta[h];
-          const uint32_t cells[4] = {meta.x & 511u, (meta.x >> kCellBitsF) & 511u, (meta.x >> (2 * kCellBitsF)) & 511u, meta.y & 511u};
+          const uint32_t meta = rec_meta[h].x;
+          const uint32_t cells[4] = {meta & 127u, (meta >> kCellBitsF) & 127u, (meta >> (2 * kCellBitsF)) & 127u,
+                                     (meta >> (3 * kCellBitsF)) & 127u};
           const float wv[4] = {w.x, w.y, w.z, w.w};
           float gn[CPL];
           int ch_off[CPL];
@@ -259,82 +375,54 @@ __global__ void __launch_bounds__(kThreads) fda_grad_value_kernel(const FdaLaunc
       }
     };
 
-    // ---- scan the keys of (image, head, level); flush the list whenever another step might overflow it
-    if (finite && gmax != 0u) {
-      // A step = kScanPerLane dwords (two keys each) per lane, loaded in one go (and one step ahead) so that
-      // the memory latency is paid once per step; the step is then tested in rounds of kRoundKeys dwords per
-      // lane, few enough that the list can always take a whole round.
-      auto load_keys = [&](int base, uint32_t (&key)[kScanPerLane]) {
-#pragma unroll
-        for (int u = 0; u < kScanPerLane; ++u) {
-          const int i = base + u * kThreads + tid;
-          key[u] = keys[min(i, n_words - 1)];             // points past the end are masked when tested
-        }
-      };
-      uint32_t key[kScanPerLane], key_next[kScanPerLane];
-      load_keys(0, key_next);
-      for (int base = 0; base < n_words; base += kScanStep) {
-#pragma unroll
-        for (int u = 0; u < kScanPerLane; ++u) key[u] = key_next[u];
-        if (base + kScanStep < n_words) load_keys(base + kScanStep, key_next);      // in flight while this step is tested
-        // a real loop (the flush below must not be replicated per round): each round tests key[0..kRoundKeys)
-        // and then shifts the rest of the step's keys down
-#pragma unroll 1
-        for (int r = 0; r < kScanPerLane / kRoundKeys; ++r) {
-          // test the round's points first, then reserve list slots for all of them with one LDS atomic per wave
-          uint64_t masks[2 * kRoundKeys];
-          uint32_t total = 0;
-#pragma unroll
-          for (int uu = 0; uu < 2 * kRoundKeys; ++uu) {
-            const uint32_t k16 = (key[uu >> 1] >> (16 * (uu & 1))) & 0xffffu;
-            const uint32_t pt = 2u * (uint32_t)(base + (r * kRoundKeys + (uu >> 1)) * kThreads + tid) + (uu & 1);
-            bool hit = false;
-            if (pt >= (uint32_t)QK) {
-            } else if (k16 == kFdaKeySaturated) {                   // position beyond the key's fields: exact test
-              float y, x;
-              uint32_t q;
-              position(pt, y, x, q);
-              const Tap tp = make_tap(y, x, lp.H, lp.W, 0u, 0u);
-              hit = tp.valid != 0 && tp.y0 + 1 >= ty0 && tp.y0 < ty0 + th && tp.x0 + 1 >= tx0 && tp.x0 < tx0 + tw;
-            } else if (k16 != kFdaKeyOutside) {
-              // key = (y0 + 1) << 8 | (x0 + 1); the corner block {x0, x0 + 1} meets [tx0, tx0 + tw) iff 0 <= x0 + 1 - tx0 <= tw
-              hit = (uint32_t)((int)(k16 & 0xffu) - tx0) <= (uint32_t)tw && (uint32_t)((int)(k16 >> 8) - ty0) <= (uint32_t)th;
+    // ---- collect this tile's slices of the chunk lists (a group of chunks at a time) and apply them
+    if (usable) {
+      for (int c0 = 0; c0 < p.n_chunks; c0 += kTabCap) {
+        const int nc = min(kTabCap, p.n_chunks - c0);
+        __syncthreads();
+        for (int c = tid; c < nc; c += kApplyThreads)
+          s_tab[c] = p.table[((size_t)seg * p.n_chunks + c0 + c) * p.tile_stride + t_in];
+        __syncthreads();
+        if (tid < kWave) {            // exclusive prefix of the counts, one wave
+          uint32_t run = 0;
+          for (int base = 0; base < nc; base += kWave) {
+            const int c = base + tid;
+            const uint32_t v = c < nc ? s_tab[c] >> 16 : 0u;
+            uint32_t incl = v;
+            for (int o = 1; o < kWave; o <<= 1) {
+              const uint32_t up = (uint32_t)__shfl_up((int)incl, o, kWave);
+              if (tid >= o) incl += up;
             }
-            masks[uu] = __builtin_amdgcn_ballot_w64(hit);
-            total += (uint32_t)__builtin_popcountll(masks[uu]);
+            if (c < nc) s_pre[c] = run + incl - v;
+            run += (uint32_t)__shfl((int)incl, kWave - 1, kWave);
           }
-          if (total != 0) {
-            uint32_t slot0 = 0;
-            if (lane == 0) slot0 = atomicAdd(&s_count, total);
-            slot0 = __builtin_amdgcn_readfirstlane(slot0);
-#pragma unroll
-            for (int uu = 0; uu < 2 * kRoundKeys; ++uu) {
-              const uint64_t mask = masks[uu];
-              if ((mask >> lane) & 1) {
-                const uint32_t pt = 2u * (uint32_t)(base + (r * kRoundKeys + (uu >> 1)) * kThreads + tid) + (uu & 1);
-                s_list[slot0 + __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u))] = pt;
-              }
-              slot0 += (uint32_t)__builtin_popcountll(mask);
+          if (tid == 0) s_pre[nc] = run;
+        }
+        __syncthreads();
+        const uint32_t total = s_pre[nc];
+        // copy the slices into s_list, kListCap entries at a time; lane -> entry -> chunk by bisection
+        for (uint32_t e0 = 0; e0 < total; e0 += kListCap) {
+          const uint32_t ne = min((uint32_t)kListCap, total - e0);
+          for (uint32_t i = tid; i < ne; i += kApplyThreads) {
+            const uint32_t e = e0 + i;
+            int lo = 0, hi = nc;                       // largest c with s_pre[c] <= e
+            while (hi - lo > 1) {
+              const int mid = (lo + hi) >> 1;
+              if (s_pre[mid] <= e) lo = mid; else hi = mid;
             }
+            const uint32_t *region = p.regions + ((size_t)seg * p.n_chunks + c0 + lo) * (4 * kFdaChunkPoints);
+            s_list[i] = region[(s_tab[lo] & 0xffffu) + (e - s_pre[lo])];
           }
           __syncthreads();
-          const uint32_t n = s_count;
-          const bool last = base + kScanStep >= n_words && r == kScanPerLane / kRoundKeys - 1;
-          if (n > (uint32_t)(kListCap - 2 * kRoundKeys * kThreads) || last) {
-            __syncthreads();                // everyone has read the count
-            if (tid == 0) s_count = 0u;
-            apply_list(n);                  // ends with a barrier
-          }
-#pragma unroll
-          for (int u = 0; u + kRoundKeys < kScanPerLane; ++u) key[u] = key[u + kRoundKeys];
+          apply_list(ne);
         }
       }
     }
     __syncthreads();
 
-    // ---- the tile is complete (zeros when the statistics are unusable: the caller then runs the atomic path)
+    // ---- the tile is complete (zeros when the statistics are unusable: the fallback kernel then adds everything)
     elem_t *gv = reinterpret_cast<elem_t *>(p.grad_value);
-    for (int i = tid; i < n_cells * D; i += kThreads) {
+    for (int i = tid; i < n_cells * D; i += kApplyThreads) {
       const int cell = i / D, ch = i - cell * D;
       const int cy = cell / tw, cx = cell - cy * tw;
       const unsigned long long a = acc[cell * DP + ch];
@@ -348,13 +436,18 @@ __global__ void __launch_bounds__(kThreads) fda_grad_value_kernel(const FdaLaunc
 
 template <typename Tag>
 hipError_t launch_t(const FdaLaunch &p, hipStream_t stream) {
+  // binning: one workgroup per chunk of every (image, head, level)
+  hipLaunchKernelGGL(fda_bin_points_kernel<Tag>, dim3((unsigned)(p.n_img * p.G * p.L * p.n_chunks)), dim3(kBinThreads), 0, stream, p);
+  if (hipError_t e = hipGetLastError()) return e;
+
   int dev = 0, cus = 256;
   if (hipGetDevice(&dev) == hipSuccess) {
     int v = 0;
     if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
   }
-  const dim3 grid((unsigned)cus), block(kThreads);
   const size_t lds = fda_grad_value_lds_bytes(p);
+  const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(4, (kMaxLdsPerWorkgroup - 4096) / (lds + 1024)));
+  const dim3 grid((unsigned)(cus * per_cu)), block(kApplyThreads);
   auto go = [&](auto kernel) -> hipError_t {
     static bool raised = false;
     if (!raised) {
@@ -378,8 +471,8 @@ hipError_t launch_t(const FdaLaunch &p, hipStream_t stream) {
 
 size_t fda_grad_value_lds_bytes(const FdaLaunch &p) {
   const size_t dp = (size_t)fda_padded_channels(p.D);
-  return ((size_t)fda_tile_cells(p.D) + 1) * dp * sizeof(unsigned long long) + kBatch * (sizeof(f32x4) + sizeof(u32x2)) +
-         kBatch * dp * sizeof(float) + (size_t)kListCap * sizeof(uint32_t);
+  return ((size_t)kTileCells + 1) * dp * sizeof(unsigned long long) + kBatch * (sizeof(f32x4) + sizeof(u32x2)) +
+         kBatch * dp * sizeof(float) + ((size_t)kListCap + 2 * kTabCap + 4) * sizeof(uint32_t);
 }
 
 hipError_t launch_fda_grad_value(int dtype, const FdaLaunch &p, hipStream_t stream) {

@@ -96,14 +96,15 @@ __global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLau
 //                  cleared fp32 image (any head width)
 //   kFdaNoScatter  grad_sampling_loc_attn, plus what the tiled grad_value kernel needs: one key per
 //                  sampling point and the maximum of |grad_out|
-//   kFdaFallback   exits at once unless max |grad_out| is not finite; then it scatters with atomics in
-//                  the tensor dtype into grad_value, which the tiled kernel has left zeroed
+//   kFdaFallback   exits at once unless max |grad_out| is not finite or the binning kernel flagged a level
+//                  it cannot hold; then it scatters with atomics in the tensor dtype into grad_value,
+//                  which the tiled kernel has left zeroed
 template <typename Tag, int CPT, int KT, int MODE>
 __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLaunch p) {
   extern __shared__ float lds[];
   typedef Pack<Tag, CPT> pack;
   if constexpr (MODE == kFdaFallback) {
-    if (p.state->go_max_bits < 0x7f800000u) return;
+    if (p.state->go_max_bits < 0x7f800000u && p.state->reserved == 0u) return;
   }
   const int LK = p.L * p.K, row_len = 3 * LK;
   const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);

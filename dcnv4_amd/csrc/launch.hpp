@@ -90,6 +90,10 @@ struct FdaLaunch {
   GradState *state;         // go_max_bits only
   uint16_t *keys;           // [n_img, G, L, QKp] one key per sampling point (QKp = Q*K rounded up to even)
   float *probs;             // same layout: softmax probability of the point
+  uint32_t *table;          // [n_img * G * L * n_chunks][tile_stride] (offset | count << 16) of every tile in every chunk's sorted list
+  uint32_t *regions;        // [n_img * G * L * n_chunks][4 * kFdaChunkPoints] point ids of a chunk, sorted by tile
+  int n_chunks;             // chunks of kFdaChunkPoints points per (image, head, level)
+  int tile_stride;          // table row length: an upper bound of the tiles of one level
   int n_img;
   int fix_bits;             // fractional bits of the fixed-point accumulators
 };
@@ -100,6 +104,8 @@ struct FdaLaunch {
 constexpr uint32_t kFdaKeyOutside = 0xfeffu;
 constexpr uint32_t kFdaKeySaturated = 0xffffu;
 constexpr int kFdaKeyFieldMax = 0xfe;
+constexpr int kFdaChunkPoints = 8192;          // points one binning workgroup sorts
+constexpr int kFdaMaxTilesPerLevel = 8192;     // LDS histogram of the binning kernel
 __host__ __device__ inline size_t fda_key_stride(int Q, int K) { return ((size_t)Q * K + 1) & ~size_t(1); }
 
 enum FdaBackwardMode {
@@ -108,15 +114,11 @@ enum FdaBackwardMode {
   kFdaFallback = 2,    // scatter with atomics in the tensor dtype, only when max |grad_out| is not finite
 };
 
-// Accumulator channels per cell (head width rounded up to 8, 16, 32 or 64) and cells per tile of the
-// tiled flash-attention grad_value kernel.
+// Accumulator channels per cell of the tiled flash-attention grad_value kernel (head width rounded up to
+// 8, 16, 32 or 64).
 __host__ __device__ inline int fda_padded_channels(int D) {
   const int c = (D + 7) / 8;
   return (c <= 2 ? c : (c <= 4 ? 4 : 8)) * 8;
-}
-__host__ __device__ inline int fda_tile_cells(int D) {
-  const int cells = 8192 / fda_padded_channels(D);
-  return cells < 256 ? cells : 256;
 }
 
 // Each returns hipSuccess or the launch error.  dtype: 0 fp32, 1 fp16, 2 bf16.
