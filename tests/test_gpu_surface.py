@@ -171,6 +171,47 @@ def test_dcnv4_adjoint_identities_at_full_benchmark_size(dtype, tol):
     assert (gom[..., 108:] == 0).all()
 
 
+@pytest.mark.parametrize("B,H,W,G,off,dtype,tol", [
+    (2, 256, 256, 10, 4.0, torch.float16, 3e-3),      # dense-prediction stage 1 (1024x1024 image, FlashInternImage-L width)
+    (128, 56, 56, 7, 3.0, torch.float16, 3e-3),       # FlashInternImage-B stage 1 at batch 128
+    (64, 7, 7, 32, 3.0, torch.float32, 2e-5),         # smallest classification stage: most groups per pixel
+], ids=["dense_256x256_g10", "b_stage1_batch128", "t_stage4_fp32"])
+def test_dcnv4_adjoint_identities_at_the_other_benchmark_shapes(B, H, W, G, off, dtype, tol):
+    torch.manual_seed(6)
+    D, K, dev = 16, 9, "cuda"
+    P = G * K * 3
+    P_pad = (P + 7) // 8 * 8
+    v = torch.randn(B, H, W, G * D, device=dev).to(dtype)
+    body = torch.cat([(torch.rand(B, H, W, G, 2 * K, device=dev) * 2 - 1) * off, torch.randn(B, H, W, G, K, device=dev)], -1)
+    om = torch.zeros(B, H, W, P_pad, device=dev)
+    om[..., :P] = body.reshape(B, H, W, P)
+    om = om.to(dtype)
+    g = torch.randn(B, H, W, G * D, device=dev).to(dtype)
+    out = cabi.dcnv4_forward(v, om, GEOM, G, D, 1.0)
+    gv, gom = cabi.dcnv4_backward(v, om, g, GEOM, G, D, 1.0)
+    lhs = (g.double() * out.double()).sum()
+    by_value = (gv.double() * v.double()).sum()
+    mask = om[..., :P].reshape(B, H, W, G, 3 * K)[..., 2 * K:].double()
+    gmask = gom[..., :P].reshape(B, H, W, G, 3 * K)[..., 2 * K:].double()
+    scale = (g.double().abs() * out.double().abs()).sum()
+    assert abs(float(lhs - by_value)) / float(scale) < tol
+    assert abs(float(lhs - (gmask * mask).sum())) / float(scale) < tol
+    assert (gom[..., P:] == 0).all()
+
+
+def test_dcnv4_benchmark_stage_shape_matches_the_oracle_element_by_element(oracle):
+    """56x56, C=64, G=4 with the benchmark's offset range, a quarter of its batch: every element against the oracle."""
+    B, H, W, G, D = 16, 56, 56, 4, 16
+    v, om, go = make_dcnv4_inputs(B, H, W, G, D, offset_range=3.0, seed=21, dtype=torch.float16)
+    want = oracle.dcnv4_forward(cabi.f64(v), cabi.f64(om), *GEOM, G, D, 1.0, coord_f32=True)
+    wgv, wgom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *GEOM, G, D, 1.0, coord_f32=True)
+    out = cabi.dcnv4_forward(v.cuda(), om.cuda(), GEOM, G, D, 1.0)
+    gv, gom = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), GEOM, G, D, 1.0)
+    cabi.assert_close(out, want, 1e-2, 1e-3, what="output")
+    cabi.assert_close(gv, wgv, 1e-2, 1e-2, what="grad_value")
+    cabi.assert_close(gom, wgom, 1e-2, 1e-2, what="grad_offset_mask")
+
+
 def test_flash_deform_attn_adjoint_identity_at_full_benchmark_size():
     torch.manual_seed(4)
     shapes = [(128, 128), (64, 64), (32, 32), (16, 16)]
