@@ -551,7 +551,7 @@ FdaScratch fda_scratch(int batch, int N, int G, int D, int L, int Q, int K) {
   sc.per = (int)std::min<uint64_t>(per, (uint64_t)batch);
   const size_t points = (size_t)G * L * fda_key_stride(Q, K);          // per image
   sc.n_chunks = (int)(((size_t)Q * K + kFdaChunkPoints - 1) / kFdaChunkPoints);
-  // a level of H x W cells is cut into tiles of min(8, ceil(dim / 8)) cells per side: at most N/8 + 64 tiles
+  // a level of H x W cells is cut into tiles of min(8, ceil(dim / 4)) cells per side: at most N/8 + 64 tiles
   sc.tile_stride = (int)std::min<size_t>(kFdaMaxTilesPerLevel, (size_t)N / 8 + 64);
   const size_t segs = (size_t)sc.per * G * L * sc.n_chunks;
   sc.keys = kStateBytes;

@@ -24,7 +24,7 @@
 //     <= 1), so the result does not depend on the order of arrival and is bit-reproducible;
 //   * the finished tile is written to grad_value with plain stores in the tensor dtype.
 //
-// Tiles are at most 8x8 cells and every level is cut into up to 64 of them or more, so items stay
+// Tiles are at most 8x8 cells and every level is cut into 16 of them or more, so items stay
 // small (several workgroups share a CU and hide each other's latencies) and comparable in size.
 // Levels and tile shapes are derived on the device from the spatial_shapes tensor; the host never
 // reads it.  A level with more tiles than the binning kernel's LDS histogram holds raises a flag in
@@ -57,8 +57,8 @@ struct LevelPlan {
 __device__ __forceinline__ LevelPlan level_plan(const FdaLaunch &p, int l) {
   LevelPlan lp;
   lp.H = (int)p.shapes[2 * l]; lp.W = (int)p.shapes[2 * l + 1]; lp.start = (int)p.level_start[l];
-  lp.th = max(1, min(8, (lp.H + 7) / 8));
-  lp.tw = max(1, min(8, (lp.W + 7) / 8));
+  lp.th = max(1, min(8, (lp.H + 3) / 4));
+  lp.tw = max(1, min(8, (lp.W + 3) / 4));
   lp.nty = lp.H > 0 ? (lp.H + lp.th - 1) / lp.th : 0;
   lp.ntx = lp.W > 0 ? (lp.W + lp.tw - 1) / lp.tw : 0;
   return lp;
