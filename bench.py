@@ -106,6 +106,16 @@ def main():
     def dcn_bwd(t, G, C):
         return ext.dcnv4_backward(t[0], t[1], *GEOM, G, C // G, 1.0, 64, t[2], 0, 0, 0, False)
 
+    def dw_inputs(B, H, W, C, dtype):
+        return (torch.randn(B, H, W, C, device=dev).to(dtype), (torch.randn(C, 1, 3, 3, device=dev) / 3).to(dtype),
+                torch.randn(C, device=dev).to(dtype), torch.randn(B, H, W, C, device=dev).to(dtype))
+
+    def dw_bytes(s, B, H, W, C):
+        # forward: input read + output written; backward: input and grad_out read, grad_input written
+        # (grad_weight and grad_bias are C * 10 elements)
+        t = B * H * W * C * s
+        return 2 * t, 3 * t
+
     def time_op(fn, iters, warm=20):
         for _ in range(warm):
             fn()
@@ -152,6 +162,19 @@ def main():
             print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "algorithmic_MB": round(nbytes / 1e6, 2),
                               "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)}))
             return
+        if op.startswith("depthwise"):       # the offset_mask_dw layer of a DCNv4 block, 3x3, NHWC
+            for name, B, H, W, C, G in CFG2 + CFG5:
+                if name != shape_name:
+                    continue
+                x, w, b, go = dw_inputs(B, H, W, C, dtype)
+                fn = (lambda: ext.depthwise_conv_forward(x, w, b, 1)) if op == "depthwise_fwd" else \
+                     (lambda: ext.depthwise_conv_backward(x, w, go, 1))
+                ms = time_op(fn, args.steps, warm=args.warmup)
+                nbytes = dw_bytes(x.element_size(), B, H, W, C)[0 if op == "depthwise_fwd" else 1]
+                print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "algorithmic_MB": round(nbytes / 1e6, 2),
+                                  "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)}))
+                return
+            sys.exit(f"--only-op {args.only_op}: no such shape")
         for table, off in ((CFG2, 3.0), (CFG3, 4.0), (CFG5, 3.0)):
             for name, B, H, W, C, G in table:
                 if name != shape_name:
@@ -213,6 +236,12 @@ def main():
             t = dcn_inputs(B, H, W, C, G, torch.float16, 3.0)
             add("dcnv4_fwd", name, torch.float16, time_op(lambda: dcn_fwd(t, G, C), args.op_iters), dcn_bytes(2, B, H, W, C, G)[0])
             del t
+            x, w, b, go = dw_inputs(B, H, W, C, torch.float16)
+            add("depthwise_fwd", name, torch.float16, time_op(lambda: ext.depthwise_conv_forward(x, w, b, 1), args.op_iters),
+                dw_bytes(2, B, H, W, C)[0])
+            add("depthwise_bwd", name, torch.float16, time_op(lambda: ext.depthwise_conv_backward(x, w, go, 1), args.op_iters),
+                dw_bytes(2, B, H, W, C)[1])
+            del x, w, b, go
         for dtype, s in ((torch.float16, 2), (torch.float32, 4)):
             (B, N, G, D, L, K), shapes, starts, v, sla, go = fda_inputs(dtype)
             fb, bb = fda_bytes(s, B, N, N, G, D, L, K)

@@ -10,7 +10,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libdcnv4_gfx950.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 OK, ERR_INVALID_ARGUMENT, ERR_RUNTIME = 0, 1, 2
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 
@@ -26,6 +26,9 @@ SIGNATURES = {
     "flash_deform_attn_gfx950_forward": (_i, [_vp] * 5 + [_i] * 11 + [_vp]),
     "flash_deform_attn_gfx950_backward_workspace_bytes": (_sz, [_i] * 8),
     "flash_deform_attn_gfx950_backward": (_i, [_vp] * 8 + [_sz] + [_i] * 11 + [_vp]),
+    "dcnv4_gfx950_depthwise_conv_forward": (_i, [_vp] * 4 + [_i] * 7 + [_vp]),
+    "dcnv4_gfx950_depthwise_conv_backward_workspace_bytes": (_sz, [_i] * 7),
+    "dcnv4_gfx950_depthwise_conv_backward": (_i, [_vp] * 7 + [_sz] + [_i] * 7 + [_vp]),
 }
 
 _lib = None

@@ -176,8 +176,8 @@ int plan_grad_value_tiles(DcnLaunch *L, int elem_bytes_of_launch) {
     else return fail(DCNV4_ERR_RUNTIME, "kernel with %d taps and %d group channels does not fit the tiled backward", L->Kp, D);
   }
   const long long contributions = (long long)visited(L->tile_h, L->sh) * visited(L->tile_w, L->sw) * L->Kp;
-  L->fix_bits = 62 - ceil_log2((int)std::min<long long>(contributions, 1 << 30));
-  if (elem_bytes_of_launch == 2) L->fix_bits = std::min(L->fix_bits, 30);   // 32-bit conversion path for 16-bit tensors
+  // a term must stay below 2^51 (the conversion's range), a sum below 2^62
+  L->fix_bits = std::min(50, 62 - ceil_log2((int)std::min<long long>(contributions, 1 << 30)));
   if (L->pack32) L->fix_bits = std::min(fix32, 22);                         // the rounding trick of the packed path needs |term| < 2^22
   // the tiled kernel addresses one image's offset_mask and grad_out with 32-bit element offsets
   if (L->Q >= (1 << 24) || (uint64_t)L->Q * (uint64_t)L->P_pad >= (1ull << 31) || (uint64_t)L->Q * (uint64_t)(L->G * L->D) >= (1ull << 31))
@@ -374,6 +374,64 @@ int check_ptrs(std::initializer_list<const void *> ptrs) {
 
 int hip_fail(const char *what, hipError_t e) {
   return fail(DCNV4_ERR_RUNTIME, "%s: %s", what, hipGetErrorString(e));
+}
+
+
+// ---------------------------------------------------------------- depthwise convolution (NHWC)
+struct DwProblem {
+  DwLaunch launch;         // geometry of one image; B, pointers and partial-sum fields set per launch
+  int s;                   // bytes per element
+  size_t in_img, out_img;  // elements per image
+  int per;                 // images per launch (tensors of a launch stay below 2 GiB)
+  int slab;                // row segments per grad_weight workgroup
+  size_t total_parts;
+};
+
+constexpr int kDwPartTarget = 2048;      // grad_weight partial sums per call, about
+constexpr int kDwGradSeg = 8;            // output columns a grad_weight lane walks per visit
+
+int dw_prepare(DwProblem *pr, int dtype, int batch, int H, int W, int C, int k, int pad) {
+  const int s = elem_bytes(dtype);
+  if (s == 0) return fail(DCNV4_ERR_RUNTIME, "unsupported dtype code %d (fp32, fp16, bf16 only)", dtype);
+  if (batch <= 0 || H <= 0 || W <= 0 || C <= 0)
+    return fail(DCNV4_ERR_RUNTIME, "empty or negative tensor extent (batch %d, H %d, W %d, channels %d)", batch, H, W, C);
+  if (k != 1 && k != 3 && k != 5 && k != 7)
+    return fail(DCNV4_ERR_INVALID_ARGUMENT, "depthwise kernel size %d is not supported (1, 3, 5 or 7)", k);
+  if (pad < 0 || pad > k - 1) return fail(DCNV4_ERR_INVALID_ARGUMENT, "padding %d does not suit a %dx%d kernel (0..%d)", pad, k, k, k - 1);
+  const int Ho = H + 2 * pad - k + 1, Wo = W + 2 * pad - k + 1;
+  if (Ho <= 0 || Wo <= 0) return fail(DCNV4_ERR_RUNTIME, "kernel does not fit the padded input (output %dx%d)", Ho, Wo);
+  DwLaunch &L = pr->launch;
+  L = DwLaunch{};
+  L.H = H; L.W = W; L.C = C; L.Ho = Ho; L.Wo = Wo; L.kh = L.kw = k; L.ph = L.pw = pad;
+  pr->s = s;
+  pr->in_img = (size_t)H * W * C;
+  pr->out_img = (size_t)Ho * Wo * C;
+  const size_t img_bytes = std::max(pr->in_img, pr->out_img) * s;
+  if (img_bytes >= (size_t(1) << 31))
+    return fail(DCNV4_ERR_RUNTIME, "one image of %zu bytes exceeds the 2 GiB addressing span of a launch", img_bytes);
+  pr->per = (int)std::min<size_t>((size_t)batch, ((size_t(1) << 31) - 1) / img_bytes);
+  // grad_weight: a workgroup takes `slab` row segments of kDwGradSeg columns, a whole number of rounds of
+  // its pixel lanes, sized for about kDwPartTarget workgroups per call
+  L.seg = std::min(kDwGradSeg, Wo);
+  L.n_seg = (Wo + L.seg - 1) / L.seg;
+  const int lanes = depthwise_grad_weight_pixel_lanes(s, C, k);
+  const size_t n_rowseg = (size_t)batch * Ho * L.n_seg;
+  const size_t rounds = std::max<size_t>(1, (n_rowseg + (size_t)kDwPartTarget * lanes - 1) / ((size_t)kDwPartTarget * lanes));
+  pr->slab = (int)std::min<size_t>(rounds * lanes, 1u << 30);
+  pr->total_parts = 0;
+  for (int b0 = 0; b0 < batch; b0 += pr->per)
+    pr->total_parts += ((size_t)std::min(pr->per, batch - b0) * Ho * L.n_seg + pr->slab - 1) / pr->slab;
+  return DCNV4_OK;
+}
+
+// output columns per lane: long enough to reuse the sliding window, short enough to fill the GPU
+void dw_segments(DwLaunch *L, int elem_bytes_of_launch) {
+  const int vec = 16 / elem_bytes_of_launch;
+  const size_t lanes_per_col = (size_t)L->B * L->Ho * std::max(1, L->C / vec);
+  int seg = 8;
+  while (seg > 2 && lanes_per_col * ((L->Wo + seg - 1) / seg) < 256u * 1024u) seg /= 2;
+  L->seg = std::min(seg, L->Wo);
+  L->n_seg = (L->Wo + L->seg - 1) / L->seg;
 }
 
 const char *at(const void *base, size_t elems, int s) { return static_cast<const char *>(base) + elems * s; }
@@ -616,8 +674,8 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
     base.n_chunks = sc.n_chunks;
     base.tile_stride = sc.tile_stride;
     // every term is grad_out * (probability * bilinear weight <= 1); at most Q * K of them meet in one cell
-    base.fix_bits = 62 - ceil_log2((int)std::min<long long>((long long)num_query * num_points, 1 << 30));
-    if (pr.s == 2) base.fix_bits = std::min(base.fix_bits, 30);
+    // (a term must also stay below 2^51, the conversion's range)
+    base.fix_bits = std::min(50, 62 - ceil_log2((int)std::min<long long>((long long)num_query * num_points, 1 << 30)));
     hipLaunchKernelGGL(init_state_kernel, dim3(1), dim3(64), 0, st, base.state);
     if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);
     for (int pass = 0; pass < 3; ++pass) {
@@ -665,6 +723,87 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
   }
   if (widen)
     if (hipError_t e = narrow_async(dtype, acc, grad_value, total, st)) return hip_fail("cast launch", e);
+  return DCNV4_OK;
+}
+
+int dcnv4_gfx950_depthwise_conv_forward(const void *input, const void *weight, const void *bias, void *output,
+                                        int dtype, int batch, int height, int width, int channels, int kernel_size,
+                                        int pad, void *stream) {
+  DwProblem pr;
+  if (int rc = dw_prepare(&pr, dtype, batch, height, width, channels, kernel_size, pad)) return rc;
+  if (int rc = check_ptrs({input, weight, output})) return rc;
+  if (bias != nullptr && !aligned16(bias)) return fail(DCNV4_ERR_RUNTIME, "tensor pointer %p is not 16-byte aligned", bias);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  for (int b0 = 0; b0 < batch; b0 += pr.per) {
+    DwLaunch L = pr.launch;
+    L.B = std::min(pr.per, batch - b0);
+    L.in = at(input, b0 * pr.in_img, pr.s);
+    L.out = at(output, b0 * pr.out_img, pr.s);
+    L.weight = weight;
+    L.bias = bias;
+    dw_segments(&L, pr.s);
+    if (hipError_t e = launch_depthwise_forward(dtype, L, st)) return hip_fail("depthwise forward launch", e);
+  }
+  return DCNV4_OK;
+}
+
+size_t dcnv4_gfx950_depthwise_conv_backward_workspace_bytes(int dtype, int batch, int height, int width, int channels,
+                                                            int kernel_size, int pad) {
+  DwProblem pr;
+  if (dw_prepare(&pr, dtype, batch, height, width, channels, kernel_size, pad)) return 0;
+  return round16(pr.total_parts * (size_t)(kernel_size * kernel_size + 1) * channels * sizeof(float));
+}
+
+int dcnv4_gfx950_depthwise_conv_backward(const void *input, const void *weight, const void *grad_output, void *grad_input,
+                                         void *grad_weight, void *grad_bias, void *workspace, size_t workspace_bytes,
+                                         int dtype, int batch, int height, int width, int channels, int kernel_size,
+                                         int pad, void *stream) {
+  DwProblem pr;
+  if (int rc = dw_prepare(&pr, dtype, batch, height, width, channels, kernel_size, pad)) return rc;
+  if (int rc = check_ptrs({grad_output})) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (grad_input != nullptr) {
+    // correlation of grad_output with the flipped kernel, padding k - 1 - pad: output extent = the input's
+    if (int rc = check_ptrs({weight, grad_input})) return rc;
+    for (int b0 = 0; b0 < batch; b0 += pr.per) {
+      DwLaunch L = pr.launch;
+      L.B = std::min(pr.per, batch - b0);
+      L.H = pr.launch.Ho; L.W = pr.launch.Wo; L.Ho = pr.launch.H; L.Wo = pr.launch.W;
+      L.ph = L.pw = kernel_size - 1 - pad;
+      L.flip = 1;
+      L.in = at(grad_output, b0 * pr.out_img, pr.s);
+      L.out = at(grad_input, b0 * pr.in_img, pr.s);
+      L.weight = weight;
+      L.bias = nullptr;
+      dw_segments(&L, pr.s);
+      if (hipError_t e = launch_depthwise_forward(dtype, L, st)) return hip_fail("depthwise grad_input launch", e);
+    }
+  }
+  if (grad_weight != nullptr) {
+    if (int rc = check_ptrs({input, grad_weight})) return rc;
+    const size_t row = (size_t)(kernel_size * kernel_size + 1) * channels;
+    const size_t need = round16(pr.total_parts * row * sizeof(float));
+    if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
+      return fail(DCNV4_ERR_RUNTIME, "workspace of %zu bytes needed, got %zu at %p", need, workspace_bytes, workspace);
+    size_t parts_done = 0;
+    for (int b0 = 0; b0 < batch; b0 += pr.per) {
+      DwLaunch L = pr.launch;
+      L.B = std::min(pr.per, batch - b0);
+      L.in = at(input, b0 * pr.in_img, pr.s);
+      L.grad_out = at(grad_output, b0 * pr.out_img, pr.s);
+      L.slab = pr.slab;
+      L.n_part = (int)(((size_t)L.B * L.Ho * L.n_seg + pr.slab - 1) / pr.slab);
+      L.partial = static_cast<float *>(workspace) + parts_done * row;
+      if (hipError_t e = launch_depthwise_grad_weight_partials(dtype, L, st)) return hip_fail("depthwise grad_weight launch", e);
+      parts_done += (size_t)L.n_part;
+    }
+    DwLaunch L = pr.launch;
+    L.partial = static_cast<float *>(workspace);
+    L.n_part = (int)parts_done;
+    L.grad_weight = grad_weight;
+    L.grad_bias = grad_bias;
+    if (hipError_t e = launch_depthwise_grad_weight_reduce(dtype, L, st)) return hip_fail("depthwise grad_weight reduction launch", e);
+  }
   return DCNV4_OK;
 }
 

@@ -238,6 +238,16 @@ __device__ __forceinline__ void atomic_add_element(void *base, size_t elem, floa
   }
 }
 
+// round-to-nearest-even(a * b) as a two's-complement 64-bit integer, for |a * b| < 2^51.  The exact
+// product is formed inside a double-precision fma whose addend, 1.5 * 2^52, pushes the integer part
+// into the low mantissa bits; the addend's bit pattern has a zero low word, so removing it is one
+// 32-bit add.  Two VALU instructions per term (fp64 fma is full rate on this GPU) once the factors
+// are widened.
+__device__ __forceinline__ unsigned long long fixed_product(double a, double b) {
+  const double d = __builtin_fma(a, b, 6755399441055744.0);
+  return __builtin_bit_cast(unsigned long long, d) - 0x4338000000000000ull;
+}
+
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
   for (int o = 32; o > 0; o >>= 1) v = max(v, (uint32_t)__shfl_xor((int)v, o, kWave));
   return v;

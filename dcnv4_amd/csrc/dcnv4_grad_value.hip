@@ -20,8 +20,9 @@
 //          one ds_add_u64 instruction touches 64 distinct channels: two conflict-free bank sweeps;
 //   * fixed point: contributions are normalised by the global maxima of |grad_out| and
 //     |modulation| (GradState, produced by the grad_offset_mask kernel that runs first) and carry
-//     `fix_bits` fractional bits, i.e. an absolute resolution of 2^-fix_bits of the largest possible
-//     contribution - finer than fp32 accumulation unless a sum is > 2^25 times smaller than that.
+//     `fix_bits` fractional bits (up to 50; each product is exact in double precision and rounded
+//     once), i.e. an absolute resolution of 2^-fix_bits of the largest possible contribution - finer
+//     than fp32 accumulation unless a sum is > 2^25 times smaller than that.
 //     Integer sums make the result bit-reproducible, independent of scheduling;
 //   * corners farther than `reach` from their output pixel's tile, and the case of non-finite
 //     statistics, are left to the fallback scatter kernel (dcnv4_kernels.hip, kBwdFallback),
@@ -38,22 +39,6 @@ constexpr int kWaves = kValThreads / kWave;
 constexpr int kTrashPad = 64;
 constexpr int kMaxChunkGroups = 4;      // rows of a wave <-> groups of the chunk
 constexpr int kCellBits = 9;            // cell index 0..n_cells (n_cells = trash), tiles up to 16x16
-
-// float -> two's-complement 64-bit integer.
-// WIDE: |t| < 2^62, exact (t carries 24 significant bits), six instructions.
-// !WIDE: |t| < 2^31, truncated toward zero, three instructions; used for 16-bit tensors, whose values
-// carry 8-11 significant bits (fix_bits is then 30: 2^-30 of the largest possible contribution).
-template <bool WIDE> __device__ __forceinline__ unsigned long long to_fixed(float t) {
-  if constexpr (WIDE) {
-    const float th = floorf(t * 0x1p-32f);
-    const int hi = (int)th;
-    const uint32_t lo = (uint32_t)fmaf(th, -0x1p32f, t);
-    return ((unsigned long long)(uint32_t)hi << 32) | lo;
-  } else {
-    const int v = (int)t;
-    return ((unsigned long long)(uint32_t)(v >> 31) << 32) | (uint32_t)v;
-  }
-}
 
 // round-to-nearest-even(a * b) for |a * b| < 2^22, two instructions: the product is formed inside an
 // fma whose addend pushes the integer part into the low mantissa bits.
@@ -342,9 +327,10 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
               __hip_atomic_fetch_add(dst + (j / 2) * kRow, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
           } else {
+            const double wd = (double)wv[cn];
 #pragma unroll
             for (int j = 0; j < CPL; ++j)
-              __hip_atomic_fetch_add(dst + ch_off[j], to_fixed<Tag::kBytes == 4>(gn[j] * wv[cn]), __ATOMIC_RELAXED,
+              __hip_atomic_fetch_add(dst + ch_off[j], fixed_product((double)gn[j], wd), __ATOMIC_RELAXED,
                                      __HIP_MEMORY_SCOPE_WORKGROUP);
           }
         }

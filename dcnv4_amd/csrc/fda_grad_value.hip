@@ -64,19 +64,6 @@ __device__ __forceinline__ LevelPlan level_plan(const FdaLaunch &p, int l) {
   return lp;
 }
 
-// float -> two's-complement 64-bit integer, see dcnv4_grad_value.hip
-template <bool WIDE> __device__ __forceinline__ unsigned long long to_fixed64(float t) {
-  if constexpr (WIDE) {
-    const float th = floorf(t * 0x1p-32f);
-    const int hi = (int)th;
-    const uint32_t lo = (uint32_t)fmaf(th, -0x1p32f, t);
-    return ((unsigned long long)(uint32_t)hi << 32) | lo;
-  } else {
-    const int v = (int)t;
-    return ((unsigned long long)(uint32_t)(v >> 31) << 32) | (uint32_t)v;
-  }
-}
-
 template <typename Tag>
 __device__ __forceinline__ float elem_at(const void *base, size_t i) {
   typedef typename RawWord<Tag::kBytes>::type elem_t;
@@ -365,9 +352,10 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
 #pragma unroll
           for (int cn = 0; cn < 4; ++cn) {
             unsigned long long *dst = acc + __umul24(cells[cn], (uint32_t)DP) + c;
+            const double wd = (double)wv[cn];
 #pragma unroll
             for (int j = 0; j < CPL; ++j)
-              __hip_atomic_fetch_add(dst + ch_off[j], to_fixed64<Tag::kBytes == 4>(gn[j] * wv[cn]), __ATOMIC_RELAXED,
+              __hip_atomic_fetch_add(dst + ch_off[j], fixed_product((double)gn[j], wd), __ATOMIC_RELAXED,
                                      __HIP_MEMORY_SCOPE_WORKGROUP);
           }
         }

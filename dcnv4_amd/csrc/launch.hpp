@@ -121,7 +121,30 @@ __host__ __device__ inline int fda_padded_channels(int D) {
   return (c <= 2 ? c : (c <= 4 ? 4 : 8)) * 8;
 }
 
+// Depthwise convolution over NHWC tensors (stride 1, dilation 1); one launch covers tensors below 2 GiB.
+struct DwLaunch {
+  const void *in;          // [B, H, W, C]
+  const void *weight;      // [C, kh, kw]
+  const void *bias;        // [C] or null
+  void *out;               // [B, Ho, Wo, C]   (forward / grad_input)
+  const void *grad_out;    // [B, Ho, Wo, C]   (grad_weight)
+  float *partial;          // [n_part][kh*kw + 1][C] partial sums of grad_weight and grad_bias
+  void *grad_weight;       // [C, kh, kw]
+  void *grad_bias;         // [C] or null
+  int B, H, W, C, Ho, Wo;
+  int kh, kw, ph, pw;
+  int seg, n_seg;          // output columns per lane visit, segments per row
+  int flip;                // forward: read the kernel back to front (grad_input)
+  int slab, n_part;        // grad_weight: row segments (seg columns each) per workgroup, workgroups
+};
+
 // Each returns hipSuccess or the launch error.  dtype: 0 fp32, 1 fp16, 2 bf16.
+hipError_t launch_depthwise_forward(int dtype, const DwLaunch &p, hipStream_t stream);
+// channels per lane of the grad_weight kernel, and lanes of a workgroup that share a channel vector
+int depthwise_grad_weight_vector(int elem_bytes, int C, int k);
+int depthwise_grad_weight_pixel_lanes(int elem_bytes, int C, int k);
+hipError_t launch_depthwise_grad_weight_partials(int dtype, const DwLaunch &p, hipStream_t stream);
+hipError_t launch_depthwise_grad_weight_reduce(int dtype, const DwLaunch &p, hipStream_t stream);
 hipError_t launch_dcnv4_forward(int dtype, const DcnLaunch &p, hipStream_t stream);
 hipError_t launch_dcnv4_backward(int dtype, const DcnLaunch &p, int mode, hipStream_t stream);
 hipError_t launch_dcnv4_grad_value(int dtype, const DcnLaunch &p, hipStream_t stream);

@@ -150,3 +150,56 @@ def flash_deform_attn_backward(value, spatial_shapes, level_start_index, samplin
             ws.data_ptr() if ws is not None else None, ws_bytes, code, batch, spatial_size, num_heads, channels,
             num_levels, num_query, int(K), int(im2col_step), _hint(d_stride), _hint(block_thread), _stream()))
     return [grad_value, grad_sla]
+
+
+def depthwise_conv_forward(input, weight, bias, pad):
+    """Depthwise convolution of an NHWC tensor, stride 1, dilation 1: the ``offset_mask_dw`` layer of a
+    DCNv4 block (DCNv4_op/DCNv4/modules/dcnv4.py:67-75,121-123) without the permutes around it.
+    ``weight`` is nn.Conv2d's (C, 1, k, k) or (C, k, k); ``bias`` (C,) or None.  Returns (N, Ho, Wo, C)."""
+    _check(input, "input")
+    _check(weight, "weight", input.dtype)
+    if bias is not None:
+        _check(bias, "bias", input.dtype)
+    if input.dim() != 4:
+        raise RuntimeError("input must be 4-d (N, H, W, C)")
+    code = _dtype_code(input, "input")
+    batch, h, w, channels = input.shape
+    k = weight.shape[-1]
+    if weight.numel() != channels * k * k or weight.shape[0] != channels or weight.shape[-2] != k:
+        raise RuntimeError(f"weight shape {tuple(weight.shape)} is not a depthwise kernel for {channels} channels")
+    if bias is not None and bias.numel() != channels:
+        raise RuntimeError(f"bias has {bias.numel()} elements for {channels} channels")
+    ho, wo = h + 2 * pad - k + 1, w + 2 * pad - k + 1
+    with torch.cuda.device(input.device):
+        output = torch.empty((batch, max(ho, 0), max(wo, 0), channels), dtype=input.dtype, device=input.device)
+        _lib.check(_L.dcnv4_gfx950_depthwise_conv_forward(
+            input.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None, output.data_ptr(),
+            code, batch, h, w, channels, k, int(pad), _stream()))
+    return output
+
+
+def depthwise_conv_backward(input, weight, grad_output, pad, has_bias=True, need_input_grad=True,
+                            need_weight_grad=True):
+    """Gradients of :func:`depthwise_conv_forward`: ``[grad_input, grad_weight, grad_bias]`` (None for
+    the ones not asked for); grad_weight has the shape of ``weight``."""
+    _check(input, "input")
+    _check(weight, "weight", input.dtype)
+    _check(grad_output, "grad_output", input.dtype)
+    code = _dtype_code(input, "input")
+    batch, h, w, channels = input.shape
+    k = weight.shape[-1]
+    ho, wo = h + 2 * pad - k + 1, w + 2 * pad - k + 1
+    if tuple(grad_output.shape) != (batch, ho, wo, channels):
+        raise RuntimeError(f"grad_output shape {tuple(grad_output.shape)} does not match the output {(batch, ho, wo, channels)}")
+    with torch.cuda.device(input.device):
+        grad_input = torch.empty_like(input) if need_input_grad else None
+        grad_weight = torch.empty_like(weight) if need_weight_grad else None
+        grad_bias = torch.empty(channels, dtype=input.dtype, device=input.device) if (need_weight_grad and has_bias) else None
+        ws_bytes = _L.dcnv4_gfx950_depthwise_conv_backward_workspace_bytes(code, batch, h, w, channels, k, int(pad)) \
+            if need_weight_grad else 0
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=input.device) if ws_bytes else None
+        ptr = lambda t: t.data_ptr() if t is not None else None
+        _lib.check(_L.dcnv4_gfx950_depthwise_conv_backward(
+            input.data_ptr(), weight.data_ptr(), grad_output.data_ptr(), ptr(grad_input), ptr(grad_weight),
+            ptr(grad_bias), ptr(ws), ws_bytes, code, batch, h, w, channels, k, int(pad), _stream()))
+    return [grad_input, grad_weight, grad_bias]

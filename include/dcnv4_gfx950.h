@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define DCNV4_GFX950_ABI_VERSION 2
+#define DCNV4_GFX950_ABI_VERSION 3
 
 #define DCNV4_DTYPE_F32 0
 #define DCNV4_DTYPE_F16 1
@@ -134,6 +134,44 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
                                       int head_channels, int num_levels, int num_query,
                                       int num_points, int im2col_step, int d_stride,
                                       int block_thread, void *stream);
+
+/*
+ * Depthwise convolution over channels-last tensors, stride 1, dilation 1, square kernel of size
+ * 1, 3, 5 or 7: the `offset_mask_dw` layer of a DCNv4 block.  Replaces the nn.Conv2d call and the
+ * NHWC -> NCHW -> NHWC permutes around it (DCNv4_op/DCNv4/modules/dcnv4.py:67-75 and :121-123).
+ *   input    [batch, height, width, channels]
+ *   weight   [channels, kernel_size, kernel_size]   (nn.Conv2d's [channels, 1, k, k])
+ *   bias     [channels] or NULL
+ *   output   [batch, height_out, width_out, channels], height_out = height + 2*pad - kernel_size + 1
+ *            (fully overwritten)
+ *   out[b,y,x,c] = bias[c] + sum_{i,j} weight[c,i,j] * input[b, y+i-pad, x+j-pad, c], zero outside
+ */
+int dcnv4_gfx950_depthwise_conv_forward(const void *input, const void *weight, const void *bias,
+                                        void *output, int dtype, int batch, int height, int width,
+                                        int channels, int kernel_size, int pad, void *stream);
+
+/* Scratch bytes dcnv4_gfx950_depthwise_conv_backward needs for grad_weight at these sizes. */
+size_t dcnv4_gfx950_depthwise_conv_backward_workspace_bytes(int dtype, int batch, int height,
+                                                            int width, int channels,
+                                                            int kernel_size, int pad);
+
+/*
+ * Gradients of the depthwise convolution above (what autograd derives for the nn.Conv2d of
+ * DCNv4_op/DCNv4/modules/dcnv4.py:121).
+ *   grad_output  like output
+ *   grad_input   like input, or NULL to skip it           (fully overwritten)
+ *   grad_weight  like weight, or NULL to skip it and grad_bias   (fully overwritten)
+ *   grad_bias    like bias, or NULL
+ *   workspace    device scratch of at least ..._workspace_bytes(), 16-byte aligned; only used for
+ *                grad_weight / grad_bias; contents are destroyed
+ * Sums are formed in fp32 in a fixed order: results are bit-reproducible.
+ */
+int dcnv4_gfx950_depthwise_conv_backward(const void *input, const void *weight,
+                                         const void *grad_output, void *grad_input,
+                                         void *grad_weight, void *grad_bias, void *workspace,
+                                         size_t workspace_bytes, int dtype, int batch, int height,
+                                         int width, int channels, int kernel_size, int pad,
+                                         void *stream);
 
 #ifdef __cplusplus
 }

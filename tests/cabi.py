@@ -85,3 +85,31 @@ def assert_close(got, want, rtol, atol, what=""):
         i = np.unravel_index(np.argmax(err - tol), err.shape)
         raise AssertionError(f"{what}: {bad.sum()} / {bad.size} elements off; worst at {i}: got {got[i]!r} want {want[i]!r} "
                              f"(rtol {rtol}, atol {atol})")
+
+
+def depthwise_forward(inp, weight, bias, pad):
+    """inp (N,H,W,C), weight (C,k,k), bias (C,) or None, all on the GPU in one dtype."""
+    L = _lib.load()
+    B, H, W, C = inp.shape
+    k = weight.shape[-1]
+    out = torch.full((B, H + 2 * pad - k + 1, W + 2 * pad - k + 1, C), float("nan"), dtype=inp.dtype, device=inp.device)
+    _lib.check(L.dcnv4_gfx950_depthwise_conv_forward(inp.data_ptr(), weight.data_ptr(),
+                                                      bias.data_ptr() if bias is not None else None, out.data_ptr(),
+                                                      CODES[inp.dtype], B, H, W, C, k, pad, _stream()))
+    return out
+
+
+def depthwise_backward(inp, weight, go, pad, with_bias=True):
+    L = _lib.load()
+    B, H, W, C = inp.shape
+    k = weight.shape[-1]
+    gi = torch.full_like(inp, float("nan"))
+    gw = torch.full_like(weight, float("nan"))
+    gb = torch.full((C,), float("nan"), dtype=inp.dtype, device=inp.device) if with_bias else None
+    nbytes = L.dcnv4_gfx950_depthwise_conv_backward_workspace_bytes(CODES[inp.dtype], B, H, W, C, k, pad)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=inp.device)
+    _lib.check(L.dcnv4_gfx950_depthwise_conv_backward(inp.data_ptr(), weight.data_ptr(), go.data_ptr(), gi.data_ptr(),
+                                                       gw.data_ptr(), gb.data_ptr() if gb is not None else None,
+                                                       ws.data_ptr(), nbytes, CODES[inp.dtype], B, H, W, C, k, pad,
+                                                       _stream()))
+    return gi, gw, gb

@@ -271,3 +271,61 @@ def test_c_abi_rejects_bad_arguments():
     with pytest.raises(ValueError, match="scales"):
         cabi.fda_forward(torch.zeros(1, 68, 1, 16, device="cuda"), shp, torch.zeros(17, dtype=torch.int64, device="cuda"),
                          torch.zeros(1, 1, 1, 17 * 3, device="cuda"), 1)
+
+
+# ---------------------------------------------------------------- depthwise convolution (offset_mask_dw layer)
+# N, H, W, C, k, pad
+DW_CASES = {
+    "stage1_56x56_c64": (2, 56, 56, 64, 3, 1),
+    "stage4_7x7_c512": (3, 7, 7, 512, 3, 1),
+    "c112_non_square": (2, 13, 29, 112, 3, 1),
+    "c2560_many_vectors": (1, 5, 6, 2560, 3, 1),
+    "odd_channels": (2, 9, 8, 7, 3, 1),
+    "channels_multiple_of_2": (1, 10, 11, 6, 3, 1),
+    "no_padding": (1, 8, 9, 16, 3, 0),
+    "full_padding": (1, 6, 7, 16, 3, 2),
+    "kernel_5": (2, 11, 10, 24, 5, 2),
+    "kernel_7": (1, 12, 9, 16, 7, 3),
+    "kernel_1": (2, 6, 6, 32, 1, 0),
+    "single_pixel": (1, 1, 1, 8, 3, 1),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("name", list(DW_CASES))
+def test_depthwise_conv_matches_oracle(name, dtype):
+    from oracle import depthwise
+    N, H, W, C, k, pad = DW_CASES[name]
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(N, H, W, C, generator=g).to(dtype)
+    w = (torch.randn(C, k, k, generator=g) / k).to(dtype)
+    b = torch.randn(C, generator=g).to(dtype)
+    go = torch.randn(N, H + 2 * pad - k + 1, W + 2 * pad - k + 1, C, generator=g).to(dtype)
+    print(f"depthwise case {name} {dtype}", flush=True)
+    want = depthwise.depthwise_forward(cabi.f64(x), cabi.f64(w), cabi.f64(b), pad)
+    wgx, wgw, wgb = depthwise.depthwise_backward(cabi.f64(x), cabi.f64(w), cabi.f64(go), pad)
+    xd, wd, bd, god = x.cuda(), w.cuda(), b.cuda(), go.cuda()
+    out = cabi.depthwise_forward(xd, wd, bd, pad)
+    out_nb = cabi.depthwise_forward(xd, wd, None, pad)
+    gx, gw, gb = cabi.depthwise_backward(xd, wd, god, pad)
+    torch.cuda.synchronize()
+    cabi.assert_close(out, want, *FWD_TOL[dtype], what="output")
+    cabi.assert_close(out_nb, want - cabi.f64(b), *FWD_TOL[dtype], what="output without bias")
+    cabi.assert_close(gx, wgx, *GRAD_TOL[dtype], what="grad_input")
+    # sums over N*Ho*Wo products: tolerance relative to the size of the sum of magnitudes
+    n_terms = go.numel() // C
+    scale = float(n_terms) ** 0.5
+    rtol, atol = GRAD_TOL[dtype]
+    cabi.assert_close(gw, wgw, rtol, atol * scale, what="grad_weight")
+    cabi.assert_close(gb, wgb, rtol, atol * scale, what="grad_bias")
+    # skipping outputs leaves them alone and gives the same values for the others
+    gx2, gw2, gb2 = cabi.depthwise_backward(xd, wd, god, pad, with_bias=False)
+    assert gb2 is None and torch.equal(gx2, gx) and torch.equal(gw2, gw)
+
+
+def test_depthwise_conv_rejects_unsupported_kernels():
+    x = torch.zeros(1, 4, 4, 8, device="cuda")
+    with pytest.raises(ValueError, match="kernel size"):
+        cabi.depthwise_forward(x, torch.zeros(8, 2, 2, device="cuda"), None, 0)
+    with pytest.raises(ValueError, match="padding"):
+        cabi.depthwise_forward(x, torch.zeros(8, 3, 3, device="cuda"), None, 3)

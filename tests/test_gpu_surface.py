@@ -20,6 +20,14 @@ def _rel_err(a, b):
     return float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
 
 
+class DepthwiseOnCpu:
+    """The reference's formulation of the offset_mask_dw layer (modules/dcnv4.py:121-123) for CPU re-evaluation."""
+
+    @staticmethod
+    def apply(inp, weight, bias, pad):
+        return F.conv2d(inp.permute(0, 3, 1, 2), weight, bias, stride=1, padding=pad, groups=inp.shape[-1]).permute(0, 2, 3, 1)
+
+
 def test_dcnv4_function_autograd_matches_grid_sample_autograd():
     import dcnv4_amd
     B, H, W, G, D = 2, 12, 10, 4, 16
@@ -311,6 +319,7 @@ def test_small_flash_intern_image_matches_the_same_network_on_the_torch_core(mon
         feats = [f.cpu() for f in model.forward_features_seq_out(x.cuda())]
         model.cpu()
         monkeypatch.setattr(dcnv4_module, "DCNv4Function", CoreOnCpu)
+        monkeypatch.setattr(dcnv4_module, "DepthwiseConvNHWCFunction", DepthwiseOnCpu)
         want = model(x)
     assert got.shape == (2, 10) and [tuple(f.shape) for f in feats] == [(2, 32, 16, 16), (2, 64, 8, 8)]
     assert _rel_err(got, want) < 1e-3
@@ -344,6 +353,7 @@ def test_dense_prediction_backbone_returns_per_level_maps_for_a_non_square_input
         got = [f.cpu() for f in model.cuda()(x.cuda())]
         model.cpu()
         monkeypatch.setattr(dcnv4_module, "DCNv4Function", CoreOnCpu)
+        monkeypatch.setattr(dcnv4_module, "DepthwiseConvNHWCFunction", DepthwiseOnCpu)
         want = model(x)
     assert [tuple(f.shape) for f in got] == [(2, 32, 8, 12), (2, 64, 4, 6), (2, 128, 2, 3)]
     for g, w in zip(got, want):

@@ -274,3 +274,53 @@ def test_fp32_coordinate_mode_tracks_the_float64_mode(oracle):
     ga = oracle.flash_deform_attn_backward(v, shp.numpy(), start.numpy(), s, g, 4)
     gb = oracle.flash_deform_attn_backward(v, shp.numpy(), start.numpy(), s, g, 4, coord_f32=True)
     assert np.abs(ga[0] - gb[0]).max() < 2e-4 and np.abs(ga[1] - gb[1]).max() < 5e-3
+
+
+# ---------------------------------------------------------------- depthwise convolution oracle (oracle/depthwise.py)
+DW_CASES = [
+    # N, H, W, C, k, pad
+    (2, 7, 9, 6, 3, 1),
+    (1, 5, 6, 4, 3, 0),
+    (1, 6, 5, 3, 3, 2),
+    (2, 8, 7, 5, 5, 2),
+    (1, 9, 9, 2, 7, 3),
+    (1, 4, 4, 8, 1, 0),
+]
+
+
+@pytest.mark.parametrize("case", DW_CASES)
+def test_depthwise_oracle_matches_torch_conv2d_and_autograd(case):
+    """The reference's layer IS nn.Conv2d(groups=C) between two permutes (modules/dcnv4.py:67-75,121-123)."""
+    from oracle import depthwise
+    N, H, W, C, k, pad = case
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(N, H, W, C, dtype=torch.float64, generator=g, requires_grad=True)
+    w = torch.randn(C, 1, k, k, dtype=torch.float64, generator=g, requires_grad=True)
+    b = torch.randn(C, dtype=torch.float64, generator=g, requires_grad=True)
+    out = F.conv2d(x.permute(0, 3, 1, 2), w, b, stride=1, padding=pad, groups=C).permute(0, 2, 3, 1)
+    go = torch.randn(out.shape, dtype=torch.float64, generator=g)
+    out.backward(go)
+    got = depthwise.depthwise_forward(x.detach().numpy(), w.detach().numpy(), b.detach().numpy(), pad)
+    np.testing.assert_allclose(got, out.detach().numpy(), rtol=1e-12, atol=1e-12)
+    gx, gw, gb = depthwise.depthwise_backward(x.detach().numpy(), w.detach().numpy(), go.numpy(), pad)
+    np.testing.assert_allclose(gx, x.grad.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(gw, w.grad.numpy().reshape(C, k, k), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(gb, b.grad.numpy(), rtol=1e-12, atol=1e-12)
+
+
+def test_depthwise_one_hot_kernel_is_a_shifted_copy_and_ones_kernel_a_box_sum():
+    """Pins the tap orientation (i = row, j = column) and the sign of the padding shift."""
+    from oracle import depthwise
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((1, 6, 7, 2))
+    w = np.zeros((2, 3, 3))
+    w[0, 0, 2] = 1.0            # channel 0 reads the pixel one row up, one column right
+    w[1, 2, 1] = 1.0            # channel 1 reads the pixel one row down
+    out = depthwise.depthwise_forward(x, w, None, 1)
+    want0 = np.zeros((6, 7)); want0[1:, :-1] = x[0, :-1, 1:, 0]
+    want1 = np.zeros((6, 7)); want1[:-1, :] = x[0, 1:, :, 1]
+    np.testing.assert_array_equal(out[0, :, :, 0], want0)
+    np.testing.assert_array_equal(out[0, :, :, 1], want1)
+    box = depthwise.depthwise_forward(x, np.ones((2, 3, 3)), np.array([0.5, -1.0]), 1)
+    assert np.isclose(box[0, 2, 3, 0], x[0, 1:4, 2:5, 0].sum() + 0.5)
+    assert np.isclose(box[0, 0, 0, 1], x[0, 0:2, 0:2, 1].sum() - 1.0)      # corner: zeros outside
