@@ -352,11 +352,21 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
 #pragma unroll
           for (int cn = 0; cn < 4; ++cn) {
             unsigned long long *dst = acc + __umul24(cells[cn], (uint32_t)DP) + c;
-            const double wd = (double)wv[cn];
+            if constexpr (Tag::kBytes == 4) {
+              const double wd = (double)wv[cn];
 #pragma unroll
-            for (int j = 0; j < CPL; ++j)
-              __hip_atomic_fetch_add(dst + ch_off[j], fixed_product((double)gn[j], wd), __ATOMIC_RELAXED,
-                                     __HIP_MEMORY_SCOPE_WORKGROUP);
+              for (int j = 0; j < CPL; ++j)
+                __hip_atomic_fetch_add(dst + ch_off[j], fixed_product((double)gn[j], wd), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_WORKGROUP);
+            } else {
+              // 16-bit tensors carry 8-11 significant bits: terms below 2^31 (fix_bits <= 30), truncated
+#pragma unroll
+              for (int j = 0; j < CPL; ++j) {
+                const int t = (int)(gn[j] * wv[cn]);
+                __hip_atomic_fetch_add(dst + ch_off[j], ((unsigned long long)(uint32_t)(t >> 31) << 32) | (uint32_t)t,
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+              }
+            }
           }
         }
         __syncthreads();
