@@ -13,11 +13,14 @@
 //       A  tap-parallel: one lane per (pixel, group, kernel tap) recomputes the sampling position
 //          and, when a corner lands inside the tile, appends a hit record (four accumulator cells,
 //          four weights, pixel) to a per-group list in LDS; the strip's grad_out is parked in LDS;
-//       B  channel-parallel: a row of 8 lanes takes one hit record, lane c owns channels c, c+8, ...
-//          and adds its four corner contributions with 64-bit integer LDS atomics on fixed-point
-//          values.  The 8 rows of a wave are dealt evenly to the groups of the chunk, and the second
-//          row of a group walks its channels in the opposite order, so with 16 channels per group
-//          one ds_add_u64 instruction touches 64 distinct channels: two conflict-free bank sweeps;
+//       B  channel-parallel: a row of R lanes (2 for groups of up to 16 channels, 4 up to 32, 8 up to
+//          64) takes one hit record, lane c owns the CPL consecutive channels from c * CPL and adds
+//          its four corner contributions with 64-bit integer LDS atomics on fixed-point values.  Few
+//          lanes per record keep the per-record work (reading and unpacking it) small next to the
+//          adds.  The 64 / R rows of a wave are dealt evenly to the groups of the chunk, and the n-th
+//          row of a group starts its walk over the lane's channels at the n-th, so the rows of one
+//          ds_add_u64 instruction spread evenly over the banks: two bank sweeps, the least 64 lanes of
+//          8 bytes can take;
 //   * fixed point: contributions are normalised by the global maxima of |grad_out| and
 //     |modulation| (GradState, produced by the grad_offset_mask kernel that runs first) and carry
 //     `fix_bits` fractional bits (up to 50; each product is exact in double precision and rounded
@@ -34,7 +37,6 @@ namespace dcn {
 namespace {
 
 constexpr int kValThreads = 1024;
-constexpr int kRow = 8;               // lanes that apply one hit record
 constexpr int kWaves = kValThreads / kWave;
 constexpr int kTrashPad = 64;
 constexpr int kMaxChunkGroups = 4;      // rows of a wave <-> groups of the chunk
@@ -51,20 +53,22 @@ struct HitMeta {
   uint32_t cell3_px;    // cell of corner 3 | strip-local pixel << 9
 };
 
-// channels per lane for a group of D channels: 1, 2, 4 or 8 (odd counts round up)
+// lanes that apply one hit record, and channels per lane (1, 2, 4 or 8; odd counts round up)
+__host__ __device__ inline int lanes_per_record(int D) { return D <= 16 ? 2 : (D <= 32 ? 4 : 8); }
 __host__ __device__ inline int channels_per_lane(int D) {
-  const int c = (D + kRow - 1) / kRow;
+  const int r = lanes_per_record(D), c = (D + r - 1) / r;
   return c <= 2 ? c : (c <= 4 ? 4 : 8);
 }
 
-// Accumulator words per cell.  PACK (16-bit tensors): one 64-bit word holds two 32-bit fixed-point
-// sums, the lane's channels c + 16k (low half) and c + 8 + 16k (high half); a group then takes
-// 4 * CPL words.  Otherwise one word per channel.
+// Accumulator words per cell, channels in their natural order.  PACK (16-bit tensors): one 64-bit word
+// holds two 32-bit fixed-point sums, channels 2w (low half) and 2w + 1 (high half).  Otherwise one word
+// per channel.
+__host__ __device__ inline int acc_words_per_group(int D, bool pack) { return pack ? (D + 1) / 2 : D; }
 __host__ __device__ inline int acc_words_per_cell(int ng_chunk, int D, bool pack) {
-  return pack ? ng_chunk * 4 * channels_per_lane(D) : ng_chunk * D;
+  return ng_chunk * acc_words_per_group(D, pack);
 }
 
-template <typename Tag, int KP, int CPL, bool PACK>
+template <typename Tag, int KP, int R, int CPL, bool PACK>
 __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const DcnLaunch p) {
   extern __shared__ unsigned long long lds64[];
   const int Kp = p.Kp, D = p.D, C = p.G * p.D;
@@ -77,8 +81,8 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   const int b = id / nty;
   const int g0 = chunk * p.ng_chunk, ng = min(p.ng_chunk, p.G - g0);
   const int ch_stride = p.ng_chunk * D;                 // channels of the chunk
-  const int acc_stride = PACK ? p.ng_chunk * 4 * CPL : ch_stride;       // accumulator words per cell
-  constexpr int kGroupWords = PACK ? 4 * CPL : 0;                       // PACK: words per group within a cell
+  const int group_words = acc_words_per_group(D, PACK);                 // accumulator words of a group within a cell
+  const int acc_stride = p.ng_chunk * group_words;                      // ... of a cell
   const int ty0 = ty << p.tile_h_log2, tx0 = tx << p.tile_w_log2;
   const int th = min(p.tile_h, p.H - ty0), tw = min(p.tile_w, p.W - tx0);
   const int n_cells = p.tile_h * p.tile_w;
@@ -110,10 +114,11 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   const int wo_lo = max(0, ceil_div_signed(tx0 - reach - cx0, p.sw));
   const int wo_hi = min(p.Wo, ceil_div_signed(tx0 + p.tile_w + reach - cx0, p.sw));
   const int nwx = wo_hi - wo_lo;
-  const int lane = threadIdx.x & (kWave - 1), c = lane & (kRow - 1);
-  static_assert(kWave / kRow == 2 * kMaxChunkGroups, "a wave holds two rows per group of a full chunk");
+  const int lane = threadIdx.x & (kWave - 1), c = lane & (R - 1);
+  static_assert(kWave / R >= kMaxChunkGroups, "a wave holds at least one row per group of a full chunk");
+  static_assert(!PACK || CPL % 2 == 0, "packed sums pair the channels of one lane");
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int row_in_wave = lane / kRow;
+  const int row_in_wave = lane / R;
   const float x_sub = mul_rn((float)half_w, p.offset_scale), y_sub = mul_rn((float)half_h, p.offset_scale);
   typedef typename RawWord<Tag::kBytes>::type elem_t;
   const elem_t *om_g = reinterpret_cast<const elem_t *>(p.offset_mask);
@@ -279,59 +284,62 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       if (npx_next > 0) pf = prefetch(s_idx + 1, npx_next);
       if (threadIdx.x < kMaxChunkGroups) s_count[((s_idx + 1) & 1) * kMaxChunkGroups + threadIdx.x] = 0u;
 
-      // ---- phase B: a row of 8 lanes applies one hit record; lane c owns channels c, c+8, ... (CPL of them).
-      // The 8 rows of a wave are split evenly over the chunk's groups (two rows per group for a full
-      // chunk); the second row of a group walks its channels in the opposite order, so with 16 channels
-      // per group every ds_add_u64 instruction of the wave touches 64 distinct channels.
-      const int rows_per_group = (kWave / kRow) / p.ng_chunk;            // 2, 4 or 8
+      // ---- phase B: a row of R lanes applies one hit record; lane c owns channels c * CPL .. c * CPL + CPL - 1.
+      // The rows of a wave are split evenly over the chunk's groups; row n of a group visits its lane's
+      // channels (channel pairs when packed) starting from the n-th, so the rows that work for one group
+      // touch different words in every instruction.
+      constexpr int kUnits = PACK ? CPL / 2 : CPL;                       // accumulator words per lane
+      const int rows_per_group = (kWave / R) / p.ng_chunk;
       const int my_group = row_in_wave / rows_per_group, my_slot = row_in_wave - my_group * rows_per_group;
       const bool group_live = my_group < ng;
       const uint32_t n_mine = group_live ? count[my_group] : 0u;
       uint32_t n_max = count[0];
       for (int g = 1; g < ng; ++g) n_max = max(n_max, count[g]);
       const int lane_group = group_live ? my_group : 0;                  // idle rows only ever add zeros to the trash slots
-      const bool flip = (my_slot & 1) != 0;
-      unsigned long long *acc_lane = acc + (PACK ? lane_group * kGroupWords : lane_group * D) + c;
-      const float *go_lane = s_go + lane_group * D + c;
+      unsigned long long *acc_lane = acc + lane_group * group_words + c * kUnits;
+      const float *go_lane = s_go + lane_group * D + c * CPL;
+      int unit_of[kUnits];                                               // this row's visiting order
+#pragma unroll
+      for (int u = 0; u < kUnits; ++u) unit_of[u] = (u + my_slot) & (kUnits - 1);
       for (uint32_t i0 = wave * rows_per_group; i0 < n_max; i0 += kWaves * rows_per_group) {
         const uint32_t i = i0 + my_slot;
         f32x4 w = {0.f, 0.f, 0.f, 0.f};
         HitMeta meta = {(uint32_t)n_cells | ((uint32_t)n_cells << kCellBits) | ((uint32_t)n_cells << (2 * kCellBits)),
                         (uint32_t)n_cells};
-        if (i < n_mine) {
-          w = hit_w[lane_group * list_cap + i];
-          meta = hit_meta[lane_group * list_cap + i];
-        }
-        const int px = meta.cell3_px >> kCellBits;
-        float gn[CPL];
-        int ch_off[CPL];
-#pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-          ch_off[j] = kRow * ((flip && !PACK) ? CPL - 1 - j : j);
-          gn[j] = (c + ch_off[j] < D) ? go_lane[px * ch_stride + ch_off[j]] : 0.f;
-        }
+        if (i >= n_mine) continue;        // rows past the end of their group's list sit this pass out
+        w = hit_w[lane_group * list_cap + i];
+        meta = hit_meta[lane_group * list_cap + i];
+        const float *go_px = go_lane + (meta.cell3_px >> kCellBits) * ch_stride;
         const uint32_t cells[4] = {meta.cells012 & 511u, (meta.cells012 >> kCellBits) & 511u,
                                    (meta.cells012 >> (2 * kCellBits)) & 511u, meta.cell3_px & 511u};
         const float wv[4] = {w.x, w.y, w.z, w.w};
+        unsigned long long *dst[4];
 #pragma unroll
-        for (int cn = 0; cn < 4; ++cn) {
-          unsigned long long *dst = acc_lane + __umul24(cells[cn], (uint32_t)acc_stride);
-          if constexpr (PACK) {
-            // two channels per atomic: sum = hi * 2^32 + lo with both halves signed, so the low term is
-            // sign-extended into the high word before the add
+        for (int cn = 0; cn < 4; ++cn) dst[cn] = acc_lane + __umul24(cells[cn], (uint32_t)acc_stride);
+        if constexpr (PACK) {
+          // two channels per atomic: sum = hi * 2^32 + lo with both halves signed, so the low term is
+          // sign-extended into the high word before the add
 #pragma unroll
-            for (int j = 0; j < CPL; j += 2) {
-              const int lo = to_fixed32(gn[j], wv[cn]);
-              const int hi = j + 1 < CPL ? to_fixed32(gn[j + 1], wv[cn]) : 0;
+          for (int u = 0; u < kUnits; ++u) {
+            const int ch = 2 * unit_of[u];
+            const float g_lo = (c * CPL + ch < D) ? go_px[ch] : 0.f;
+            const float g_hi = (c * CPL + ch + 1 < D) ? go_px[ch + 1] : 0.f;
+#pragma unroll
+            for (int cn = 0; cn < 4; ++cn) {
+              const int lo = to_fixed32(g_lo, wv[cn]), hi = to_fixed32(g_hi, wv[cn]);
               const unsigned long long v = ((unsigned long long)(uint32_t)(hi + (lo >> 31)) << 32) | (uint32_t)lo;
-              __hip_atomic_fetch_add(dst + (j / 2) * kRow, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+              __hip_atomic_fetch_add(dst[cn] + unit_of[u], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
-          } else {
-            const double wd = (double)wv[cn];
+          }
+        } else {
+          const double wd[4] = {(double)wv[0], (double)wv[1], (double)wv[2], (double)wv[3]};
 #pragma unroll
-            for (int j = 0; j < CPL; ++j)
-              __hip_atomic_fetch_add(dst + ch_off[j], fixed_product((double)gn[j], wd), __ATOMIC_RELAXED,
-                                     __HIP_MEMORY_SCOPE_WORKGROUP);
+          for (int u = 0; u < kUnits; ++u) {
+            const int ch = unit_of[u];
+            const double gd = (c * CPL + ch < D) ? (double)go_px[ch] : 0.0;
+#pragma unroll
+            for (int cn = 0; cn < 4; ++cn)
+              __hip_atomic_fetch_add(dst[cn] + ch, fixed_product(gd, wd[cn]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
           }
         }
       }
@@ -352,10 +360,10 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
     for (int ch = lane; ch < n_ch; ch += kWave) {
       float f[1];
       if constexpr (PACK) {
-        const int g = ch / D, cg = ch - g * D, j = cg / kRow;
-        const unsigned long long a = src[g * kGroupWords + (j >> 1) * kRow + (cg & (kRow - 1))];
+        const int g = ch / D, cg = ch - g * D;
+        const unsigned long long a = src[g * group_words + (cg >> 1)];
         const int lo = (int)(uint32_t)a;
-        const int field = (j & 1) ? (int)(uint32_t)(a >> 32) + (lo < 0 ? 1 : 0) : lo;
+        const int field = (cg & 1) ? (int)(uint32_t)(a >> 32) + (lo < 0 ? 1 : 0) : lo;
         f[0] = ldexpf((float)field, e_out);
       } else {
         const unsigned long long a = src[ch];
@@ -385,19 +393,21 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
     return hipGetLastError();
   };
-  const int cpl = channels_per_lane(p.D);
+  const int r = lanes_per_record(p.D), cpl = channels_per_lane(p.D);
   constexpr bool kCanPack = Tag::kBytes == 2;
 #define GV_CASE(KPV)                                                                        \
   do {                                                                                      \
     if constexpr (kCanPack) {                                                               \
-      if (p.pack32 && cpl == 2) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, true>);      \
-      if (p.pack32 && cpl == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, true>);      \
-      if (p.pack32 && cpl == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, true>);      \
+      if (p.pack32 && r == 2 && cpl == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, true>);   \
+      if (p.pack32 && r == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, 8, true>);     \
+      if (p.pack32 && r == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, 8, true>);     \
     }                                                                                       \
-    if (cpl == 1) return go(dcnv4_grad_value_kernel<Tag, KPV, 1, false>);                   \
-    if (cpl == 2) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, false>);                   \
-    if (cpl == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, false>);                   \
-    return go(dcnv4_grad_value_kernel<Tag, KPV, 8, false>);                                 \
+    if (r == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, 8, false>);                  \
+    if (r == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, 8, false>);                  \
+    if (cpl == 1) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 1, false>);                \
+    if (cpl == 2) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 2, false>);                \
+    if (cpl == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 4, false>);                \
+    return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, false>);                              \
   } while (0)
   if (k3 && !p.remove_center) GV_CASE(9);
   if (k3 && p.remove_center) GV_CASE(8);
