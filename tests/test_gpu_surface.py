@@ -358,3 +358,39 @@ def test_dense_prediction_backbone_returns_per_level_maps_for_a_non_square_input
     assert [tuple(f.shape) for f in got] == [(2, 32, 8, 12), (2, 64, 4, 6), (2, 128, 2, 3)]
     for g, w in zip(got, want):
         assert _rel_err(g, w) < 1e-3
+
+
+def test_dcnv4_module_under_autocast_runs_the_half_kernels_and_returns_fp32_parameter_gradients():
+    """AMP wiring of both autograd Functions (torch.amp.custom_fwd / custom_bwd, device_type="cuda"): activations
+    in fp16 inside the module, fp32 parameters and fp32 parameter gradients outside, values within fp16 tolerance of
+    the fp32 run."""
+    import dcnv4_amd
+    torch.manual_seed(4)
+    C, G, H, W, N = 64, 4, 10, 9, 2
+    m = dcnv4_amd.DCNv4(channels=C, group=G, dw_kernel_size=3).cuda()
+    with torch.no_grad():
+        m.offset_mask.weight.normal_(0, 0.3)
+        m.offset_mask.bias.normal_(0, 0.5)
+    x = torch.randn(N, H * W, C, device="cuda")
+    ref = m(x.clone().requires_grad_(True), shape=(H, W))
+    ref.sum().backward()
+    ref_grads = {k: p.grad.clone() for k, p in m.named_parameters()}
+    m.zero_grad()
+    seen = []
+    real = dcnv4_amd.ext.dcnv4_forward
+    try:
+        dcnv4_amd.ext.dcnv4_forward = lambda v, om, *a: (seen.append((v.dtype, om.dtype)), real(v, om, *a))[1]
+        xa = x.clone().requires_grad_(True)
+        with torch.autocast(device_type="cuda", dtype=torch.float16):
+            out = m(xa, shape=(H, W))
+        out.float().sum().backward()
+    finally:
+        dcnv4_amd.ext.dcnv4_forward = real
+    assert seen == [(torch.float16, torch.float16)]
+    assert out.dtype == torch.float16 and xa.grad.dtype == torch.float32
+    assert _rel_err(out.float().cpu(), ref.detach().cpu()) < 1e-2
+    for k, p in m.named_parameters():
+        assert p.grad is not None and p.grad.dtype == torch.float32, k
+        # gradients that pass through the sampling positions see the fp16 rounding of the offsets
+        tol = 0.15 if k.startswith("offset_mask") else 3e-2
+        assert _rel_err(p.grad.cpu(), ref_grads[k].cpu()) < tol, k

@@ -141,3 +141,44 @@ def test_flash_intern_image_state_dict_uses_the_reference_key_names():
     assert "levels.3.downsample.conv.weight" not in keys and "levels.0.norm.0.weight" not in keys   # post_norm variant
     t_keys = set(flash_intern_image("t").state_dict())
     assert "levels.0.norm.0.weight" in t_keys and "levels.0.blocks.0.gamma1" not in t_keys
+
+
+@pytest.mark.parametrize("variant", ["t", "s", "b", "l"])
+def test_model_state_dict_equals_the_schema_written_from_the_reference_definitions(variant):
+    """Names, shapes and order of every parameter and buffer, both ways (classification/models/flash_intern_image.py)."""
+    from dcnv4_amd.models import check_state_dict, flash_intern_image, reference_schema
+    schema = reference_schema(variant)
+    state = flash_intern_image(variant).state_dict()
+    assert check_state_dict(state, schema) == []
+    assert list(state) == list(schema)
+
+
+def test_offset_mask_projection_is_padded_to_a_multiple_of_eight():
+    from dcnv4_amd.models import offset_mask_features, reference_schema
+    assert [offset_mask_features(g) for g in (4, 7, 5, 10, 56)] == [112, 192, 136, 272, 1512]   # 108, 189, 135, 270, 1512
+    assert reference_schema("b")["levels.0.blocks.0.dcn.offset_mask.weight"] == (192, 112)
+    assert reference_schema("t")["levels.3.blocks.3.dcn.offset_mask.bias"] == (864,)
+
+
+def test_checkpoint_in_the_reference_file_layout_loads_and_misfits_are_named(tmp_path):
+    from dcnv4_amd.models import FlashInternImage, check_state_dict, load_checkpoint, reference_schema
+    kw = dict(channels=16, depths=(1, 1), groups=(1, 2), layer_scale=1e-5, post_norm=True, dw_kernel_size=3, num_classes=5)
+    src, dst = FlashInternImage(**kw), FlashInternImage(**kw)
+    with torch.no_grad():
+        for p in src.parameters():
+            p.normal_()
+    path = tmp_path / "flash_intern_image_tiny.pth"
+    torch.save({"model": {"module." + k: v for k, v in src.state_dict().items()}, "epoch": 3}, path)   # classification/utils.py layout
+    assert load_checkpoint(dst, path) == []
+    assert all(torch.equal(a, b) for a, b in zip(src.state_dict().values(), dst.state_dict().values()))
+    # a checkpoint whose offset_mask projection was saved without the padding is reported, with the reason
+    bad = dict(src.state_dict())
+    bad["levels.0.blocks.0.dcn.offset_mask.weight"] = bad["levels.0.blocks.0.dcn.offset_mask.weight"][:27]
+    del bad["head.bias"]
+    bad["extra.weight"] = torch.zeros(1)
+    problems = check_state_dict(bad, {k: tuple(v.shape) for k, v in dst.state_dict().items()})
+    assert len(problems) == 3 and any("multiple of 8" in p for p in problems) and any("missing key head.bias" in p for p in problems)
+    assert any("unexpected key extra.weight" in p for p in problems)
+    torch.save({"model": bad}, path)
+    with pytest.raises(RuntimeError, match="does not fit"):
+        load_checkpoint(dst, path)
