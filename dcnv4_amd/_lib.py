@@ -20,6 +20,7 @@ _vp, _i, _f, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_
 SIGNATURES = {
     "dcnv4_gfx950_abi_version": (_i, []),
     "dcnv4_gfx950_last_error": (ctypes.c_char_p, []),
+    "dcnv4_gfx950_set_launch_option": (_i, [ctypes.c_char_p, _i]),
     "dcnv4_gfx950_forward": (_i, [_vp, _vp, _vp, _i] + [_i] * 13 + [_f] + [_i] * 6 + [_vp]),
     "dcnv4_gfx950_backward_workspace_bytes": (_sz, [_i] * 6),
     "dcnv4_gfx950_backward": (_i, [_vp] * 6 + [_sz, _i] + [_i] * 13 + [_f] + [_i] * 6 + [_vp]),

@@ -121,14 +121,21 @@ __global__ void init_state_kernel(GradState *st) {
 constexpr size_t kStateBytes = 256;     // GradState, padded
 constexpr int kTiledMaxGroupChannels = 64;
 
-bool tiled_grad_value(int D) { return D <= kTiledMaxGroupChannels; }
+// Per-thread launch options (dcnv4_gfx950_set_launch_option); 0 = not set: the environment variable of the
+// same purpose decides, then the library's default.
+enum { kOptAuto = 0, kOptTiled = 1, kOptPlain = 2 };
+thread_local int g_opt_gather = kOptAuto;       // LDS-tiled / direct gathers (forward, grad_offset_mask)
+thread_local int g_opt_scatter = kOptAuto;      // tiled LDS accumulation / global atomics (grad_value)
+thread_local int g_opt_reach = 0;               // 0 = not set, else reach + 1
+
+bool tiled_grad_value(int D) { return D <= kTiledMaxGroupChannels && g_opt_scatter != kOptPlain; }
 
 // Tuning override, read on every call: DCNV4_GFX950_REACH = distance (input pixels) from an output
 // pixel's reference point that the tiled kernels cover; sampling points beyond it take the
 // global-memory paths.  Default 5.
 int reach_setting() {
   const char *e = getenv("DCNV4_GFX950_REACH");
-  const int r = e ? atoi(e) : 5;
+  const int r = g_opt_reach > 0 ? g_opt_reach - 1 : (e ? atoi(e) : 5);
   return r < 0 ? 0 : (r > 64 ? 64 : r);
 }
 
@@ -140,6 +147,7 @@ bool fda_tiled_shape(int D, int L, int Q, int K) {
 
 // Tuning override, read on every call: DCNV4_GFX950_FDA_SCATTER=atomic keeps the fp32 atomic scatter.
 bool fda_tiled_enabled() {
+  if (g_opt_scatter != kOptAuto) return g_opt_scatter == kOptTiled;
   const char *e = getenv("DCNV4_GFX950_FDA_SCATTER");
   return !(e && strcmp(e, "atomic") == 0);
 }
@@ -188,6 +196,7 @@ int plan_grad_value_tiles(DcnLaunch *L, int elem_bytes_of_launch) {
 // Tuning override, read on every call: DCNV4_GFX950_GATHER=direct keeps the gathers on the
 // global-memory kernels.
 bool tiled_gather_enabled() {
+  if (g_opt_gather != kOptAuto) return g_opt_gather == kOptTiled;
   const char *e = getenv("DCNV4_GFX950_GATHER");
   return !(e && strcmp(e, "direct") == 0);
 }
@@ -447,6 +456,16 @@ extern "C" {
 int dcnv4_gfx950_abi_version(void) { return DCNV4_GFX950_ABI_VERSION; }
 
 const char *dcnv4_gfx950_last_error(void) { return g_error; }
+
+int dcnv4_gfx950_set_launch_option(const char *name, int value) {
+  if (name == nullptr) return fail(DCNV4_ERR_INVALID_ARGUMENT, "null option name");
+  const bool family = value == kOptAuto || value == kOptTiled || value == kOptPlain;
+  if (std::strcmp(name, "gather") == 0 && family) g_opt_gather = value;
+  else if (std::strcmp(name, "scatter") == 0 && family) g_opt_scatter = value;
+  else if (std::strcmp(name, "reach") == 0 && value >= -1 && value <= 64) g_opt_reach = value + 1;
+  else return fail(DCNV4_ERR_INVALID_ARGUMENT, "unknown launch option %s = %d", name, value);
+  return DCNV4_OK;
+}
 
 int dcnv4_gfx950_forward(const void *value, const void *offset_mask, void *output, int dtype, int batch,
                          int height_in, int width_in, int group, int group_channels, int kernel_h,

@@ -40,6 +40,29 @@ def _hint(v):
     return int(v) if v is not None else 0
 
 
+_FAMILY = {"auto": 0, "tiled": 1, "direct": 2, "atomic": 2}
+
+
+class launch_options:
+    """Context manager over the calling thread's launch options (include/dcnv4_gfx950.h,
+    ``dcnv4_gfx950_set_launch_option``): ``gather`` in auto / tiled / direct, ``scatter`` in auto / tiled / atomic,
+    ``reach`` an int or None.  Used by the tuner and by dispatch-table entries that carry options; the options are
+    back at the library's choice on exit.  Results do not depend on them beyond the rounding of sums."""
+
+    def __init__(self, gather="auto", scatter="auto", reach=None):
+        self.values = {"gather": _FAMILY[gather], "scatter": _FAMILY[scatter], "reach": -1 if reach is None else int(reach)}
+
+    def __enter__(self):
+        for name, value in self.values.items():
+            _lib.check(_L.dcnv4_gfx950_set_launch_option(name.encode(), value))
+        return self
+
+    def __exit__(self, *exc):
+        for name in self.values:
+            _L.dcnv4_gfx950_set_launch_option(name.encode(), -1 if name == "reach" else 0)
+        return False
+
+
 def _out_hw(h, w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w):
     return ((h + 2 * pad_h - (dilation_h * (kernel_h - 1) + 1)) // stride_h + 1,
             (w + 2 * pad_w - (dilation_w * (kernel_w - 1) + 1)) // stride_w + 1)

@@ -8,7 +8,7 @@ from torch.autograd import Function
 from torch.autograd.function import once_differentiable
 
 from .. import ext
-from .launch_spec import find_spec_bwd, findspec
+from .launch_spec import find_spec_bwd, findspec, launch_options_for
 
 
 class DCNv4Function(Function):
@@ -25,8 +25,13 @@ class DCNv4Function(Function):
         ctx.remove_center = remove_center
         ctx.backward_d_stride = bwd_d_stride
         ctx.backward_block_thread = bwd_threads
-        output = ext.dcnv4_forward(input, offset_mask, *ctx.geometry, remove_center, fwd_d_stride,
-                                   fwd_threads, False)
+        ctx.backward_options = launch_options_for(B, H, W, group, group_channels, es, "bwd")
+        options = launch_options_for(B, H, W, group, group_channels, es, "fwd")
+        if options:        # a tuned table entry that names kernel families
+            with ext.launch_options(**options):
+                output = ext.dcnv4_forward(input, offset_mask, *ctx.geometry, remove_center, fwd_d_stride, fwd_threads, False)
+        else:
+            output = ext.dcnv4_forward(input, offset_mask, *ctx.geometry, remove_center, fwd_d_stride, fwd_threads, False)
         ctx.save_for_backward(input, offset_mask)
         return output
 
@@ -35,7 +40,11 @@ class DCNv4Function(Function):
     @custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
         input, offset_mask = ctx.saved_tensors
-        grad_input, grad_offset_mask = ext.dcnv4_backward(
-            input, offset_mask, *ctx.geometry, grad_output.contiguous(), ctx.remove_center,
-            ctx.backward_d_stride, ctx.backward_block_thread, False)
+        args = (input, offset_mask, *ctx.geometry, grad_output.contiguous(), ctx.remove_center,
+                ctx.backward_d_stride, ctx.backward_block_thread, False)
+        if ctx.backward_options:
+            with ext.launch_options(**ctx.backward_options):
+                grad_input, grad_offset_mask = ext.dcnv4_backward(*args)
+        else:
+            grad_input, grad_offset_mask = ext.dcnv4_backward(*args)
         return (grad_input, grad_offset_mask) + (None,) * 13

@@ -1,18 +1,41 @@
-"""Launch hints for gfx950, the counterpart of the reference's ``findspec`` / ``find_spec_bwd``
+"""Launch specs for gfx950, the counterpart of the reference's ``findspec`` / ``find_spec_bwd``
 (DCNv4_op/DCNv4/functions/dcnv4_func.py:21-60, flash_deform_attn_func.py:38-67) and of its
 NVIDIA-tuned ``table.py``.
 
 A spec is ``(d_stride, n_thread)``: channels per lane and lanes per workgroup.  On gfx950 a lane
 always moves 16 bytes when the group width allows it, and a workgroup is sized to roughly 256
-lanes made of whole pixels; both follow in O(1) from (G, C, element size), so there is no factor
-scan over B*H*W and nothing to memoise.  ``GFX950_TABLE`` holds measured overrides keyed like the
-reference's table (``"BxHxWxGxC"``); entries are optional.
-"""
+lanes made of whole pixels; both follow in O(1) from (G, C, element size), and the answer is
+memoised per shape, so a call costs one dictionary look-up (the reference scans the factors of
+B*H*W on every call).
 
-GFX950_TABLE = {}
-GFX950_BWD_TABLE = {}
+Measured overrides live in ``gfx950_table.json`` next to this file, written by ``python -m dcnv4_amd.tune``
+(the counterpart of DCNv4_op/scripts/search_dcnv4.py, search_dcnv4_bwd.py and find_best.py).  Its keys are the
+reference's ``"BxHxWxGxC"`` plus the element size and the direction; an entry holds the two hints and, optionally,
+the kernel families to use (``gather`` = tiled / direct, ``scatter`` = tiled / atomic), which
+:func:`launch_options_for` hands to the library as thread-local launch options around the call.
+"""
+import functools
+import json
+import os
+
+TABLE_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gfx950_table.json")
 
 _TARGET_LANES = 256
+
+
+def _load_table(path=TABLE_PATH):
+    if not os.path.exists(path):
+        return {}
+    with open(path) as f:
+        return json.load(f).get("entries", {})
+
+
+# key -> {"d_stride": int, "n_thread": int, "gather": str (optional), "scatter": str (optional)}
+GFX950_TABLE = _load_table()
+
+
+def table_key(B, H, W, G, C, elem_bytes, direction):
+    return f"{B}x{H}x{W}x{G}x{C}:{elem_bytes}:{direction}"
 
 
 def _vector_channels(group_channels, elem_bytes):
@@ -33,18 +56,26 @@ def _spec(group, group_channels, elem_bytes, scatter=False):
     return d_stride, pixels * lanes_per_pixel
 
 
+@functools.lru_cache(maxsize=None)
+def _lookup(B, H, W, G, C, elem_bytes, direction):
+    entry = GFX950_TABLE.get(table_key(B, H, W, G, C, elem_bytes, direction))
+    if entry is not None:
+        options = {k: entry[k] for k in ("gather", "scatter") if entry.get(k, "auto") != "auto"}
+        return (int(entry["d_stride"]), int(entry["n_thread"])), options
+    return _spec(G, C, elem_bytes, scatter=direction == "bwd"), {}
+
+
 def findspec(B, H, W, G, C, elem_bytes=2):
-    key = f"{B}x{H}x{W}x{G}x{C}"
-    if key in GFX950_TABLE:
-        return GFX950_TABLE[key][0], GFX950_TABLE[key][1]
-    return _spec(G, C, elem_bytes)
+    return _lookup(B, H, W, G, C, elem_bytes, "fwd")[0]
 
 
 def find_spec_bwd(B, H, W, G, C, elem_bytes=2):
-    key = f"{B}x{H}x{W}x{G}x{C}"
-    if key in GFX950_BWD_TABLE:
-        return GFX950_BWD_TABLE[key][0], GFX950_BWD_TABLE[key][1]
-    return _spec(G, C, elem_bytes, scatter=True)
+    return _lookup(B, H, W, G, C, elem_bytes, "bwd")[0]
+
+
+def launch_options_for(B, H, W, G, C, elem_bytes, direction):
+    """Kernel-family options a table entry asks for ({} for shapes without an entry: the library chooses)."""
+    return _lookup(B, H, W, G, C, elem_bytes, direction)[1]
 
 
 def findspec_attn(B, Q, G, C, elem_bytes=2):

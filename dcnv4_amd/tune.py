@@ -1,0 +1,126 @@
+"""Launch-spec tuner for gfx950: ``python -m dcnv4_amd.tune [--shapes t,b,dense] [--dtypes float16,float32]``.
+
+Counterpart of the reference's DCNv4_op/scripts/search_dcnv4.py, search_dcnv4_bwd.py and find_best.py, which
+time every (d_stride, block_thread) pair per ``BxHxWxGxC`` and paste the winners into functions/table.py.
+Here the candidates are the kernel family (LDS-tiled or direct gathers; tiled LDS accumulation or global atomics
+for grad_value) and, for the direct family, the two hints; each is timed with HIP events through the same
+``dcnv4_amd.ext`` calls the autograd Function makes, and the winners go to ``functions/gfx950_table.json``, which
+``functions/launch_spec.py`` loads at import.  An entry is only written when it beats the library's own choice by
+more than ``--margin`` (default 3 %) and by more than ``--min-gain-us`` (default 10 us: applying an entry's
+kernel-family options costs a few microseconds of host time per call), so an empty table is a valid outcome.
+"""
+import argparse
+import json
+import math
+import sys
+import time
+
+SHAPES = {
+    # the reference's benchmark shapes (DCNv4_op/scripts/test_dcnv4.py:23-31, classification configs)
+    "t": [(64, 56, 56, 4, 16), (64, 28, 28, 8, 16), (64, 14, 14, 16, 16), (64, 7, 7, 32, 16)],
+    "b": [(128, 56, 56, 7, 16), (128, 28, 28, 14, 16), (128, 14, 14, 28, 16), (128, 7, 7, 56, 16)],
+    "dense": [(2, 256, 256, 10, 16), (2, 128, 128, 20, 16), (2, 64, 64, 40, 16), (2, 32, 32, 80, 16)],
+}
+GEOM = (3, 3, 1, 1, 1, 1, 1, 1)
+
+
+def _time(fn, iters, warm):
+    import torch
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def candidates(G, D, elem_bytes, direction):
+    """(label, options, d_stride, n_thread); the first one is the library's own choice."""
+    out = [("library", {}, 0, 0)]
+    if direction == "fwd":
+        widths = [c for c in (8, 4, 2) if D % c == 0 and c * elem_bytes <= 16]
+        for d in widths:
+            for n in (128, 256, 512):
+                out.append((f"direct d{d} n{n}", {"gather": "direct"}, d, n))
+    else:
+        out.append(("direct gathers", {"gather": "direct"}, 0, 0))
+        out.append(("atomic scatter", {"scatter": "atomic"}, 0, 0))
+        out.append(("direct gathers, atomic scatter", {"gather": "direct", "scatter": "atomic"}, 0, 0))
+    return out
+
+
+def tune(shape_sets, dtypes, iters=50, warm=10, margin=0.03, min_gain_us=10.0, offset_range=3.0, log=print):
+    import torch
+    from . import ext
+    dev = torch.device("cuda:0")
+    entries, report = {}, []
+    for set_name in shape_sets:
+        for B, H, W, G, D in SHAPES[set_name]:
+            C, K = G * D, 9
+            p_pad = int(math.ceil(G * K * 3 / 8) * 8)
+            for dt_name in dtypes:
+                dtype = getattr(torch, dt_name)
+                es = torch.empty(0, dtype=dtype).element_size()
+                value = torch.randn(B, H, W, C, device=dev).to(dtype)
+                om = torch.zeros(B, H, W, p_pad, device=dev)
+                om[..., :G * K * 3] = torch.cat([(torch.rand(B, H, W, G, 2 * K, device=dev) * 2 - 1) * offset_range,
+                                                 torch.randn(B, H, W, G, K, device=dev)], -1).reshape(B, H, W, G * K * 3)
+                om = om.to(dtype)
+                go = torch.randn(B, H, W, C, device=dev).to(dtype)
+                for direction in ("fwd", "bwd"):
+                    timings = []
+                    for label, options, d_stride, n_thread in candidates(G, D, es, direction):
+                        if direction == "fwd":
+                            call = lambda: ext.dcnv4_forward(value, om, *GEOM, G, D, 1.0, 64, 0, d_stride, n_thread, False)
+                        else:
+                            call = lambda: ext.dcnv4_backward(value, om, *GEOM, G, D, 1.0, 64, go, 0, d_stride, n_thread, False)
+                        with ext.launch_options(**options):
+                            ms = _time(call, iters, warm)
+                        timings.append((ms, label, options, d_stride, n_thread))
+                    base = timings[0][0]
+                    best = min(timings)
+                    key = f"{B}x{H}x{W}x{G}x{C}:{es}:{direction}"
+                    report.append({"key": key, "library_ms": round(base, 5), "best_ms": round(best[0], 5), "best": best[1]})
+                    log(f"{key:28s} library {base * 1e3:8.1f} us   best {best[0] * 1e3:8.1f} us  ({best[1]})")
+                    if best[0] < base * (1.0 - margin) and (base - best[0]) * 1e3 > min_gain_us:
+                        from .functions.launch_spec import _spec
+                        d, n = (best[3], best[4]) if best[3] else _spec(G, D, es, scatter=direction == "bwd")
+                        entries[key] = dict(d_stride=d, n_thread=n, **best[2])
+                del value, om, go
+    return entries, report
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--shapes", default="t,b,dense", help="comma-separated shape sets: " + ", ".join(SHAPES))
+    ap.add_argument("--dtypes", default="float16,float32")
+    ap.add_argument("--iters", type=int, default=50)
+    ap.add_argument("--margin", type=float, default=0.03)
+    ap.add_argument("--min-gain-us", type=float, default=10.0)
+    ap.add_argument("--out", default=None, help="table file (default: dcnv4_amd/functions/gfx950_table.json)")
+    ap.add_argument("--report", default=None, help="also write every timing to this JSON file")
+    args = ap.parse_args(argv)
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("the tuner needs an MI355X (torch.cuda.is_available() is False)")
+    from .functions import launch_spec
+    entries, report = tune(args.shapes.split(","), args.dtypes.split(","), iters=args.iters, margin=args.margin,
+                           min_gain_us=args.min_gain_us)
+    table = {"device": torch.cuda.get_device_name(0), "made": time.strftime("%Y-%m-%d"), "margin": args.margin,
+             "min_gain_us": args.min_gain_us, "entries": entries}
+    out = args.out or launch_spec.TABLE_PATH
+    with open(out, "w") as f:
+        json.dump(table, f, indent=1, sort_keys=True)
+    if args.report:
+        with open(args.report, "w") as f:
+            json.dump(report, f, indent=1)
+    print(f"{len(entries)} of {len(report)} cases beat the library's choice by more than {args.margin:.0%} and "
+          f"{args.min_gain_us:g} us; table written to {out}")
+
+
+if __name__ == "__main__":
+    main()

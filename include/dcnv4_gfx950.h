@@ -48,6 +48,22 @@ int dcnv4_gfx950_abi_version(void);
 const char *dcnv4_gfx950_last_error(void);
 
 /*
+ * Launch options of the calling thread, for tuners and for dispatch tables made by them; they play the
+ * part of the reference's per-shape launch table (DCNv4_op/DCNv4/functions/table.py, filled by
+ * DCNv4_op/scripts/search_dcnv4.py, search_dcnv4_bwd.py and find_best.py).  Results never depend on them
+ * beyond the rounding of sums.
+ *   "gather"   0 library's choice, 1 LDS-tiled gathers where the shape allows, 2 direct gathers
+ *              (forward and grad_offset_mask kernels)
+ *   "scatter"  0 library's choice, 1 tiled LDS accumulation where the shape allows, 2 global atomics
+ *              (grad_value of both operators; decides the workspace size as well)
+ *   "reach"    -1 library's choice, else 0..64: input pixels around an output pixel's reference point that
+ *              the tiled DCNv4 kernels cover
+ * An option that is not set falls back to the environment variable of the same purpose
+ * (DCNV4_GFX950_GATHER=direct, DCNV4_GFX950_FDA_SCATTER=atomic, DCNV4_GFX950_REACH=n).
+ */
+int dcnv4_gfx950_set_launch_option(const char *name, int value);
+
+/*
  * DCNv4 forward.  Replaces dcnv4_forward / dcnv4_cuda_forward
  * (DCNv4_op/src/dcnv4.h:64-83, DCNv4_op/src/cuda/dcnv4_cuda.cu:26-90).
  *   value        [batch, height_in, width_in, group*group_channels]

@@ -31,7 +31,7 @@ setup(
     version="0.1.0",
     description="DCNv4 and flash deformable attention operators for AMD MI355X (gfx950)",
     packages=find_packages(include=["dcnv4_amd", "dcnv4_amd.*", "DCNv4"]),
-    package_data={"dcnv4_amd": ["libdcnv4_gfx950.so", "csrc/*"]},
+    package_data={"dcnv4_amd": ["libdcnv4_gfx950.so", "csrc/*", "functions/gfx950_table.json"]},
     cmdclass={"build_ext": build_ext},
     python_requires=">=3.8",
 )

@@ -394,3 +394,25 @@ def test_dcnv4_module_under_autocast_runs_the_half_kernels_and_returns_fp32_para
         # gradients that pass through the sampling positions see the fp16 rounding of the offsets
         tol = 0.15 if k.startswith("offset_mask") else 3e-2
         assert _rel_err(p.grad.cpu(), ref_grads[k].cpu()) < tol, k
+
+
+@pytest.mark.parametrize("options", [dict(gather="direct"), dict(scatter="atomic"), dict(gather="direct", scatter="atomic"),
+                                     dict(gather="tiled", scatter="tiled", reach=2)])
+def test_launch_options_change_the_kernels_not_the_results(options):
+    """Thread-local launch options (what a tuned table entry applies around a call) against the library's own choice."""
+    import dcnv4_amd
+    from dcnv4_amd import ext
+    v, om, go = make_dcnv4_inputs(2, 20, 18, 4, 16, offset_range=3.0, seed=7, dtype=torch.float16)
+    v, om, go = v.cuda(), om.cuda(), go.cuda()
+    geom = (3, 3, 1, 1, 1, 1, 1, 1)
+    want = ext.dcnv4_forward(v, om, *geom, 4, 16, 1.0, 64, 0, 0, 0, False)
+    wgv, wgom = ext.dcnv4_backward(v, om, *geom, 4, 16, 1.0, 64, go, 0, 0, 0, False)
+    with ext.launch_options(**options):
+        out = ext.dcnv4_forward(v, om, *geom, 4, 16, 1.0, 64, 0, 8, 128, False)
+        gv, gom = ext.dcnv4_backward(v, om, *geom, 4, 16, 1.0, 64, go, 0, 0, 0, False)
+    assert _rel_err(out.float().cpu(), want.float().cpu()) < 2e-3
+    assert _rel_err(gv.float().cpu(), wgv.float().cpu()) < 1e-2
+    assert _rel_err(gom.float().cpu(), wgom.float().cpu()) < 2e-3
+    # the options are back at the library's choice afterwards: same bits as before
+    again = ext.dcnv4_backward(v, om, *geom, 4, 16, 1.0, 64, go, 0, 0, 0, False)
+    assert torch.equal(again[0], wgv) and torch.equal(again[1], wgom)

@@ -24,7 +24,7 @@ def test_library_exports_every_symbol_the_header_declares():
     from dcnv4_amd import _lib
     lib = ctypes.CDLL(_lib.LIB_PATH)
     declared = _declared_functions()
-    assert len(declared) == 11, sorted(declared)
+    assert len(declared) == 12, sorted(declared)
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in include/dcnv4_gfx950.h but not exported"
     assert set(declared) == set(_lib.SIGNATURES), "ctypes table and header list different functions"
@@ -182,3 +182,38 @@ def test_checkpoint_in_the_reference_file_layout_loads_and_misfits_are_named(tmp
     torch.save({"model": bad}, path)
     with pytest.raises(RuntimeError, match="does not fit"):
         load_checkpoint(dst, path)
+
+
+def test_launch_table_entries_reach_the_dispatcher_and_lookups_are_memoised(monkeypatch):
+    """A tuned entry (dcnv4_amd/tune.py output format) overrides the O(1) hints and carries kernel-family options."""
+    from dcnv4_amd.functions import launch_spec as ls
+    key = ls.table_key(3, 11, 13, 2, 32, 2, "fwd")
+    monkeypatch.setitem(ls.GFX950_TABLE, key, {"d_stride": 4, "n_thread": 128, "gather": "direct"})
+    ls._lookup.cache_clear()
+    try:
+        assert ls.findspec(3, 11, 13, 2, 32, 2) == (4, 128)
+        assert ls.launch_options_for(3, 11, 13, 2, 32, 2, "fwd") == {"gather": "direct"}
+        assert ls.launch_options_for(3, 11, 13, 2, 32, 2, "bwd") == {}                  # no entry: the library chooses
+        assert ls.find_spec_bwd(3, 11, 13, 2, 32, 2) == ls._spec(2, 32, 2, scatter=True)
+        hits = ls._lookup.cache_info().hits
+        ls.findspec(3, 11, 13, 2, 32, 2)
+        assert ls._lookup.cache_info().hits == hits + 1
+    finally:
+        ls._lookup.cache_clear()
+
+
+def test_launch_options_are_validated_without_a_gpu():
+    from dcnv4_amd import _lib
+    lib = _lib.load()
+    assert lib.dcnv4_gfx950_set_launch_option(b"gather", 2) == 0 and lib.dcnv4_gfx950_set_launch_option(b"gather", 0) == 0
+    assert lib.dcnv4_gfx950_set_launch_option(b"reach", 7) == 0 and lib.dcnv4_gfx950_set_launch_option(b"reach", -1) == 0
+    assert lib.dcnv4_gfx950_set_launch_option(b"gather", 5) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.dcnv4_gfx950_set_launch_option(b"nonsense", 1) == _lib.ERR_INVALID_ARGUMENT
+    assert b"nonsense" in lib.dcnv4_gfx950_last_error()
+    # the scatter option decides the workspace: global atomics need an fp32 image for 16-bit tensors
+    tiled = lib.dcnv4_gfx950_backward_workspace_bytes(1, 2, 8, 8, 2, 16)
+    lib.dcnv4_gfx950_set_launch_option(b"scatter", 2)
+    try:
+        assert lib.dcnv4_gfx950_backward_workspace_bytes(1, 2, 8, 8, 2, 16) == 2 * 8 * 8 * 32 * 4 and tiled == 256
+    finally:
+        lib.dcnv4_gfx950_set_launch_option(b"scatter", 0)
