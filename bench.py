@@ -148,6 +148,18 @@ def main():
         go = torch.randn(B, N, G * D, device=dev).to(dtype)
         return (B, N, G, D, L, K), shapes, starts, v, sla, go
 
+    if args.only_op and args.only_op.startswith("model:"):
+        # FlashInternImage forward only (for profiling): model:<t|s|b|l>:<dtype>, batch 128, --warmup / --steps passes
+        from dcnv4_amd.models import flash_intern_image
+        _, variant, dt_name = args.only_op.split(":")
+        dtype = getattr(torch, dt_name)
+        model = flash_intern_image(variant).to(dev).to(dtype).eval()
+        images = torch.randn(128, 3, 224, 224, device=dev).to(dtype)
+        with torch.no_grad():
+            ms = time_op(lambda: model(images), args.steps, warm=args.warmup)
+        print(json.dumps({"only_op": args.only_op, "ms": round(ms, 4), "img_per_s": round(128 / (ms * 1e-3), 1)}))
+        return
+
     if args.only_op:
         op, shape_name, dt_name = args.only_op.split(":")
         dtype = getattr(torch, dt_name)

@@ -36,7 +36,8 @@ __global__ void __launch_bounds__(kDwThreads) dwconv_forward_kernel(const DwLaun
   constexpr int kVecBytes = V * Tag::kBytes;
   const int kh = KH > 0 ? KH : p.kh, kw = KH > 0 ? KW : p.kw;
   const int nvec = p.C / V;
-  uint32_t t = blockIdx.x * kDwThreads + threadIdx.x;
+  // consecutive workgroups share input rows: keep them on one XCD (one L2)
+  uint32_t t = xcd_contiguous_block(blockIdx.x, gridDim.x) * kDwThreads + threadIdx.x;
   const int cvec = t % nvec; t /= nvec;
   const int xs = t % p.n_seg; t /= p.n_seg;
   const int y = t % p.Ho;
