@@ -30,6 +30,7 @@ SIGNATURES = {
     "dcnv4_gfx950_depthwise_conv_forward": (_i, [_vp] * 4 + [_i] * 7 + [_vp]),
     "dcnv4_gfx950_depthwise_conv_backward_workspace_bytes": (_sz, [_i] * 7),
     "dcnv4_gfx950_depthwise_conv_backward": (_i, [_vp] * 7 + [_sz] + [_i] * 7 + [_vp]),
+    "dcnv4_gfx950_layer_norm_residual_forward": (_i, [_vp] * 6 + [_i, ctypes.c_longlong, _i, _f, _vp]),
 }
 
 _lib = None

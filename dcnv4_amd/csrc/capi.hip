@@ -827,4 +827,29 @@ int dcnv4_gfx950_depthwise_conv_backward(const void *input, const void *weight, 
   return DCNV4_OK;
 }
 
+int dcnv4_gfx950_layer_norm_residual_forward(const void *input, const void *residual, const void *weight,
+                                             const void *bias, const void *gamma, void *output, int dtype,
+                                             long long rows, int channels, float eps, void *stream) {
+  const int s = elem_bytes(dtype);
+  if (s == 0) return fail(DCNV4_ERR_RUNTIME, "unsupported dtype code %d (fp32, fp16, bf16 only)", dtype);
+  if (rows <= 0 || channels <= 0) return fail(DCNV4_ERR_RUNTIME, "empty or negative extent (rows %lld, channels %d)", rows, channels);
+  const int V = 16 / s;
+  if (channels % V != 0) return fail(DCNV4_ERR_INVALID_ARGUMENT, "channels (%d) must be a multiple of %d for this dtype", channels, V);
+  const int nvec = channels / V;
+  if (nvec > 64 * 8) return fail(DCNV4_ERR_INVALID_ARGUMENT, "rows of %d channels are too long (at most %d)", channels, 64 * 8 * V);
+  if (int rc = check_ptrs({input, weight, bias, output})) return rc;
+  if ((residual != nullptr && !aligned16(residual)) || (gamma != nullptr && !aligned16(gamma)))
+    return fail(DCNV4_ERR_RUNTIME, "tensor pointer is not 16-byte aligned");
+  LnLaunch L{};
+  L.y = input; L.residual = residual; L.weight = weight; L.bias = bias; L.gamma = gamma; L.out = output;
+  L.rows = rows; L.C = channels; L.eps = eps;
+  L.team = 1;
+  while (L.team < 64 && L.team < nvec) L.team *= 2;
+  L.vpl = 1;
+  while (L.team * L.vpl < nvec) L.vpl *= 2;
+  if (hipError_t e = launch_layer_norm_residual(dtype, L, static_cast<hipStream_t>(stream)))
+    return hip_fail("layer norm launch", e);
+  return DCNV4_OK;
+}
+
 }  // extern "C"

@@ -138,6 +138,18 @@ struct DwLaunch {
   int slab, n_part;        // grad_weight: row segments (seg columns each) per workgroup, workgroups
 };
 
+// out = residual + gamma * LayerNorm(y) over rows of C channels (residual and gamma may be null).
+struct LnLaunch {
+  const void *y, *residual, *weight, *bias, *gamma;
+  void *out;
+  long long rows;
+  int C;
+  float eps;
+  int team;      // lanes per row: a power of two, <= 64
+  int vpl;       // 16-byte vectors per lane: 1, 2, 4 or 8 (team * vpl * 16 bytes cover a row)
+};
+hipError_t launch_layer_norm_residual(int dtype, const LnLaunch &p, hipStream_t stream);
+
 // Each returns hipSuccess or the launch error.  dtype: 0 fp32, 1 fp16, 2 bf16.
 hipError_t launch_depthwise_forward(int dtype, const DwLaunch &p, hipStream_t stream);
 // channels per lane of the grad_weight kernel, and lanes of a workgroup that share a channel vector

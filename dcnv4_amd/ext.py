@@ -226,3 +226,29 @@ def depthwise_conv_backward(input, weight, grad_output, pad, has_bias=True, need
             input.data_ptr(), weight.data_ptr(), grad_output.data_ptr(), ptr(grad_input), ptr(grad_weight),
             ptr(grad_bias), ptr(ws), ws_bytes, code, batch, h, w, channels, k, int(pad), _stream()))
     return [grad_input, grad_weight, grad_bias]
+
+
+def layer_norm_residual_forward(input, residual, weight, bias, gamma, eps):
+    """``residual + gamma * layer_norm(input)`` over the last axis in one kernel; ``residual`` and ``gamma`` may be
+    None.  All tensors share one dtype; the channel count must be a whole number of 16-byte vectors."""
+    _check(input, "input")
+    _check(weight, "weight", input.dtype)
+    _check(bias, "bias", input.dtype)
+    if residual is not None:
+        _check(residual, "residual", input.dtype)
+        if residual.shape != input.shape:
+            raise RuntimeError("residual must have the shape of the input")
+    if gamma is not None:
+        _check(gamma, "gamma", input.dtype)
+    code = _dtype_code(input, "input")
+    channels = input.shape[-1]
+    if weight.numel() != channels or bias.numel() != channels or (gamma is not None and gamma.numel() != channels):
+        raise RuntimeError(f"weight, bias and gamma must have {channels} elements")
+    with torch.cuda.device(input.device):
+        output = torch.empty_like(input)
+        if input.numel():
+            _lib.check(_L.dcnv4_gfx950_layer_norm_residual_forward(
+                input.data_ptr(), residual.data_ptr() if residual is not None else None, weight.data_ptr(), bias.data_ptr(),
+                gamma.data_ptr() if gamma is not None else None, output.data_ptr(), code, input.numel() // channels,
+                channels, float(eps), _stream()))
+    return output

@@ -11,6 +11,7 @@ FlashInternImage config enables.
 import torch
 from torch import nn
 
+from ..functions import layer_norm_residual
 from ..modules import DCNv4
 
 
@@ -69,7 +70,10 @@ class StemLayer(nn.Module):
         self.norm2 = _norm(out_chans, norm_layer, "channels_first", "channels_last")
 
     def forward(self, x):
-        return self.norm2(self.conv2(self.act(self.norm1(self.conv1(x)))))
+        # channels-last memory from the first convolution on: the NHWC view the blocks work on is then dense, so
+        # every kernel after the stem sees contiguous rows of channels (no strided elementwise kernels, no copies)
+        x = x.contiguous(memory_format=torch.channels_last)
+        return self.norm2(self.conv2(self.act(self.norm1(self.conv1(x))))).contiguous()
 
 
 class DownsampleLayer(nn.Module):
@@ -114,14 +118,25 @@ class InternImageLayer(nn.Module):
             self.gamma1 = nn.Parameter(layer_scale * torch.ones(channels))
             self.gamma2 = nn.Parameter(layer_scale * torch.ones(channels))
 
+    def _scaled_norm(self, norm, gamma, y, residual):
+        """residual + drop_path(gamma * norm(y)); one kernel when stochastic depth is idle (always in eval mode)."""
+        ln = norm[0] if len(norm) == 1 and isinstance(norm[0], nn.LayerNorm) else None
+        if ln is None:
+            return residual + self.drop_path((gamma * norm(y)) if gamma is not None else norm(y))
+        if isinstance(self.drop_path, nn.Identity) or not self.training:
+            return layer_norm_residual(y, ln, gamma, residual)
+        return residual + self.drop_path(layer_norm_residual(y, ln, gamma))
+
     def forward(self, x, shape):
-        g1, g2 = (self.gamma1, self.gamma2) if self.layer_scale else (1.0, 1.0)
+        g1, g2 = (self.gamma1, self.gamma2) if self.layer_scale else (None, None)
         if self.post_norm:
-            x = x + self.drop_path(g1 * self.norm1(self.dcn(x, shape)))
-            x = x + self.drop_path(g2 * self.norm2(self.mlp(x, shape)))
+            x = self._scaled_norm(self.norm1, g1, self.dcn(x, shape), x)
+            x = self._scaled_norm(self.norm2, g2, self.mlp(x, shape), x)
         else:
-            x = x + self.drop_path(g1 * self.dcn(self.norm1(x), shape))
-            x = x + self.drop_path(g2 * self.mlp(self.norm2(x), shape))
+            y = self.dcn(layer_norm_residual(x, self.norm1[0]), shape)
+            x = x + self.drop_path(y if g1 is None else g1 * y)
+            y = self.mlp(layer_norm_residual(x, self.norm2[0]), shape)
+            x = x + self.drop_path(y if g2 is None else g2 * y)
         return x
 
 

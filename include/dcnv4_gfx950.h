@@ -189,6 +189,19 @@ int dcnv4_gfx950_depthwise_conv_backward(const void *input, const void *weight,
                                          int width, int channels, int kernel_size, int pad,
                                          void *stream);
 
+/*
+ * output = residual + gamma * LayerNorm(input) over rows of `channels` elements (biased variance, affine
+ * weight and bias, fp32 arithmetic, one rounding): the tail of a FlashInternImage block,
+ * `x + drop_path(gamma1 * norm1(dcn(x)))` (classification/models/flash_intern_image.py:425-440), which the
+ * framework runs as three kernels.  `residual` and `gamma` may be NULL (plain layer normalisation when both
+ * are).  channels must be a multiple of 16 bytes' worth of elements and at most 512 such vectors.
+ *   input, residual, output  [rows, channels];  weight, bias, gamma  [channels]
+ */
+int dcnv4_gfx950_layer_norm_residual_forward(const void *input, const void *residual, const void *weight,
+                                             const void *bias, const void *gamma, void *output,
+                                             int dtype, long long rows, int channels, float eps,
+                                             void *stream);
+
 #ifdef __cplusplus
 }
 #endif

