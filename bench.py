@@ -153,6 +153,7 @@ def main():
         from dcnv4_amd.models import flash_intern_image
         _, variant, dt_name = args.only_op.split(":")
         dtype = getattr(torch, dt_name)
+        torch.backends.cudnn.benchmark = True         # as the reference's entry point does (classification/main.py:635)
         model = flash_intern_image(variant).to(dev).to(dtype).eval()
         images = torch.randn(128, 3, 224, 224, device=dev).to(dtype)
         with torch.no_grad():
@@ -267,6 +268,7 @@ def main():
     model_line = None
     if not args.no_model:
         from dcnv4_amd.models import flash_intern_image
+        torch.backends.cudnn.benchmark = True         # as the reference's entry point does (classification/main.py:635)
         model = flash_intern_image("b").to(dev).half().eval()
         images = torch.randn(128, 3, 224, 224, device=dev).half()
         spans = []                                    # (start, end) events around every DCNv4 operator call
