@@ -248,6 +248,24 @@ __device__ __forceinline__ unsigned long long fixed_product(double a, double b) 
   return __builtin_bit_cast(unsigned long long, d) - 0x4338000000000000ull;
 }
 
+// round-to-nearest-even(a * b) for |a * b| < 2^22, two instructions: the product is formed inside an
+// fma whose addend pushes the integer part into the low mantissa bits.
+__device__ __forceinline__ int to_fixed32(float a, float b) {
+  return (int)(__builtin_bit_cast(uint32_t, fmaf(a, b, 12582912.f)) - 0x4B400000u);
+}
+
+// Two signed 32-bit fixed-point terms in one 64-bit addend: the sum of such words is hi * 2^32 + lo with both
+// halves signed, so the low term is sign-extended into the high word before the add.
+__device__ __forceinline__ unsigned long long pack_fixed32(int lo, int hi) {
+  return ((unsigned long long)(uint32_t)(hi + (lo >> 31)) << 32) | (uint32_t)lo;
+}
+
+// the two fields of a sum of pack_fixed32 words
+__device__ __forceinline__ int packed_field(unsigned long long a, int high) {
+  const int lo = (int)(uint32_t)a;
+  return high ? (int)(uint32_t)(a >> 32) + (lo < 0 ? 1 : 0) : lo;
+}
+
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
   for (int o = 32; o > 0; o >>= 1) v = max(v, (uint32_t)__shfl_xor((int)v, o, kWave));
   return v;

@@ -42,12 +42,6 @@ constexpr int kTrashPad = 64;
 constexpr int kMaxChunkGroups = 4;      // rows of a wave <-> groups of the chunk
 constexpr int kCellBits = 9;            // cell index 0..n_cells (n_cells = trash), tiles up to 16x16
 
-// round-to-nearest-even(a * b) for |a * b| < 2^22, two instructions: the product is formed inside an
-// fma whose addend pushes the integer part into the low mantissa bits.
-__device__ __forceinline__ int to_fixed32(float a, float b) {
-  return (int)(__builtin_bit_cast(uint32_t, fmaf(a, b, 12582912.f)) - 0x4B400000u);
-}
-
 struct HitMeta {
   uint32_t cells012;    // accumulator cell of corners 0,1,2 (9 bits each); n_cells = "nowhere" (weight 0)
   uint32_t cell3_px;    // cell of corner 3 | strip-local pixel << 9
@@ -326,9 +320,8 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
             const float g_hi = (c * CPL + ch + 1 < D) ? go_px[ch + 1] : 0.f;
 #pragma unroll
             for (int cn = 0; cn < 4; ++cn) {
-              const int lo = to_fixed32(g_lo, wv[cn]), hi = to_fixed32(g_hi, wv[cn]);
-              const unsigned long long v = ((unsigned long long)(uint32_t)(hi + (lo >> 31)) << 32) | (uint32_t)lo;
-              __hip_atomic_fetch_add(dst[cn] + unit_of[u], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+              __hip_atomic_fetch_add(dst[cn] + unit_of[u], pack_fixed32(to_fixed32(g_lo, wv[cn]), to_fixed32(g_hi, wv[cn])),
+                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
           }
         } else {
@@ -361,10 +354,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       float f[1];
       if constexpr (PACK) {
         const int g = ch / D, cg = ch - g * D;
-        const unsigned long long a = src[g * group_words + (cg >> 1)];
-        const int lo = (int)(uint32_t)a;
-        const int field = (cg & 1) ? (int)(uint32_t)(a >> 32) + (lo < 0 ? 1 : 0) : lo;
-        f[0] = ldexpf((float)field, e_out);
+        f[0] = ldexpf((float)packed_field(src[g * group_words + (cg >> 1)], cg & 1), e_out);
       } else {
         const unsigned long long a = src[ch];
         f[0] = (float)ldexp((double)(int)(a >> 32) * 4294967296.0 + (double)(uint32_t)a, e_out);
