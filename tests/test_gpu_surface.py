@@ -317,12 +317,37 @@ def test_small_flash_intern_image_matches_the_same_network_on_the_torch_core(mon
     with torch.no_grad():
         got = model.cuda()(x.cuda()).cpu()
         feats = [f.cpu() for f in model.forward_features_seq_out(x.cuda())]
-        model.cpu()
-        monkeypatch.setattr(dcnv4_module, "DCNv4Function", CoreOnCpu)
-        monkeypatch.setattr(dcnv4_module, "DepthwiseConvNHWCFunction", DepthwiseOnCpu)
+    # one training-style backward on the GPU (every autograd Function of the library in place) ...
+    import copy
+    state = copy.deepcopy(model.state_dict())           # the training pass moves the batch-norm statistics
+    model.train()
+    weights = torch.randn(2, 10)
+    (model(x.cuda()) * weights.cuda()).sum().backward()
+    gpu_grads = {k: p.grad.detach().cpu().clone() for k, p in model.named_parameters() if p.grad is not None}
+    model.zero_grad()
+    model.load_state_dict(state)
+    model.cpu().eval()
+    # ... against the same network on the CPU with the operators swapped for torch formulations
+    monkeypatch.setattr(dcnv4_module, "DCNv4Function", CoreOnCpu)
+    monkeypatch.setattr(dcnv4_module, "DepthwiseConvNHWCFunction", DepthwiseOnCpu)
+    with torch.no_grad():
         want = model(x)
+    model.train()
+    (model(x) * weights).sum().backward()
     assert got.shape == (2, 10) and [tuple(f.shape) for f in feats] == [(2, 32, 16, 16), (2, 64, 8, 8)]
     assert _rel_err(got, want) < 1e-3
+    checked = 0
+    scale = max(float(p.grad.abs().max()) for p in model.parameters() if p.grad is not None)
+    for k, p in model.named_parameters():
+        if p.grad is None:
+            continue
+        assert k in gpu_grads, k
+        if float(p.grad.abs().max()) < 1e-5 * scale:         # e.g. a bias in front of a batch norm: zero up to rounding
+            assert float(gpu_grads[k].abs().max()) < 1e-4 * scale, k
+            continue
+        assert _rel_err(gpu_grads[k], p.grad) < 5e-3, k
+        checked += 1
+    assert checked > 60
 
 
 def test_dense_prediction_backbone_returns_per_level_maps_for_a_non_square_input(monkeypatch):
@@ -441,3 +466,54 @@ def test_fused_block_tail_has_autograd_gradients_and_falls_back_under_autocast()
     with torch.autocast(device_type="cuda", dtype=torch.float16):
         mixed = layer_norm_residual(y, norm, gamma, x)                # torch's operators: autocast semantics kept
     assert "LayerNormResidualFunction" not in type(mixed.grad_fn).__name__
+
+
+def test_depthwise_and_block_tail_replay_correctly_from_a_hip_graph():
+    from dcnv4_amd import ext
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(4, 20, 18, 64, generator=g).half().cuda()
+    w = (torch.randn(64, 1, 3, 3, generator=g) / 3).half().cuda()
+    b = torch.randn(64, generator=g).half().cuda()
+    go = torch.randn(4, 20, 18, 64, generator=g).half().cuda()
+    gamma = torch.randn(64, generator=g).half().cuda()
+
+    def run():
+        y = ext.depthwise_conv_forward(x, w, b, 1)
+        gi, gw, gb = ext.depthwise_conv_backward(x, w, go, 1)
+        return y, gi, gw, gb, ext.layer_norm_residual_forward(y, x, w.flatten()[:64].contiguous(), b, gamma, 1e-6)
+
+    eager = run()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = run()
+    for _ in range(3):
+        for t in captured:
+            t.fill_(7.0)
+        (x.float().sum() + 1).item()                                     # unrelated eager work + sync between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, e) for a, e in zip(captured, eager))
+
+
+def test_depthwise_adjoint_identities_at_a_benchmark_shape():
+    """<go, conv(x)> = <grad_x, x> = <grad_w, w> + <grad_b, b> ... at 32x56x56x112 in fp32 (linear in x and in (w, b))."""
+    from dcnv4_amd import ext
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(32, 56, 56, 112, generator=g).cuda()
+    w = (torch.randn(112, 1, 3, 3, generator=g) / 3).cuda()
+    b = torch.randn(112, generator=g).cuda()
+    go = torch.randn(32, 56, 56, 112, generator=g).cuda()
+    y = ext.depthwise_conv_forward(x, w, b, 1)
+    y0 = ext.depthwise_conv_forward(x, w, None, 1)
+    gi, gw, gb = ext.depthwise_conv_backward(x, w, go, 1)
+    dot = lambda a, c: (a.double() * c.double()).sum().item()
+    lhs = dot(go, y0)
+    assert abs(dot(gi, x) - lhs) < 1e-5 * abs(lhs) + 1e-2
+    assert abs(dot(gw, w) - lhs) < 1e-4 * abs(lhs) + 1e-1
+    assert abs(dot(go, y) - lhs - dot(gb, b)) < 1e-4 * abs(lhs) + 1e-1
