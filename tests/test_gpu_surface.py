@@ -517,3 +517,27 @@ def test_depthwise_adjoint_identities_at_a_benchmark_shape():
     assert abs(dot(gi, x) - lhs) < 1e-5 * abs(lhs) + 1e-2
     assert abs(dot(gw, w) - lhs) < 1e-4 * abs(lhs) + 1e-1
     assert abs(dot(go, y) - lhs - dot(gb, b)) < 1e-4 * abs(lhs) + 1e-1
+
+
+def test_depthwise_batches_beyond_the_32_bit_addressing_span_are_chunked_consistently():
+    # 2.7 GB of input: more than one launch addresses with 32-bit buffer offsets; images are independent, so any
+    # slice of the batch must give the same bits, and grad_weight must equal the sum over slices
+    torch.manual_seed(6)
+    B, H, W, C = 20, 512, 512, 128
+    x = torch.randn(B, H, W, C, device="cuda")
+    w = torch.randn(C, 3, 3, device="cuda") / 3
+    b = torch.randn(C, device="cuda")
+    out = cabi.depthwise_forward(x, w, b, 1)
+    for lo, hi in [(0, 2), (7, 9), (18, 20)]:
+        assert torch.equal(out[lo:hi], cabi.depthwise_forward(x[lo:hi].contiguous(), w, b, 1))
+    go = out                                   # any values do as the incoming gradient
+    gi, gw, gb = cabi.depthwise_backward(x, w, go, 1)
+    pi, _, _ = cabi.depthwise_backward(x[7:9].contiguous(), w, go[7:9].contiguous(), 1)
+    assert torch.equal(gi[7:9], pi)
+    gw_sum = torch.zeros_like(gw, dtype=torch.float64)
+    gb_sum = torch.zeros_like(gb, dtype=torch.float64)
+    for lo in range(0, B, 5):
+        _, pw, pb = cabi.depthwise_backward(x[lo:lo + 5].contiguous(), w, go[lo:lo + 5].contiguous(), 1)
+        gw_sum += pw.double()
+        gb_sum += pb.double()
+    assert _rel_err(gw.double(), gw_sum) < 1e-5 and _rel_err(gb.double(), gb_sum) < 1e-5
