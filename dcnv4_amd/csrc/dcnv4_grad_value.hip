@@ -284,7 +284,17 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       // touch different words in every instruction.
       constexpr int kUnits = PACK ? CPL / 2 : CPL;                       // accumulator words per lane
       const int rows_per_group = (kWave / R) / p.ng_chunk;
-      const int my_group = row_in_wave / rows_per_group, my_slot = row_in_wave - my_group * rows_per_group;
+      int my_group = row_in_wave / rows_per_group, my_slot = row_in_wave - my_group * rows_per_group;
+      int first_unit = my_slot;
+      if (PACK && R == 2 && p.ng_chunk == 4 && group_words == 8) {
+        // A cell of packed sums is 32 words, one bank sweep, and the LDS takes a wave's 64-bit atomics half a wave
+        // at a time: deal the 16 rows of each half-wave as 4 groups x 4 starting units, so that a half-wave touches
+        // 32 distinct words (groups in consecutive rows would put two rows of a half-wave on every word).
+        const int half = row_in_wave >> 4, i = row_in_wave & 15;
+        my_group = i >> 2;
+        first_unit = i & 3;
+        my_slot = half * 4 + first_unit;
+      }
       const bool group_live = my_group < ng;
       const uint32_t n_mine = group_live ? count[my_group] : 0u;
       uint32_t n_max = count[0];
@@ -294,7 +304,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       const float *go_lane = s_go + lane_group * D + c * CPL;
       int unit_of[kUnits];                                               // this row's visiting order
 #pragma unroll
-      for (int u = 0; u < kUnits; ++u) unit_of[u] = (u + my_slot) & (kUnits - 1);
+      for (int u = 0; u < kUnits; ++u) unit_of[u] = (u + first_unit) & (kUnits - 1);
       for (uint32_t i0 = wave * rows_per_group; i0 < n_max; i0 += kWaves * rows_per_group) {
         const uint32_t i = i0 + my_slot;
         f32x4 w = {0.f, 0.f, 0.f, 0.f};
