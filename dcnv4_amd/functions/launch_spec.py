@@ -35,6 +35,7 @@ GFX950_TABLE = _load_table()
 
 
 def table_key(B, H, W, G, C, elem_bytes, direction):
+    """``C`` is the number of channels per group, as in the reference's table keys ("64x56x56x4x16")."""
     return f"{B}x{H}x{W}x{G}x{C}:{elem_bytes}:{direction}"
 
 

@@ -56,6 +56,7 @@ def candidates(G, D, elem_bytes, direction):
 def tune(shape_sets, dtypes, iters=50, warm=10, margin=0.03, min_gain_us=10.0, offset_range=3.0, log=print):
     import torch
     from . import ext
+    from .functions import launch_spec
     dev = torch.device("cuda:0")
     entries, report = {}, []
     for set_name in shape_sets:
@@ -83,12 +84,11 @@ def tune(shape_sets, dtypes, iters=50, warm=10, margin=0.03, min_gain_us=10.0, o
                         timings.append((ms, label, options, d_stride, n_thread))
                     base = timings[0][0]
                     best = min(timings)
-                    key = f"{B}x{H}x{W}x{G}x{C}:{es}:{direction}"
+                    key = launch_spec.table_key(B, H, W, G, D, es, direction)      # C of the key = channels per group
                     report.append({"key": key, "library_ms": round(base, 5), "best_ms": round(best[0], 5), "best": best[1]})
                     log(f"{key:28s} library {base * 1e3:8.1f} us   best {best[0] * 1e3:8.1f} us  ({best[1]})")
                     if best[0] < base * (1.0 - margin) and (base - best[0]) * 1e3 > min_gain_us:
-                        from .functions.launch_spec import _spec
-                        d, n = (best[3], best[4]) if best[3] else _spec(G, D, es, scatter=direction == "bwd")
+                        d, n = (best[3], best[4]) if best[3] else launch_spec._spec(G, D, es, scatter=direction == "bwd")
                         entries[key] = dict(d_stride=d, n_thread=n, **best[2])
                 del value, om, go
     return entries, report

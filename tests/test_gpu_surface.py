@@ -541,3 +541,35 @@ def test_depthwise_batches_beyond_the_32_bit_addressing_span_are_chunked_consist
         gw_sum += pw.double()
         gb_sum += pb.double()
     assert _rel_err(gw.double(), gw_sum) < 1e-5 and _rel_err(gb.double(), gb_sum) < 1e-5
+
+
+def test_autograd_function_applies_a_tuned_table_entry(monkeypatch):
+    """DCNv4Function looks shapes up as (B, H, W, group, channels per group), the reference's key convention; an
+    entry with a kernel family must reach the library as a launch option around the call, and only around it."""
+    import dcnv4_amd
+    from dcnv4_amd import _lib, ext
+    from dcnv4_amd.functions import launch_spec as ls
+    B, H, W, G, D = 2, 12, 10, 2, 16
+    v, om, go = (t.cuda() for t in make_dcnv4_inputs(B, H, W, G, D, seed=14, dtype=torch.float16))
+    want = dcnv4_amd.DCNv4Function.apply(v, om, *GEOM, G, D, 1.0, 256, 0)
+    monkeypatch.setitem(ls.GFX950_TABLE, ls.table_key(B, H, W, G, D, 2, "fwd"), {"d_stride": 8, "n_thread": 128, "gather": "direct"})
+    monkeypatch.setitem(ls.GFX950_TABLE, ls.table_key(B, H, W, G, D, 2, "bwd"), {"d_stride": 1, "n_thread": 64, "scatter": "atomic"})
+    ls._lookup.cache_clear()
+    seen = []
+    real = _lib.load().dcnv4_gfx950_set_launch_option
+
+    class Spy:
+        def __call__(self, name, value):
+            seen.append((name, value))
+            return real(name, value)
+
+    monkeypatch.setattr(ext._L, "dcnv4_gfx950_set_launch_option", Spy(), raising=False)
+    try:
+        vg, omg = v.clone().requires_grad_(True), om.clone().requires_grad_(True)
+        out = dcnv4_amd.DCNv4Function.apply(vg, omg, *GEOM, G, D, 1.0, 256, 0)
+        out.backward(go)
+    finally:
+        ls._lookup.cache_clear()
+    assert (b"gather", 2) in seen and (b"scatter", 2) in seen
+    assert seen[-3:] == [(b"gather", 0), (b"scatter", 0), (b"reach", -1)]          # back at the library's choice
+    assert _rel_err(out.float().cpu(), want.float().cpu()) < 2e-3 and vg.grad is not None and omg.grad is not None
