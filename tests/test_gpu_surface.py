@@ -573,3 +573,19 @@ def test_autograd_function_applies_a_tuned_table_entry(monkeypatch):
     assert (b"gather", 2) in seen and (b"scatter", 2) in seen
     assert seen[-3:] == [(b"gather", 0), (b"scatter", 0), (b"reach", -1)]          # back at the library's choice
     assert _rel_err(out.float().cpu(), want.float().cpu()) < 2e-3 and vg.grad is not None and omg.grad is not None
+
+
+def test_block_tail_at_the_model_stage_one_size_normalises_every_row():
+    """128 x 56 x 56 rows of 112 channels (FlashInternImage-B stage 1) in fp16: with unit weight and zero bias every
+    output row has zero mean and unit (biased) variance; with residual and gamma the result is that plus the residual."""
+    from dcnv4_amd import ext
+    torch.manual_seed(15)
+    y = (torch.randn(128 * 56 * 56, 112, device="cuda") * 3 + 1).half()
+    ones, zeros = torch.ones(112, device="cuda").half(), torch.zeros(112, device="cuda").half()
+    out = ext.layer_norm_residual_forward(y, None, ones, zeros, None, 1e-6).float()
+    assert out.mean(-1).abs().max().item() < 2e-3
+    assert (out.pow(2).mean(-1) - 1).abs().max().item() < 5e-3
+    res = torch.randn_like(y)
+    gamma = torch.full((112,), 0.5, device="cuda").half()
+    both = ext.layer_norm_residual_forward(y, res, ones, zeros, gamma, 1e-6).float()
+    assert (both - (res.float() + 0.5 * out)).abs().max().item() < 4e-3

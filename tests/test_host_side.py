@@ -217,3 +217,15 @@ def test_launch_options_are_validated_without_a_gpu():
         assert lib.dcnv4_gfx950_backward_workspace_bytes(1, 2, 8, 8, 2, 16) == 2 * 8 * 8 * 32 * 4 and tiled == 256
     finally:
         lib.dcnv4_gfx950_set_launch_option(b"scatter", 0)
+
+
+def test_tuner_candidates_are_valid_hints_and_start_with_the_library_choice():
+    from dcnv4_amd import tune
+    for G, D, es in [(4, 16, 2), (4, 16, 4), (8, 32, 2), (5, 24, 4)]:
+        fwd = tune.candidates(G, D, es, "fwd")
+        assert fwd[0] == ("library", {}, 0, 0)
+        for _, options, d_stride, n_thread in fwd[1:]:
+            assert options == {"gather": "direct"} and D % d_stride == 0 and d_stride * es <= 16 and n_thread in (128, 256, 512)
+        bwd = tune.candidates(G, D, es, "bwd")
+        assert bwd[0] == ("library", {}, 0, 0) and {"scatter": "atomic"} in [c[1] for c in bwd]
+    assert set(tune.SHAPES) == {"t", "b", "dense"} and all(len(v) == 4 for v in tune.SHAPES.values())
