@@ -145,6 +145,15 @@ bool fda_tiled_shape(int D, int L, int Q, int K) {
   return D % 8 == 0 && D <= 32 && L >= 1 && K >= 1 && (long long)Q * K < (1ll << 31);
 }
 
+constexpr size_t kL2BytesPerXcd = 4u << 20;
+
+// Tuning override, read on every call: DCNV4_GFX950_FDA_ORDER=rows keeps the attention forward on whole rows
+// (all heads of a query in one workgroup) whatever the sizes.
+bool fda_head_major_enabled() {
+  const char *e = getenv("DCNV4_GFX950_FDA_ORDER");
+  return !(e && strcmp(e, "rows") == 0);
+}
+
 // Tuning override, read on every call: DCNV4_GFX950_FDA_SCATTER=atomic keeps the fp32 atomic scatter.
 bool fda_tiled_enabled() {
   if (g_opt_scatter != kOptAuto) return g_opt_scatter == kOptTiled;
@@ -364,6 +373,21 @@ int fda_prepare(FdaProblem *pr, bool backward, bool scatter, int dtype, int batc
   if ((uint64_t)pr->img_elems * (backward ? 4 : s) > kMaxSpanBytes)
     return fail(DCNV4_ERR_RUNTIME, "one value image of %zu elements exceeds the 2 GiB addressing span of a launch", pr->img_elems);
   return DCNV4_OK;
+}
+
+// One head per workgroup, workgroups ordered [image][head][block of queries], when a head's slice of a value image
+// fits an XCD's L2 and the whole image does not: the gathers then hit L2.  A workgroup takes as many queries as fill
+// it with one head's lanes (and fit the LDS).
+void fda_choose_order(FdaLaunch *F, const FdaProblem &pr, int N, int G, int D, int L, int K, bool backward) {
+  const size_t line = 128, head_bytes = (size_t)D * pr.s;
+  const size_t lines_per_pixel = (std::max(head_bytes, line) + line - 1) / line;      // cache lines a head touches per pixel
+  const size_t head_footprint = (size_t)N * lines_per_pixel * line;
+  F->head_major = 0;
+  if (!fda_head_major_enabled() || G <= 1 || pr.img_elems * pr.s <= kL2BytesPerXcd / 2 || head_footprint > kL2BytesPerXcd) return;
+  F->head_major = 1;
+  const int width = 1 << F->lanes.tpgp_log2;
+  const size_t lds_per_row = (size_t)3 * L * K * sizeof(float) * (backward ? 2 : 1);
+  F->nq_block = std::max(1, std::min(kBlockThreads / width, (int)(kMaxDynamicLds / lds_per_row)));
 }
 
 int images_per_launch(const FdaProblem &pr, bool backward) {
@@ -607,6 +631,7 @@ int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_s
     F.level_start = level_start_index;
     F.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
     F.n_row = nb * F.Q;
+    fda_choose_order(&F, pr, spatial_size, num_heads, head_channels, num_levels, num_points, false);
     if (hipError_t e = launch_fda_forward(dtype, F, static_cast<hipStream_t>(stream)))
       return hip_fail("flash_deform_attn forward launch", e);
   }
@@ -715,6 +740,7 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
         F.n_row = nb * F.Q;
         F.n_img = nb;
         hipError_t e = hipSuccess;
+        if (pass == 0) fda_choose_order(&F, pr, spatial_size, num_heads, head_channels, num_levels, num_points, true);
         if (pass == 0) e = launch_fda_backward(dtype, F, kFdaNoScatter, st);
         else if (pass == 1) e = launch_fda_grad_value(dtype, F, st);
         else e = launch_fda_backward(dtype, F, kFdaFallback, st);

@@ -34,16 +34,39 @@ __global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLau
   typedef Pack<Tag, CPT> pack;
   const int LK = p.L * p.K, row_len = 3 * LK;
   const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
-  const int row0 = (int)blk * p.nq_block;
-  const int nrow = min(p.nq_block, p.n_row - row0);
-  const int span = nrow * p.G * row_len;
-  const bool vec16 = ((size_t)p.G * row_len * Tag::kBytes) % 16 == 0;
-  stage_rows_to_lds<Tag>(lds, (const char *)p.sla + (size_t)row0 * p.G * row_len * Tag::kBytes, span, vec16);
+  int row0, nrow, heads_here = p.G, g_fixed = 0;
+  if (p.head_major) {
+    // Workgroups ordered [image][head][block of queries], each for ONE head: an XCD then works through one head of one
+    // image at a time, whose slice of `value` (N x D elements, one or two heads per cache line) fits its L2, where the
+    // whole image does not.
+    const int blocks_per_image = (p.Q + p.nq_block - 1) / p.nq_block;
+    const int rb = (int)(blk % (uint32_t)blocks_per_image), bg = (int)(blk / (uint32_t)blocks_per_image);
+    const int b = bg / p.G;
+    g_fixed = bg - b * p.G;
+    heads_here = 1;
+    const int q0 = rb * p.nq_block;
+    nrow = min(p.nq_block, p.Q - q0);
+    row0 = b * p.Q + q0;
+    typedef typename RawWord<Tag::kBytes>::type elem_t;
+    const elem_t *src = reinterpret_cast<const elem_t *>(p.sla) + ((size_t)row0 * p.G + g_fixed) * row_len;
+    for (int i = threadIdx.x; i < nrow * row_len; i += blockDim.x) {
+      const int r = i / row_len, e = i - r * row_len;
+      float f[1];
+      Pack<Tag, 1>::decode(src[(size_t)r * p.G * row_len + e], f);
+      lds[i] = f[0];
+    }
+  } else {
+    row0 = (int)blk * p.nq_block;
+    nrow = min(p.nq_block, p.n_row - row0);
+    const int span = nrow * p.G * row_len;
+    const bool vec16 = ((size_t)p.G * row_len * Tag::kBytes) % 16 == 0;
+    stage_rows_to_lds<Tag>(lds, (const char *)p.sla + (size_t)row0 * p.G * row_len * Tag::kBytes, span, vec16);
+  }
   __syncthreads();
 
   const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
   const int tpgp_log2 = p.lanes.tpgp_log2;
-  const int items = (nrow * p.G) << tpgp_log2;
+  const int items = (nrow * heads_here) << tpgp_log2;
   const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
   const int K = KT > 0 ? KT : p.K;
 
@@ -51,7 +74,7 @@ __global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLau
     const int chunk = it & ((1 << tpgp_log2) - 1);
     if (chunk >= p.lanes.tpg) continue;
     const int rg = it >> tpgp_log2;                 // (row, head) index inside the workgroup
-    const int lr = rg / p.G, g = rg - lr * p.G;
+    const int lr = rg / heads_here, g = g_fixed + rg - lr * heads_here;
     const int b = (row0 + lr) / p.Q;
     const float *s = lds + rg * row_len;
     float mx, inv;
@@ -108,18 +131,41 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
   }
   const int LK = p.L * p.K, row_len = 3 * LK;
   const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
-  const int row0 = (int)blk * p.nq_block;
-  const int nrow = min(p.nq_block, p.n_row - row0);
-  const int span = nrow * p.G * row_len;
+  int row0, nrow, heads_here = p.G, g_fixed = 0;
+  typedef typename RawWord<Tag::kBytes>::type elem_t;
   const bool vec16 = ((size_t)p.G * row_len * Tag::kBytes) % 16 == 0;
-  float *s_in = lds, *s_grad = lds + p.nq_block * p.G * row_len;
-  stage_rows_to_lds<Tag>(s_in, (const char *)p.sla + (size_t)row0 * p.G * row_len * Tag::kBytes, span, vec16);
+  if (p.head_major) {       // one head per workgroup, workgroups ordered [image][head][block of queries] (see the forward kernel)
+    const int blocks_per_image = (p.Q + p.nq_block - 1) / p.nq_block;
+    const int rb = (int)(blk % (uint32_t)blocks_per_image), bg = (int)(blk / (uint32_t)blocks_per_image);
+    const int b = bg / p.G;
+    g_fixed = bg - b * p.G;
+    heads_here = 1;
+    const int q0 = rb * p.nq_block;
+    nrow = min(p.nq_block, p.Q - q0);
+    row0 = b * p.Q + q0;
+  } else {
+    row0 = (int)blk * p.nq_block;
+    nrow = min(p.nq_block, p.n_row - row0);
+  }
+  const int span = nrow * heads_here * row_len;
+  float *s_in = lds, *s_grad = lds + p.nq_block * heads_here * row_len;
+  if (p.head_major) {
+    const elem_t *src = reinterpret_cast<const elem_t *>(p.sla) + ((size_t)row0 * p.G + g_fixed) * row_len;
+    for (int i = threadIdx.x; i < span; i += blockDim.x) {
+      const int r = i / row_len, e = i - r * row_len;
+      float f[1];
+      Pack<Tag, 1>::decode(src[(size_t)r * p.G * row_len + e], f);
+      s_in[i] = f[0];
+    }
+  } else {
+    stage_rows_to_lds<Tag>(s_in, (const char *)p.sla + (size_t)row0 * p.G * row_len * Tag::kBytes, span, vec16);
+  }
   __syncthreads();      // every slot of s_grad is written below: no clearing needed
 
   const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
   const __amdgpu_buffer_rsrc_t gacc = make_rsrc(p.grad_value_acc, p.value_bytes / Tag::kBytes * 4);
   const int tpgp_log2 = p.lanes.tpgp_log2, width = 1 << tpgp_log2;
-  const int items = (nrow * p.G) << tpgp_log2;
+  const int items = (nrow * heads_here) << tpgp_log2;
   const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
   const int K = KT > 0 ? KT : p.K;
   uint32_t go_max = 0;
@@ -128,7 +174,7 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
     const int chunk = it & (width - 1);
     const bool active = chunk < p.lanes.tpg;
     const int rg = it >> tpgp_log2;
-    const int lr = rg / p.G, g = rg - lr * p.G;
+    const int lr = rg / heads_here, g = g_fixed + rg - lr * heads_here;
     const int b = (row0 + lr) / p.Q;
     const float *s = s_in + rg * row_len;
     float *gs = s_grad + rg * row_len;
@@ -245,7 +291,16 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
     }
   }
   __syncthreads();
-  unstage_rows_from_lds<Tag>((char *)p.grad_sla + (size_t)row0 * p.G * row_len * Tag::kBytes, s_grad, span, vec16);
+  if (p.head_major) {
+    elem_t *dst = reinterpret_cast<elem_t *>(p.grad_sla) + ((size_t)row0 * p.G + g_fixed) * row_len;
+    for (int i = threadIdx.x; i < span; i += blockDim.x) {
+      const int r = i / row_len, e = i - r * row_len;
+      const float f[1] = {s_grad[i]};
+      dst[(size_t)r * p.G * row_len + e] = Pack<Tag, 1>::encode(f);
+    }
+  } else {
+    unstage_rows_from_lds<Tag>((char *)p.grad_sla + (size_t)row0 * p.G * row_len * Tag::kBytes, s_grad, span, vec16);
+  }
 }
 
 template <typename Tag, int CPT, int MODE>      // MODE -1: forward
@@ -264,7 +319,10 @@ hipError_t launch_k(const FdaLaunch &p, hipStream_t stream, dim3 grid, dim3 bloc
 
 template <typename Tag, int MODE>
 hipError_t launch_by_cpt(const FdaLaunch &p, hipStream_t stream) {
-  const dim3 grid((p.n_row + p.nq_block - 1) / p.nq_block), block(kBlockThreads);
+  const bool head_major = p.head_major != 0;
+  const dim3 grid(head_major ? (unsigned)((p.n_row / p.Q) * p.G * ((p.Q + p.nq_block - 1) / p.nq_block))
+                             : (unsigned)((p.n_row + p.nq_block - 1) / p.nq_block)),
+      block(kBlockThreads);
   const size_t lds = MODE >= 0 ? fda_backward_lds_bytes(p) : fda_forward_lds_bytes(p);
 #define FDA_CASE(N)                                                                       \
   case N:                                                                                 \
@@ -289,7 +347,7 @@ template <int MODE> hipError_t launch_by_dtype(int dtype, const FdaLaunch &p, hi
 }  // namespace
 
 size_t fda_forward_lds_bytes(const FdaLaunch &p) {
-  return (size_t)p.nq_block * p.G * 3 * p.L * p.K * sizeof(float);
+  return (size_t)p.nq_block * (p.head_major ? 1 : p.G) * 3 * p.L * p.K * sizeof(float);
 }
 size_t fda_backward_lds_bytes(const FdaLaunch &p) { return 2 * fda_forward_lds_bytes(p); }
 

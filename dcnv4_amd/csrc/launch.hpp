@@ -84,6 +84,7 @@ struct FdaLaunch {
   int n_row;
   int Q, N, G, D, L, K;
   int nq_block;             // queries per workgroup
+  int head_major;           // forward: a workgroup takes nq_block queries of ONE head, workgroups ordered [image][head][block]
   LaneMap lanes;
   // tiled grad_value path
   void *grad_value;         // [n_img, N, G, D] in the tensor dtype

@@ -367,3 +367,26 @@ def test_layer_norm_residual_rejects_unsupported_widths():
     w = torch.ones(8192, device="cuda", dtype=torch.float16)
     with pytest.raises(ValueError, match="too long"):
         cabi.layer_norm_residual(y, None, w, w, None, 1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16], ids=["fp32", "fp16"])
+def test_flash_deform_attn_head_major_order_matches_oracle_and_row_order(oracle, dtype, monkeypatch):
+    """A value image larger than half an L2 slice whose heads each fit one: the library then gives every workgroup one
+    head and orders workgroups [image][head][queries].  Same arithmetic per (query, head), so the same bits as the
+    row order, and parity with the oracle."""
+    B, shapes, G, D, K, Q = 2, [(64, 64), (32, 32)], 8, 32, 4, 150
+    v, shp, st, sla, go = make_fda_inputs(B, shapes, G, D, K, Q, seed=21, dtype=dtype, loc_lo=-0.05, loc_hi=1.05)
+    assert v[0].numel() * v.element_size() > (2 << 20)
+    args = (v.cuda(), shp.cuda(), st.cuda(), sla.cuda())
+    print(f"head-major case {dtype}", flush=True)
+    out = cabi.fda_forward(*args, K)
+    gv, gs = cabi.fda_backward(*args, go.cuda(), K)
+    monkeypatch.setenv("DCNV4_GFX950_FDA_ORDER", "rows")
+    out_rows = cabi.fda_forward(*args, K)
+    gv_rows, gs_rows = cabi.fda_backward(*args, go.cuda(), K)
+    assert torch.equal(out, out_rows) and torch.equal(gs, gs_rows) and torch.equal(gv, gv_rows)
+    want = oracle.flash_deform_attn_forward(cabi.f64(v), shp.numpy(), st.numpy(), cabi.f64(sla), K, coord_f32=True)
+    wgv, wgs = oracle.flash_deform_attn_backward(cabi.f64(v), shp.numpy(), st.numpy(), cabi.f64(sla), cabi.f64(go), K, coord_f32=True)
+    cabi.assert_close(out, want, *FWD_TOL[dtype], what="output")
+    cabi.assert_close(gv, wgv, *GRAD_TOL[dtype], what="grad_value")
+    cabi.assert_close(gs, wgs, *GRAD_TOL[dtype], what="grad_sampling_loc_attn")
