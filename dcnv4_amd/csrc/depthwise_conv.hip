@@ -166,7 +166,8 @@ __global__ void __launch_bounds__(kDwThreads) dwconv_grad_weight_kernel(const Dw
   // KH x KW input window sliding in registers: KH new input vectors and one grad_out vector per pixel
   typedef typename RawWord<kVecBytes>::type raw_t;
   const uint32_t n_rowseg = (uint32_t)p.B * p.Ho * p.n_seg;
-  const uint32_t first = blockIdx.x * (uint32_t)p.slab, last = min(n_rowseg, first + (uint32_t)p.slab);
+  const uint32_t slab_id = xcd_contiguous_block(blockIdx.x, gridDim.x);      // neighbouring slabs share rows: same XCD
+  const uint32_t first = slab_id * (uint32_t)p.slab, last = min(n_rowseg, first + (uint32_t)p.slab);
   if (live)
     for (uint32_t q = first + pl; q < last; q += px_lanes) {
       const uint32_t row = q / (uint32_t)p.n_seg;                       // b * Ho + y
@@ -214,7 +215,7 @@ __global__ void __launch_bounds__(kDwThreads) dwconv_grad_weight_kernel(const Dw
     }
 
   // lanes of the workgroup, one tap at a time: the first lane of each channel vector adds the others in order
-  float *part = p.partial + ((size_t)blockIdx.x * (kTaps + 1)) * p.C + (size_t)cvec * V;
+  float *part = p.partial + ((size_t)slab_id * (kTaps + 1)) * p.C + (size_t)cvec * V;
 #pragma unroll
   for (int k = 0; k <= kTaps; ++k) {
     __syncthreads();
