@@ -133,6 +133,12 @@ bool tiled_grad_value(int D) { return D <= kTiledMaxGroupChannels && g_opt_scatt
 // Tuning override, read on every call: DCNV4_GFX950_REACH = distance (input pixels) from an output
 // pixel's reference point that the tiled kernels cover; sampling points beyond it take the
 // global-memory paths.  Default 5.
+// Tuning override, read on every call: DCNV4_GFX950_TILE=16 keeps the tiled grad_value kernel on 16x16 tiles.
+bool large_tiles_enabled() {
+  const char *e = getenv("DCNV4_GFX950_TILE");
+  return !(e && strcmp(e, "16") == 0);
+}
+
 int reach_setting() {
   const char *e = getenv("DCNV4_GFX950_REACH");
   const int r = g_opt_reach > 0 ? g_opt_reach - 1 : (e ? atoi(e) : 5);
@@ -172,26 +178,35 @@ int plan_grad_value_tiles(DcnLaunch *L, int elem_bytes_of_launch) {
   const long long per_cell = (long long)(2 * L->reach + 1) * (2 * L->reach + 1) * L->Kp;
   const int fix32 = 31 - ceil_log2((int)std::min<long long>(per_cell, 1 << 30));
   L->pack32 = (elem_bytes_of_launch == 2 && D > 8 && fix32 >= 18) ? 1 : 0;
-  // power-of-two tiles (the reach rule uses shifts); shrink until the LDS footprint fits
-  L->tile_h_log2 = 4;
-  L->tile_w_log2 = 4;
-  while (L->tile_h_log2 > 0 && (1 << (L->tile_h_log2 - 1)) >= L->H) --L->tile_h_log2;
-  while (L->tile_w_log2 > 0 && (1 << (L->tile_w_log2 - 1)) >= L->W) --L->tile_w_log2;
+  // Power-of-two tiles (the reach rule uses shifts); shrink until the LDS footprint fits.  Images wider or taller
+  // than 16 pixels first try 32x32 tiles with ONE group per workgroup: the accumulators take the same LDS as four
+  // groups of a 16x16 tile, the workgroup count is the same, but a tile visits (32 + 2 reach)^2 / 32^2 = 1.7 output
+  // pixels per input pixel instead of 2.6 (1.0 when the tile covers the whole image), and every sampling point
+  // belongs to exactly one group, so nothing is evaluated twice.
   auto visited = [&](int tile, int stride) { return (tile + 2 * L->reach + stride - 1) / stride + 1; };
-  for (;;) {
-    L->tile_h = 1 << L->tile_h_log2;
-    L->tile_w = 1 << L->tile_w_log2;
-    const int row = visited(L->tile_w, L->sw);
-    bool fits = false;
-    for (int rows = 4; rows >= 1 && !fits; --rows) {       // up to 4 visited rows per strip
-      L->strip_pix = std::min(rows * row, 1023);           // pixel index field of a hit record
-      fits = dcnv4_grad_value_lds_bytes(*L) <= kMaxLdsPerWorkgroup - 256;
+  auto plan = [&](int max_log2, int groups) {
+    L->ng_chunk = groups;
+    L->tile_h_log2 = L->tile_w_log2 = max_log2;
+    while (L->tile_h_log2 > 0 && (1 << (L->tile_h_log2 - 1)) >= L->H) --L->tile_h_log2;
+    while (L->tile_w_log2 > 0 && (1 << (L->tile_w_log2 - 1)) >= L->W) --L->tile_w_log2;
+    for (;;) {
+      L->tile_h = 1 << L->tile_h_log2;
+      L->tile_w = 1 << L->tile_w_log2;
+      const int row = visited(L->tile_w, L->sw);
+      for (int rows = 4; rows >= 1; --rows) {                // up to 4 visited rows per strip
+        L->strip_pix = std::min(rows * row, 1023);           // pixel index field of a hit record
+        if (dcnv4_grad_value_lds_bytes(*L) <= kMaxLdsPerWorkgroup - 256) return true;
+      }
+      if (max_log2 > 4) return false;                        // the large-tile plan is all or nothing
+      if (L->tile_h_log2 > 0 && L->tile_h_log2 >= L->tile_w_log2) --L->tile_h_log2;
+      else if (L->tile_w_log2 > 0) --L->tile_w_log2;
+      else return false;
     }
-    if (fits) break;
-    if (L->tile_h_log2 > 0 && L->tile_h_log2 >= L->tile_w_log2) --L->tile_h_log2;
-    else if (L->tile_w_log2 > 0) --L->tile_w_log2;
-    else return fail(DCNV4_ERR_RUNTIME, "kernel with %d taps and %d group channels does not fit the tiled backward", L->Kp, D);
-  }
+  };
+  const int groups16 = L->ng_chunk;
+  const bool large = (L->H > 16 || L->W > 16) && large_tiles_enabled() && plan(5, 1);
+  if (!large && !plan(4, groups16))
+    return fail(DCNV4_ERR_RUNTIME, "kernel with %d taps and %d group channels does not fit the tiled backward", L->Kp, D);
   const long long contributions = (long long)visited(L->tile_h, L->sh) * visited(L->tile_w, L->sw) * L->Kp;
   // a term must stay below 2^51 (the conversion's range), a sum below 2^62
   L->fix_bits = std::min(50, 62 - ceil_log2((int)std::min<long long>(contributions, 1 << 30)));

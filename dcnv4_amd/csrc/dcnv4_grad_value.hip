@@ -40,12 +40,12 @@ constexpr int kValThreads = 1024;
 constexpr int kWaves = kValThreads / kWave;
 constexpr int kTrashPad = 64;
 constexpr int kMaxChunkGroups = 4;      // rows of a wave <-> groups of the chunk
-constexpr int kCellBits = 9;            // cell index 0..n_cells (n_cells = trash), tiles up to 16x16
+constexpr int kMetaPosBits = 6;         // row + 1 and column + 1 of a record's first corner inside the tile: 0..32
 
-struct HitMeta {
-  uint32_t cells012;    // accumulator cell of corners 0,1,2 (9 bits each); n_cells = "nowhere" (weight 0)
-  uint32_t cell3_px;    // cell of corner 3 | strip-local pixel << 9
-};
+// A hit record's second word: (row + 1) | (column + 1) << 6 of the first corner relative to the tile (-1 when the
+// corner block starts one row or column before it), the corners inside the tile (4 bits) << 12, and the strip-local
+// output pixel << 16.
+typedef uint32_t HitMeta;
 
 // lanes that apply one hit record, and channels per lane (1, 2, 4 or 8; odd counts round up)
 __host__ __device__ inline int lanes_per_record(int D) { return D <= 16 ? 2 : (D <= 32 ? 4 : 8); }
@@ -220,7 +220,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
         const bool valid_item = it.in_range && it.px < npx;
         bool hit = false;
         f32x4 w = {0.f, 0.f, 0.f, 0.f};
-        HitMeta meta = {0u, 0u};
+        HitMeta meta = 0u;
         if (valid_item) {
           const elem_t *om = om_img + (it.om_off + (uint32_t)s_idx * om_strip);
           const float off_x = round == 0 ? to_f(pf.ox) : load_f(om + 2 * it.t);
@@ -244,16 +244,9 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
               m = __expf(m - mx) / sum;
             }
             const float ms = ldexpf(m, p.fix_bits - e_m);
-            const int cell = (ly << p.tile_w_log2) + lx;
-            uint32_t cells[4];
 #pragma unroll
-            for (int cn = 0; cn < 4; ++cn) {
-              const bool ok = valid & (1u << cn);
-              cells[cn] = ok ? (uint32_t)(cell + (cn >> 1) * p.tile_w + (cn & 1)) : (uint32_t)n_cells;
-              w[cn] = ok ? ms * tp.w[cn] : 0.f;
-            }
-            meta.cells012 = cells[0] | (cells[1] << kCellBits) | (cells[2] << (2 * kCellBits));
-            meta.cell3_px = cells[3] | ((uint32_t)it.px << kCellBits);
+            for (int cn = 0; cn < 4; ++cn) w[cn] = (valid & (1u << cn)) ? ms * tp.w[cn] : 0.f;
+            meta = (uint32_t)(ly + 1) | ((uint32_t)(lx + 1) << kMetaPosBits) | (valid << (2 * kMetaPosBits)) | ((uint32_t)it.px << 16);
           }
         }
       // append the wave's hits to its group's list: one LDS counter bump per wave
@@ -307,15 +300,15 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       for (int u = 0; u < kUnits; ++u) unit_of[u] = (u + first_unit) & (kUnits - 1);
       for (uint32_t i0 = wave * rows_per_group; i0 < n_max; i0 += kWaves * rows_per_group) {
         const uint32_t i = i0 + my_slot;
-        f32x4 w = {0.f, 0.f, 0.f, 0.f};
-        HitMeta meta = {(uint32_t)n_cells | ((uint32_t)n_cells << kCellBits) | ((uint32_t)n_cells << (2 * kCellBits)),
-                        (uint32_t)n_cells};
         if (i >= n_mine) continue;        // rows past the end of their group's list sit this pass out
-        w = hit_w[lane_group * list_cap + i];
-        meta = hit_meta[lane_group * list_cap + i];
-        const float *go_px = go_lane + (meta.cell3_px >> kCellBits) * ch_stride;
-        const uint32_t cells[4] = {meta.cells012 & 511u, (meta.cells012 >> kCellBits) & 511u,
-                                   (meta.cells012 >> (2 * kCellBits)) & 511u, meta.cell3_px & 511u};
+        const f32x4 w = hit_w[lane_group * list_cap + i];
+        const HitMeta meta = hit_meta[lane_group * list_cap + i];
+        const float *go_px = go_lane + (meta >> 16) * ch_stride;
+        const int first_cell = ((int)(meta & 63u) - 1) * p.tile_w + (int)((meta >> kMetaPosBits) & 63u) - 1;
+        uint32_t cells[4];
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn)      // corners outside the tile carry weight 0: send them to the trash cell
+          cells[cn] = (meta & (1u << (2 * kMetaPosBits + cn))) ? (uint32_t)(first_cell + (cn >> 1) * p.tile_w + (cn & 1)) : (uint32_t)n_cells;
         const float wv[4] = {w.x, w.y, w.z, w.w};
         unsigned long long *dst[4];
 #pragma unroll
@@ -356,11 +349,16 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   // fallback kernel then adds every corner)
   const int e_out = e_go + e_m - p.fix_bits;
   const int n_ch = ng * D;
-  for (int cell = wave; cell < th * tw; cell += kValThreads / kWave) {     // one cell per wave: contiguous channels
+  // a wave writes whole cells (contiguous channels): one per step, or 64 / n_ch of them when the chunk is narrow
+  const int cells_per_wave = (n_ch <= 32 && (kWave % n_ch) == 0) ? kWave / n_ch : 1;
+  const int sub = cells_per_wave > 1 ? lane / n_ch : 0, lane_ch = cells_per_wave > 1 ? lane - sub * n_ch : lane;
+  for (int cell0 = wave * cells_per_wave; cell0 < th * tw; cell0 += kWaves * cells_per_wave) {
+    const int cell = cell0 + sub;
+    if (cell >= th * tw) continue;
     const int ly = cell / tw, lx = cell - ly * tw;
     const unsigned long long *src = acc + ((ly << p.tile_w_log2) + lx) * acc_stride;
     elem_t *dst = reinterpret_cast<elem_t *>(p.grad_value) + (((size_t)b * p.H + ty0 + ly) * p.W + tx0 + lx) * C + g0 * D;
-    for (int ch = lane; ch < n_ch; ch += kWave) {
+    for (int ch = lane_ch; ch < n_ch; ch += (cells_per_wave > 1 ? n_ch : kWave)) {
       float f[1];
       if constexpr (PACK) {
         const int g = ch / D, cg = ch - g * D;

@@ -76,6 +76,8 @@ KERNEL_PATHS = {
     "reach1": {"DCNV4_GFX950_REACH": "1"},
     "reach0": {"DCNV4_GFX950_REACH": "0"},
     "reach9": {"DCNV4_GFX950_REACH": "9"},
+    "tile16": {"DCNV4_GFX950_TILE": "16"},                                   # grad_value on 16x16 tiles, four groups each
+    "tile16_reach1": {"DCNV4_GFX950_TILE": "16", "DCNV4_GFX950_REACH": "1"},
 }
 
 
