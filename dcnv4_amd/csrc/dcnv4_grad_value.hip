@@ -126,7 +126,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
     // this image's tensors, addressed with 32-bit element offsets (the entry point checks they fit)
     const elem_t *om_img = om_g + (size_t)b * p.Q * p.P_pad;
     const elem_t *go_img = go_g + (size_t)b * p.Q * C;
-    constexpr int kStageRounds = 2;     // pixels per wave whose grad_out is prefetched (16 waves: 32 pixels)
+    constexpr int kStageRounds = 3;     // staging rounds whose grad_out is prefetched (a round: 16 waves x ppw pixels)
 
     // Phase A work item of a (wave slot, lane): group, strip-local pixel, tap.  The decode depends only
     // on the strip geometry, not on the strip, so the first round's item is decoded once per lane.
@@ -160,19 +160,22 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       return it;
     };
     const Item my_item = item_of(wave);
-    // staging: wave w parks pixel w (+16, ...) of the strip, lane = channel of the chunk
+    // staging: a wave parks ppw pixels of the strip per round (one when the chunk is wider than 32 channels),
+    // lane = (pixel of the round, channel of the chunk)
+    const int ppw = (ch_stride <= 32 && kWave % ch_stride == 0) ? kWave / ch_stride : 1;
+    const int lane_px = ppw > 1 ? lane / ch_stride : 0, lane_ch = ppw > 1 ? lane - lane_px * ch_stride : lane;
     uint32_t go_off[kStageRounds];
 #pragma unroll
     for (int u = 0; u < kStageRounds; ++u) {
-      const int px = wave + u * kWaves, r = px / nwx;
-      go_off[u] = (uint32_t)(((ho_lo + r) * p.Wo + wo_lo + (px - r * nwx)) * C + g0 * D + lane);
+      const int px = (wave + u * kWaves) * ppw + lane_px, r = px / nwx;
+      go_off[u] = (uint32_t)(((ho_lo + r) * p.Wo + wo_lo + (px - r * nwx)) * C + g0 * D + lane_ch);
     }
     const uint32_t om_strip = (uint32_t)(rows_per_strip * p.Wo) * (uint32_t)p.P_pad;   // offset step per strip
     const uint32_t go_strip = (uint32_t)(rows_per_strip * p.Wo * C);
 
     struct Prefetch {
       elem_t ox, oy, m;                 // phase A, first round: this lane's tap
-      elem_t go[kStageRounds];          // staging: this lane's channel of up to two pixels
+      elem_t go[kStageRounds];          // staging: this lane's channel of its pixel in the first rounds
     };
     // loads of the next strip, issued before the current strip's phase B so their latency hides there
     auto prefetch = [&](int s_idx, int npx) {
@@ -185,7 +188,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
 #pragma unroll
       for (int u = 0; u < kStageRounds; ++u) {
         pf.go[u] = elem_t(0);
-        if (wave + u * kWaves < npx && lane < ng * D) pf.go[u] = go_img[go_off[u] + (uint32_t)s_idx * go_strip];
+        if ((wave + u * kWaves) * ppw + lane_px < npx && lane_ch < ng * D) pf.go[u] = go_img[go_off[u] + (uint32_t)s_idx * go_strip];
       }
       return pf;
     };
@@ -200,19 +203,26 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       uint32_t *count = s_count + (s_idx & 1) * kMaxChunkGroups;
       __syncthreads();      // previous strip's phase B is done (first time: acc and counters are clear)
 
-      // ---- park the strip's grad_out (this chunk's channels), normalised to [-1, 1]: a wave per pixel
-      for (int px = wave, u = 0; px < npx; px += kWaves, ++u)
-        for (int ch = lane; ch < ch_stride; ch += kWave) {
+      // ---- park the strip's grad_out (this chunk's channels), normalised to [-1, 1]
+      for (int base = wave * ppw, u = 0; base < npx; base += kWaves * ppw, ++u) {
+        const int px = base + lane_px;
+        if (px >= npx) continue;
+        for (int ch = lane_ch; ch < ch_stride; ch += (ppw > 1 ? ch_stride : kWave)) {
           float g = 0.f;
           if (ch < ng * D) {
-            if (u < kStageRounds && ch < kWave) g = to_f(u == 0 ? pf.go[0] : pf.go[kStageRounds - 1]);
-            else {
+            if (u < kStageRounds && ch < kWave) {
+              elem_t raw = pf.go[0];
+#pragma unroll
+              for (int v = 1; v < kStageRounds; ++v) raw = u == v ? pf.go[v] : raw;
+              g = to_f(raw);
+            } else {
               const int r = px / nwx;
               g = load_f(go_img + ((size_t)((hs + r) * p.Wo + wo_lo + (px - r * nwx)) * C + g0 * D + ch));
             }
           }
           s_go[px * ch_stride + ch] = ldexpf(g, -e_go);
         }
+      }
 
       // ---- phase A: one lane per (group, pixel, tap); a wave never mixes groups
       for (int wk = wave, round = 0; wk < n_wk; wk += kWaves, ++round) {
