@@ -15,6 +15,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
 
 // dtype tags; the numeric values are the dtype codes of the C ABI
 struct F32 { static constexpr int kBytes = 4; static constexpr int kCode = 0; };

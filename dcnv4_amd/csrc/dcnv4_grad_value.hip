@@ -86,9 +86,9 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   const int list_cap = p.strip_pix * Kp;                // hit records per group list
   unsigned long long *acc = lds64;
   f32x4 *hit_w = reinterpret_cast<f32x4 *>(lds64 + n_acc);                       // [ng_chunk][list_cap]
-  HitMeta *hit_meta = reinterpret_cast<HitMeta *>(hit_w + p.ng_chunk * list_cap);  // [ng_chunk][list_cap]
-  float *s_go = reinterpret_cast<float *>(hit_meta + p.ng_chunk * list_cap);       // [strip_pix][ch_stride]
-  uint32_t *s_count = reinterpret_cast<uint32_t *>(s_go + p.strip_pix * ch_stride);  // [kMaxChunkGroups]
+  float *s_go = reinterpret_cast<float *>(hit_w + p.ng_chunk * list_cap);          // [strip_pix][ch_stride], 16-byte aligned
+  HitMeta *hit_meta = reinterpret_cast<HitMeta *>(s_go + p.strip_pix * ch_stride);  // [ng_chunk][list_cap]
+  uint32_t *s_count = reinterpret_cast<uint32_t *>(hit_meta + p.ng_chunk * list_cap);  // two sets of [kMaxChunkGroups]
 
   const uint32_t gmax = p.state->go_max_bits, mmax = p.state->mask_max_bits;
   const bool finite = gmax < 0x7f800000u && mmax < 0x7f800000u;
@@ -126,7 +126,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
     // this image's tensors, addressed with 32-bit element offsets (the entry point checks they fit)
     const elem_t *om_img = om_g + (size_t)b * p.Q * p.P_pad;
     const elem_t *go_img = go_g + (size_t)b * p.Q * C;
-    constexpr int kStageRounds = 3;     // staging rounds whose grad_out is prefetched (a round: 16 waves x ppw pixels)
+    constexpr int kStageRounds = 2;     // staging rounds whose grad_out is prefetched (a round: 16 waves x ppw pixels)
 
     // Phase A work item of a (wave slot, lane): group, strip-local pixel, tap.  The decode depends only
     // on the strip geometry, not on the strip, so the first round's item is decoded once per lane.
@@ -159,11 +159,20 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       it.x_base = sub_rn((float)(cx0 + wo * p.sw), x_sub);
       return it;
     };
-    const Item my_item = item_of(wave);
-    // staging: a wave parks ppw pixels of the strip per round (one when the chunk is wider than 32 channels),
-    // lane = (pixel of the round, channel of the chunk)
-    const int ppw = (ch_stride <= 32 && kWave % ch_stride == 0) ? kWave / ch_stride : 1;
-    const int lane_px = ppw > 1 ? lane / ch_stride : 0, lane_ch = ppw > 1 ? lane - lane_px * ch_stride : lane;
+    constexpr int kItemRounds = 2;      // phase A rounds whose items are decoded once and whose taps are prefetched
+    Item my_item[kItemRounds];
+#pragma unroll
+    for (int v = 0; v < kItemRounds; ++v) my_item[v] = item_of(wave + v * kWaves);
+    // staging: a lane parks one 16-byte vector of grad_out (kVec channels of a pixel), a wave ppw whole pixels per
+    // round; the first kStageRounds rounds are prefetched.  Group widths that are not whole vectors, and chunks
+    // whose vector count is not a power of two, park element by element without prefetch.
+    constexpr int kVec = 16 / Tag::kBytes;
+    typedef typename Pack<Tag, kVec>::raw_t vec_t;
+    const int px_lanes = ch_stride / kVec;
+    const bool vec_park = D % kVec == 0 && px_lanes <= kWave && (px_lanes & (px_lanes - 1)) == 0;
+    const int px_lanes_log2 = vec_park ? 31 - __builtin_clz(px_lanes) : 0;
+    const int ppw = kWave >> px_lanes_log2;
+    const int lane_px = lane >> px_lanes_log2, lane_ch = (lane & (px_lanes - 1)) * kVec;
     uint32_t go_off[kStageRounds];
 #pragma unroll
     for (int u = 0; u < kStageRounds; ++u) {
@@ -174,21 +183,25 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
     const uint32_t go_strip = (uint32_t)(rows_per_strip * p.Wo * C);
 
     struct Prefetch {
-      elem_t ox, oy, m;                 // phase A, first round: this lane's tap
-      elem_t go[kStageRounds];          // staging: this lane's channel of its pixel in the first rounds
+      elem_t ox[kItemRounds], oy[kItemRounds], m[kItemRounds];      // phase A, first rounds: this lane's tap
+      vec_t go[kStageRounds];           // staging: this lane's vector of its pixel in the first rounds
     };
     // loads of the next strip, issued before the current strip's phase B so their latency hides there
     auto prefetch = [&](int s_idx, int npx) {
       Prefetch pf;
-      pf.ox = pf.oy = pf.m = elem_t(0);
-      if (my_item.in_range && my_item.px < npx) {
-        const elem_t *om = om_img + (my_item.om_off + (uint32_t)s_idx * om_strip);
-        pf.ox = om[2 * my_item.t]; pf.oy = om[2 * my_item.t + 1]; pf.m = om[2 * Kp + my_item.t];
+#pragma unroll
+      for (int v = 0; v < kItemRounds; ++v) {
+        pf.ox[v] = pf.oy[v] = pf.m[v] = elem_t(0);
+        if (my_item[v].in_range && my_item[v].px < npx) {
+          const elem_t *om = om_img + (my_item[v].om_off + (uint32_t)s_idx * om_strip);
+          pf.ox[v] = om[2 * my_item[v].t]; pf.oy[v] = om[2 * my_item[v].t + 1]; pf.m[v] = om[2 * Kp + my_item[v].t];
+        }
       }
 #pragma unroll
       for (int u = 0; u < kStageRounds; ++u) {
-        pf.go[u] = elem_t(0);
-        if ((wave + u * kWaves) * ppw + lane_px < npx && lane_ch < ng * D) pf.go[u] = go_img[go_off[u] + (uint32_t)s_idx * go_strip];
+        pf.go[u] = vec_t{};
+        if (vec_park && (wave + u * kWaves) * ppw + lane_px < npx && lane_ch < ng * D)
+          pf.go[u] = *reinterpret_cast<const vec_t *>(go_img + (go_off[u] + (uint32_t)s_idx * go_strip));
       }
       return pf;
     };
@@ -204,37 +217,57 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       __syncthreads();      // previous strip's phase B is done (first time: acc and counters are clear)
 
       // ---- park the strip's grad_out (this chunk's channels), normalised to [-1, 1]
-      for (int base = wave * ppw, u = 0; base < npx; base += kWaves * ppw, ++u) {
-        const int px = base + lane_px;
-        if (px >= npx) continue;
-        for (int ch = lane_ch; ch < ch_stride; ch += (ppw > 1 ? ch_stride : kWave)) {
-          float g = 0.f;
-          if (ch < ng * D) {
-            if (u < kStageRounds && ch < kWave) {
-              elem_t raw = pf.go[0];
+      if (vec_park) {
+        for (int base = wave * ppw, u = 0; base < npx; base += kWaves * ppw, ++u) {
+          const int px = base + lane_px;
+          if (px >= npx) continue;
+          float f[kVec];
+#pragma unroll
+          for (int i = 0; i < kVec; ++i) f[i] = 0.f;
+          if (lane_ch < ng * D) {
+            vec_t raw = pf.go[0];
+            if (u < kStageRounds) {
 #pragma unroll
               for (int v = 1; v < kStageRounds; ++v) raw = u == v ? pf.go[v] : raw;
-              g = to_f(raw);
             } else {
               const int r = px / nwx;
-              g = load_f(go_img + ((size_t)((hs + r) * p.Wo + wo_lo + (px - r * nwx)) * C + g0 * D + ch));
+              raw = *reinterpret_cast<const vec_t *>(go_img + ((uint32_t)(((hs + r) * p.Wo + wo_lo + (px - r * nwx)) * C) + g0 * D + lane_ch));
             }
+            Pack<Tag, kVec>::decode(raw, f);
           }
-          s_go[px * ch_stride + ch] = ldexpf(g, -e_go);
+          f32x4 *dst = reinterpret_cast<f32x4 *>(s_go + px * ch_stride + lane_ch);
+#pragma unroll
+          for (int i = 0; i < kVec / 4; ++i)
+            dst[i] = f32x4{ldexpf(f[4 * i], -e_go), ldexpf(f[4 * i + 1], -e_go), ldexpf(f[4 * i + 2], -e_go), ldexpf(f[4 * i + 3], -e_go)};
+        }
+      } else {
+        for (int px = wave; px < npx; px += kWaves) {
+          const int r = px / nwx;
+          const elem_t *src = go_img + ((uint32_t)(((hs + r) * p.Wo + wo_lo + (px - r * nwx)) * C) + g0 * D);
+          for (int ch = lane; ch < ch_stride; ch += kWave) s_go[px * ch_stride + ch] = ch < ng * D ? ldexpf(load_f(src + ch), -e_go) : 0.f;
         }
       }
 
       // ---- phase A: one lane per (group, pixel, tap); a wave never mixes groups
       for (int wk = wave, round = 0; wk < n_wk; wk += kWaves, ++round) {
-        const Item it = round == 0 ? my_item : item_of(wk);
+        Item it;
+        elem_t pf_ox = elem_t(0), pf_oy = elem_t(0), pf_m = elem_t(0);
+        if (round < kItemRounds) {
+          it = my_item[0]; pf_ox = pf.ox[0]; pf_oy = pf.oy[0]; pf_m = pf.m[0];
+#pragma unroll
+          for (int v = 1; v < kItemRounds; ++v)
+            if (round == v) { it = my_item[v]; pf_ox = pf.ox[v]; pf_oy = pf.oy[v]; pf_m = pf.m[v]; }
+        } else {
+          it = item_of(wk);
+        }
         const bool valid_item = it.in_range && it.px < npx;
         bool hit = false;
         f32x4 w = {0.f, 0.f, 0.f, 0.f};
         HitMeta meta = 0u;
         if (valid_item) {
           const elem_t *om = om_img + (it.om_off + (uint32_t)s_idx * om_strip);
-          const float off_x = round == 0 ? to_f(pf.ox) : load_f(om + 2 * it.t);
-          const float off_y = round == 0 ? to_f(pf.oy) : load_f(om + 2 * it.t + 1);
+          const float off_x = round < kItemRounds ? to_f(pf_ox) : load_f(om + 2 * it.t);
+          const float off_y = round < kItemRounds ? to_f(pf_oy) : load_f(om + 2 * it.t + 1);
           const float y_base = sub_rn((float)(cy0 + (hs + it.r) * p.sh), y_sub);
           const float x = add_rn(it.x_base, mul_rn(add_rn((float)(it.ti * p.dw), off_x), p.offset_scale));
           const float y = add_rn(y_base, mul_rn(add_rn((float)(it.tj * p.dh), off_y), p.offset_scale));
@@ -246,7 +279,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
                                              ((uint32_t)(r1 && c0) << 2) | ((uint32_t)(r1 && c1) << 3));
           hit = valid != 0;
           if (hit) {
-            float m = round == 0 ? to_f(pf.m) : load_f(om + 2 * Kp + it.t);
+            float m = round < kItemRounds ? to_f(pf_m) : load_f(om + 2 * Kp + it.t);
             if (p.softmax) {          // rare: normalise over this group's taps
               float mx = load_f(om + 2 * Kp), sum = 0.f;
               for (int k = 1; k < Kp; ++k) mx = fmaxf(mx, load_f(om + 2 * Kp + k));
@@ -359,25 +392,54 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   // fallback kernel then adds every corner)
   const int e_out = e_go + e_m - p.fix_bits;
   const int n_ch = ng * D;
-  // a wave writes whole cells (contiguous channels): one per step, or 64 / n_ch of them when the chunk is narrow
-  const int cells_per_wave = (n_ch <= 32 && (kWave % n_ch) == 0) ? kWave / n_ch : 1;
-  const int sub = cells_per_wave > 1 ? lane / n_ch : 0, lane_ch = cells_per_wave > 1 ? lane - sub * n_ch : lane;
-  for (int cell0 = wave * cells_per_wave; cell0 < th * tw; cell0 += kWaves * cells_per_wave) {
-    const int cell = cell0 + sub;
-    if (cell >= th * tw) continue;
-    const int ly = cell / tw, lx = cell - ly * tw;
-    const unsigned long long *src = acc + ((ly << p.tile_w_log2) + lx) * acc_stride;
-    elem_t *dst = reinterpret_cast<elem_t *>(p.grad_value) + (((size_t)b * p.H + ty0 + ly) * p.W + tx0 + lx) * C + g0 * D;
-    for (int ch = lane_ch; ch < n_ch; ch += (cells_per_wave > 1 ? n_ch : kWave)) {
-      float f[1];
+  // A lane converts four consecutive channels of a cell and stores them as one vector, a wave whole cells (64 / lanes
+  // per cell of them per step).  Group widths that are not multiples of four, and chunks whose lane count per cell is
+  // not a power of two, go element by element, one cell per wave and step.
+  const int cell_lanes = n_ch >> 2;
+  if ((D & 3) == 0 && cell_lanes <= kWave && (cell_lanes & (cell_lanes - 1)) == 0) {
+    const int cl_log2 = 31 - __builtin_clz(cell_lanes);
+    const int sub = lane >> cl_log2, ch = (lane & (cell_lanes - 1)) * 4;
+    const int g = ch / D, cg = ch - g * D;
+    const int word = PACK ? g * group_words + (cg >> 1) : ch;
+    typedef typename Pack<Tag, 4>::raw_t out_t;
+    for (int cell0 = wave << (6 - cl_log2); cell0 < n_cells; cell0 += kValThreads >> cl_log2) {
+      const int cell = cell0 + sub;
+      const int ly = cell >> p.tile_w_log2, lx = cell & (p.tile_w - 1);
+      if (ly >= th || lx >= tw) continue;
+      const u64x2 *src = reinterpret_cast<const u64x2 *>(acc + cell * acc_stride + word);
+      float f[4];
       if constexpr (PACK) {
-        const int g = ch / D, cg = ch - g * D;
-        f[0] = ldexpf((float)packed_field(src[g * group_words + (cg >> 1)], cg & 1), e_out);
+        const u64x2 a = src[0];
+        const unsigned long long a0 = a.x, a1 = a.y;
+        f[0] = ldexpf((float)packed_field(a0, 0), e_out); f[1] = ldexpf((float)packed_field(a0, 1), e_out);
+        f[2] = ldexpf((float)packed_field(a1, 0), e_out); f[3] = ldexpf((float)packed_field(a1, 1), e_out);
       } else {
-        const unsigned long long a = src[ch];
-        f[0] = (float)ldexp((double)(int)(a >> 32) * 4294967296.0 + (double)(uint32_t)a, e_out);
+        const u64x2 a = src[0], b2 = src[1];
+        const unsigned long long w4[4] = {a.x, a.y, b2.x, b2.y};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          f[i] = (float)ldexp((double)(int)(w4[i] >> 32) * 4294967296.0 + (double)(uint32_t)w4[i], e_out);
       }
-      dst[ch] = Pack<Tag, 1>::encode(f);
+      out_t *dst = reinterpret_cast<out_t *>(reinterpret_cast<elem_t *>(p.grad_value) +
+                                             ((((size_t)b * p.H + ty0 + ly) * p.W + tx0 + lx) * C + g0 * D + ch));
+      *dst = Pack<Tag, 4>::encode(f);
+    }
+  } else {
+    for (int cell = wave; cell < th * tw; cell += kWaves) {
+      const int ly = cell / tw, lx = cell - ly * tw;
+      const unsigned long long *src = acc + ((ly << p.tile_w_log2) + lx) * acc_stride;
+      elem_t *dst = reinterpret_cast<elem_t *>(p.grad_value) + (((size_t)b * p.H + ty0 + ly) * p.W + tx0 + lx) * C + g0 * D;
+      for (int ch = lane; ch < n_ch; ch += kWave) {
+        float f[1];
+        if constexpr (PACK) {
+          const int g = ch / D, cg = ch - g * D;
+          f[0] = ldexpf((float)packed_field(src[g * group_words + (cg >> 1)], cg & 1), e_out);
+        } else {
+          const unsigned long long a = src[ch];
+          f[0] = (float)ldexp((double)(int)(a >> 32) * 4294967296.0 + (double)(uint32_t)a, e_out);
+        }
+        dst[ch] = Pack<Tag, 1>::encode(f);
+      }
     }
   }
 }
@@ -429,8 +491,8 @@ size_t dcnv4_grad_value_lds_bytes(const DcnLaunch &p) {
   const size_t ch_stride = (size_t)p.ng_chunk * p.D, list = (size_t)p.ng_chunk * p.strip_pix * p.Kp;
   const size_t acc_stride = acc_words_per_cell(p.ng_chunk, p.D, p.pack32 != 0);
   return ((((size_t)(p.tile_h * p.tile_w + 1) * acc_stride + kTrashPad + 1) & ~size_t(1)) * sizeof(unsigned long long)) +  // accumulators
-         list * (sizeof(f32x4) + sizeof(HitMeta)) +                                                    // hit lists
-         (size_t)p.strip_pix * ch_stride * sizeof(float) + 2 * kMaxChunkGroups * sizeof(uint32_t);     // grad_out, two counter sets
+         list * sizeof(f32x4) + (size_t)p.strip_pix * ch_stride * sizeof(float) +                      // hit weights, grad_out
+         list * sizeof(HitMeta) + 2 * kMaxChunkGroups * sizeof(uint32_t);                              // hit cells, two counter sets
 }
 
 hipError_t launch_dcnv4_grad_value(int dtype, const DcnLaunch &p, hipStream_t stream) {
