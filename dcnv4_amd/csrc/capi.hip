@@ -193,7 +193,7 @@ int plan_grad_value_tiles(DcnLaunch *L, int elem_bytes_of_launch) {
       L->tile_h = 1 << L->tile_h_log2;
       L->tile_w = 1 << L->tile_w_log2;
       const int row = visited(L->tile_w, L->sw);
-      for (int rows = 4; rows >= 1; --rows) {                // up to 4 visited rows per strip
+      for (int rows = 8; rows >= 1; --rows) {                // up to 8 visited rows per strip: every strip costs two barriers
         L->strip_pix = std::min(rows * row, 1023);           // pixel index field of a hit record
         if (dcnv4_grad_value_lds_bytes(*L) <= kMaxLdsPerWorkgroup - 256) return true;
       }

@@ -62,7 +62,11 @@ __host__ __device__ inline int acc_words_per_cell(int ng_chunk, int D, bool pack
   return ng_chunk * acc_words_per_group(D, pack);
 }
 
-template <typename Tag, int KP, int R, int CPL, bool PACK>
+// FAST: 32-pixel-wide tiles, one group of 16 channels per workgroup.  The four corners of a hit record then lie at
+// compile-time distances from the first one, so their addresses are immediates of one base register; a corner outside
+// the tile carries weight zero and its add lands, harmlessly, on whatever the LDS holds there - another cell, or the
+// hit weights in front of the accumulators or the parked grad_out behind them (adding the integer 0 changes nothing).
+template <typename Tag, int KP, int R, int CPL, bool PACK, bool FAST>
 __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const DcnLaunch p) {
   extern __shared__ unsigned long long lds64[];
   const int Kp = p.Kp, D = p.D, C = p.G * p.D;
@@ -84,9 +88,10 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   // whose channel index runs past D (group widths that are not multiples of 16)
   const int n_acc = ((n_cells + 1) * acc_stride + kTrashPad + 1) & ~1;     // even: keeps the lists 16-byte aligned
   const int list_cap = p.strip_pix * Kp;                // hit records per group list
-  unsigned long long *acc = lds64;
-  f32x4 *hit_w = reinterpret_cast<f32x4 *>(lds64 + n_acc);                       // [ng_chunk][list_cap]
-  float *s_go = reinterpret_cast<float *>(hit_w + p.ng_chunk * list_cap);          // [strip_pix][ch_stride], 16-byte aligned
+  // FAST keeps the hit weights in front of the accumulators: they are the landing zone of corners above the tile
+  unsigned long long *acc = FAST ? lds64 + 2 * (size_t)p.ng_chunk * list_cap : lds64;
+  f32x4 *hit_w = reinterpret_cast<f32x4 *>(FAST ? lds64 : lds64 + n_acc);         // [ng_chunk][list_cap]
+  float *s_go = reinterpret_cast<float *>(FAST ? reinterpret_cast<f32x4 *>(acc + n_acc) : hit_w + p.ng_chunk * list_cap);   // [strip_pix][ch_stride], 16-byte aligned
   HitMeta *hit_meta = reinterpret_cast<HitMeta *>(s_go + p.strip_pix * ch_stride);  // [ng_chunk][list_cap]
   uint32_t *s_count = reinterpret_cast<uint32_t *>(hit_meta + p.ng_chunk * list_cap);  // two sets of [kMaxChunkGroups]
 
@@ -341,44 +346,89 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       int unit_of[kUnits];                                               // this row's visiting order
 #pragma unroll
       for (int u = 0; u < kUnits; ++u) unit_of[u] = (u + first_unit) & (kUnits - 1);
-      for (uint32_t i0 = wave * rows_per_group; i0 < n_max; i0 += kWaves * rows_per_group) {
-        const uint32_t i = i0 + my_slot;
-        if (i >= n_mine) continue;        // rows past the end of their group's list sit this pass out
-        const f32x4 w = hit_w[lane_group * list_cap + i];
-        const HitMeta meta = hit_meta[lane_group * list_cap + i];
-        const float *go_px = go_lane + (meta >> 16) * ch_stride;
-        const int first_cell = ((int)(meta & 63u) - 1) * p.tile_w + (int)((meta >> kMetaPosBits) & 63u) - 1;
-        uint32_t cells[4];
+      if constexpr (FAST) {
+        // one group of 16 channels, 32 cells per tile row: kCellWords accumulator words per cell
+        constexpr int kCellWords = PACK ? 8 : 16;
+        constexpr int kCorner[4] = {0, kCellWords, 32 * kCellWords, 33 * kCellWords};
+        unsigned long long *acc_row = acc + c * kUnits;
+        const float *go_row = s_go + c * CPL;
+        for (uint32_t i0 = wave * rows_per_group; i0 < n_max; i0 += kWaves * rows_per_group) {
+          const uint32_t i = i0 + my_slot;
+          if (i >= n_mine) continue;
+          const f32x4 w = hit_w[i];
+          const HitMeta meta = hit_meta[i];
+          const float *go_px = go_row + (meta >> 16) * 16;
+          const int first_cell = ((int)(meta & 63u) - 1) * 32 + (int)((meta >> kMetaPosBits) & 63u) - 1;
+          unsigned long long *base = acc_row + first_cell * kCellWords;
+          const float wv[4] = {w.x, w.y, w.z, w.w};
+          if constexpr (PACK) {
+            f32x2 g[kUnits];
 #pragma unroll
-        for (int cn = 0; cn < 4; ++cn)      // corners outside the tile carry weight 0: send them to the trash cell
-          cells[cn] = (meta & (1u << (2 * kMetaPosBits + cn))) ? (uint32_t)(first_cell + (cn >> 1) * p.tile_w + (cn & 1)) : (uint32_t)n_cells;
-        const float wv[4] = {w.x, w.y, w.z, w.w};
-        unsigned long long *dst[4];
+            for (int u = 0; u < kUnits; ++u) g[u] = *reinterpret_cast<const f32x2 *>(go_px + 2 * unit_of[u]);
 #pragma unroll
-        for (int cn = 0; cn < 4; ++cn) dst[cn] = acc_lane + __umul24(cells[cn], (uint32_t)acc_stride);
-        if constexpr (PACK) {
-          // two channels per atomic: sum = hi * 2^32 + lo with both halves signed, so the low term is
-          // sign-extended into the high word before the add
+            for (int u = 0; u < kUnits; ++u) {
+              const float g_lo = g[u].x, g_hi = g[u].y;
+              unsigned long long *dst = base + unit_of[u];
 #pragma unroll
-          for (int u = 0; u < kUnits; ++u) {
-            const int ch = 2 * unit_of[u];
-            const float g_lo = (c * CPL + ch < D) ? go_px[ch] : 0.f;
-            const float g_hi = (c * CPL + ch + 1 < D) ? go_px[ch + 1] : 0.f;
+              for (int cn = 0; cn < 4; ++cn)
+                __hip_atomic_fetch_add(dst + kCorner[cn], pack_fixed32(to_fixed32(g_lo, wv[cn]), to_fixed32(g_hi, wv[cn])),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+          } else {
+            const double wd[4] = {(double)wv[0], (double)wv[1], (double)wv[2], (double)wv[3]};
+            float g[kUnits];
 #pragma unroll
-            for (int cn = 0; cn < 4; ++cn) {
-              __hip_atomic_fetch_add(dst[cn] + unit_of[u], pack_fixed32(to_fixed32(g_lo, wv[cn]), to_fixed32(g_hi, wv[cn])),
-                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            for (int u = 0; u < kUnits; ++u) g[u] = go_px[unit_of[u]];
+#pragma unroll
+            for (int u = 0; u < kUnits; ++u) {
+              const double gd = (double)g[u];
+              unsigned long long *dst = base + unit_of[u];
+#pragma unroll
+              for (int cn = 0; cn < 4; ++cn)
+                __hip_atomic_fetch_add(dst + kCorner[cn], fixed_product(gd, wd[cn]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
           }
-        } else {
-          const double wd[4] = {(double)wv[0], (double)wv[1], (double)wv[2], (double)wv[3]};
-#pragma unroll
-          for (int u = 0; u < kUnits; ++u) {
-            const int ch = unit_of[u];
-            const double gd = (c * CPL + ch < D) ? (double)go_px[ch] : 0.0;
-#pragma unroll
-            for (int cn = 0; cn < 4; ++cn)
-              __hip_atomic_fetch_add(dst[cn] + ch, fixed_product(gd, wd[cn]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+      } else {
+        for (uint32_t i0 = wave * rows_per_group; i0 < n_max; i0 += kWaves * rows_per_group) {
+          const uint32_t i = i0 + my_slot;
+          if (i >= n_mine) continue;        // rows past the end of their group's list sit this pass out
+          const f32x4 w = hit_w[lane_group * list_cap + i];
+          const HitMeta meta = hit_meta[lane_group * list_cap + i];
+          const float *go_px = go_lane + (meta >> 16) * ch_stride;
+          const int first_cell = ((int)(meta & 63u) - 1) * p.tile_w + (int)((meta >> kMetaPosBits) & 63u) - 1;
+          uint32_t cells[4];
+  #pragma unroll
+          for (int cn = 0; cn < 4; ++cn)      // corners outside the tile carry weight 0: send them to the trash cell
+            cells[cn] = (meta & (1u << (2 * kMetaPosBits + cn))) ? (uint32_t)(first_cell + (cn >> 1) * p.tile_w + (cn & 1)) : (uint32_t)n_cells;
+          const float wv[4] = {w.x, w.y, w.z, w.w};
+          unsigned long long *dst[4];
+  #pragma unroll
+          for (int cn = 0; cn < 4; ++cn) dst[cn] = acc_lane + __umul24(cells[cn], (uint32_t)acc_stride);
+          if constexpr (PACK) {
+            // two channels per atomic: sum = hi * 2^32 + lo with both halves signed, so the low term is
+            // sign-extended into the high word before the add
+  #pragma unroll
+            for (int u = 0; u < kUnits; ++u) {
+              const int ch = 2 * unit_of[u];
+              const float g_lo = (c * CPL + ch < D) ? go_px[ch] : 0.f;
+              const float g_hi = (c * CPL + ch + 1 < D) ? go_px[ch + 1] : 0.f;
+  #pragma unroll
+              for (int cn = 0; cn < 4; ++cn) {
+                __hip_atomic_fetch_add(dst[cn] + unit_of[u], pack_fixed32(to_fixed32(g_lo, wv[cn]), to_fixed32(g_hi, wv[cn])),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+              }
+            }
+          } else {
+            const double wd[4] = {(double)wv[0], (double)wv[1], (double)wv[2], (double)wv[3]};
+  #pragma unroll
+            for (int u = 0; u < kUnits; ++u) {
+              const int ch = unit_of[u];
+              const double gd = (c * CPL + ch < D) ? (double)go_px[ch] : 0.0;
+  #pragma unroll
+              for (int cn = 0; cn < 4; ++cn)
+                __hip_atomic_fetch_add(dst[cn] + ch, fixed_product(gd, wd[cn]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
           }
         }
       }
@@ -465,19 +515,27 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
   };
   const int r = lanes_per_record(p.D), cpl = channels_per_lane(p.D);
   constexpr bool kCanPack = Tag::kBytes == 2;
+  // the immediate-offset variant: its stray zero adds reach 33 cells before and after the accumulators, which must
+  // stay inside the hit weights in front and the trash slots plus the parked grad_out behind
+  const size_t cell_bytes = (size_t)acc_words_per_cell(1, 16, p.pack32 != 0) * sizeof(unsigned long long);
+  const bool fast = p.tile_w_log2 == 5 && p.ng_chunk == 1 && p.D == 16 &&
+                    (size_t)p.strip_pix * p.Kp * sizeof(f32x4) >= 33 * cell_bytes &&
+                    cell_bytes + (size_t)p.strip_pix * 16 * sizeof(float) >= 33 * cell_bytes;
 #define GV_CASE(KPV)                                                                        \
   do {                                                                                      \
     if constexpr (kCanPack) {                                                               \
-      if (p.pack32 && r == 2 && cpl == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, true>);   \
-      if (p.pack32 && r == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, 8, true>);     \
-      if (p.pack32 && r == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, 8, true>);     \
+      if (p.pack32 && fast) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, true, true>);  \
+      if (p.pack32 && r == 2 && cpl == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, true, false>);   \
+      if (p.pack32 && r == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, 8, true, false>);     \
+      if (p.pack32 && r == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, 8, true, false>);     \
     }                                                                                       \
-    if (r == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, 8, false>);                  \
-    if (r == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, 8, false>);                  \
-    if (cpl == 1) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 1, false>);                \
-    if (cpl == 2) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 2, false>);                \
-    if (cpl == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 4, false>);                \
-    return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, false>);                              \
+    if (fast && !p.pack32) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, false, true>); \
+    if (r == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, 8, false, false>);                  \
+    if (r == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, 8, false, false>);                  \
+    if (cpl == 1) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 1, false, false>);                \
+    if (cpl == 2) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 2, false, false>);                \
+    if (cpl == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 4, false, false>);                \
+    return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, false, false>);                              \
   } while (0)
   if (k3 && !p.remove_center) GV_CASE(9);
   if (k3 && p.remove_center) GV_CASE(8);
