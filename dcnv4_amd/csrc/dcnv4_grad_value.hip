@@ -62,11 +62,12 @@ __host__ __device__ inline int acc_words_per_cell(int ng_chunk, int D, bool pack
   return ng_chunk * acc_words_per_group(D, pack);
 }
 
-// FAST: 32-pixel-wide tiles, one group of 16 channels per workgroup.  The four corners of a hit record then lie at
-// compile-time distances from the first one, so their addresses are immediates of one base register; a corner outside
+// FAST (0 = off, else log2 of the tile width): groups of 16 channels in 32-wide tiles with one group per workgroup, or
+// 16- and 8-wide tiles with four.  The four corners of a hit record then lie at compile-time distances from the
+// first one, so their addresses are immediates of one base register; a corner outside
 // the tile carries weight zero and its add lands, harmlessly, on whatever the LDS holds there - another cell, or the
 // hit weights in front of the accumulators or the parked grad_out behind them (adding the integer 0 changes nothing).
-template <typename Tag, int KP, int R, int CPL, bool PACK, bool FAST>
+template <typename Tag, int KP, int R, int CPL, bool PACK, int FAST>
 __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const DcnLaunch p) {
   extern __shared__ unsigned long long lds64[];
   const int Kp = p.Kp, D = p.D, C = p.G * p.D;
@@ -89,9 +90,9 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   const int n_acc = ((n_cells + 1) * acc_stride + kTrashPad + 1) & ~1;     // even: keeps the lists 16-byte aligned
   const int list_cap = p.strip_pix * Kp;                // hit records per group list
   // FAST keeps the hit weights in front of the accumulators: they are the landing zone of corners above the tile
-  unsigned long long *acc = FAST ? lds64 + 2 * (size_t)p.ng_chunk * list_cap : lds64;
-  f32x4 *hit_w = reinterpret_cast<f32x4 *>(FAST ? lds64 : lds64 + n_acc);         // [ng_chunk][list_cap]
-  float *s_go = reinterpret_cast<float *>(FAST ? reinterpret_cast<f32x4 *>(acc + n_acc) : hit_w + p.ng_chunk * list_cap);   // [strip_pix][ch_stride], 16-byte aligned
+  unsigned long long *acc = FAST != 0 ? lds64 + 2 * (size_t)p.ng_chunk * list_cap : lds64;
+  f32x4 *hit_w = reinterpret_cast<f32x4 *>(FAST != 0 ? lds64 : lds64 + n_acc);         // [ng_chunk][list_cap]
+  float *s_go = reinterpret_cast<float *>(FAST != 0 ? reinterpret_cast<f32x4 *>(acc + n_acc) : hit_w + p.ng_chunk * list_cap);   // [strip_pix][ch_stride], 16-byte aligned
   HitMeta *hit_meta = reinterpret_cast<HitMeta *>(s_go + p.strip_pix * ch_stride);  // [ng_chunk][list_cap]
   uint32_t *s_count = reinterpret_cast<uint32_t *>(hit_meta + p.ng_chunk * list_cap);  // two sets of [kMaxChunkGroups]
 
@@ -346,19 +347,22 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       int unit_of[kUnits];                                               // this row's visiting order
 #pragma unroll
       for (int u = 0; u < kUnits; ++u) unit_of[u] = (u + first_unit) & (kUnits - 1);
-      if constexpr (FAST) {
-        // one group of 16 channels, 32 cells per tile row: kCellWords accumulator words per cell
-        constexpr int kCellWords = PACK ? 8 : 16;
-        constexpr int kCorner[4] = {0, kCellWords, 32 * kCellWords, 33 * kCellWords};
-        unsigned long long *acc_row = acc + c * kUnits;
-        const float *go_row = s_go + c * CPL;
+      if constexpr (FAST != 0) {
+        static_assert(R == 2 && CPL == 8, "groups of 16 channels");
+        constexpr int kGroups = FAST == 5 ? 1 : 4, kTileW = 1 << FAST;            // groups per workgroup, cells per tile row
+        constexpr int kGroupWords = PACK ? 8 : 16, kCellWords = kGroups * kGroupWords;
+        constexpr int kCorner[4] = {0, kCellWords, kTileW * kCellWords, (kTileW + 1) * kCellWords};
+        unsigned long long *acc_row = acc + lane_group * kGroupWords + c * kUnits;
+        const float *go_row = s_go + lane_group * 16 + c * CPL;
+        const f32x4 *w_list = hit_w + lane_group * list_cap;
+        const HitMeta *meta_list = hit_meta + lane_group * list_cap;
         for (uint32_t i0 = wave * rows_per_group; i0 < n_max; i0 += kWaves * rows_per_group) {
           const uint32_t i = i0 + my_slot;
           if (i >= n_mine) continue;
-          const f32x4 w = hit_w[i];
-          const HitMeta meta = hit_meta[i];
-          const float *go_px = go_row + (meta >> 16) * 16;
-          const int first_cell = ((int)(meta & 63u) - 1) * 32 + (int)((meta >> kMetaPosBits) & 63u) - 1;
+          const f32x4 w = w_list[i];
+          const HitMeta meta = meta_list[i];
+          const float *go_px = go_row + (meta >> 16) * (kGroups * 16);
+          const int first_cell = ((int)(meta & 63u) - 1) * kTileW + (int)((meta >> kMetaPosBits) & 63u) - 1;
           unsigned long long *base = acc_row + first_cell * kCellWords;
           const float wv[4] = {w.x, w.y, w.z, w.w};
           if constexpr (PACK) {
@@ -515,27 +519,35 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
   };
   const int r = lanes_per_record(p.D), cpl = channels_per_lane(p.D);
   constexpr bool kCanPack = Tag::kBytes == 2;
-  // the immediate-offset variant: its stray zero adds reach 33 cells before and after the accumulators, which must
-  // stay inside the hit weights in front and the trash slots plus the parked grad_out behind
-  const size_t cell_bytes = (size_t)acc_words_per_cell(1, 16, p.pack32 != 0) * sizeof(unsigned long long);
-  const bool fast = p.tile_w_log2 == 5 && p.ng_chunk == 1 && p.D == 16 &&
-                    (size_t)p.strip_pix * p.Kp * sizeof(f32x4) >= 33 * cell_bytes &&
-                    cell_bytes + (size_t)p.strip_pix * 16 * sizeof(float) >= 33 * cell_bytes;
+  // the immediate-offset variants: their stray zero adds reach tile_w + 1 cells before and after the accumulators,
+  // which must stay inside the hit weights in front and the trash slots plus the parked grad_out behind
+  int fast = 0;
+  if (p.D == 16 && p.tile_w_log2 >= 3 && p.tile_w_log2 <= 5 && p.ng_chunk == (p.tile_w_log2 == 5 ? 1 : 4)) {
+    const size_t cell_bytes = (size_t)acc_words_per_cell(p.ng_chunk, 16, p.pack32 != 0) * sizeof(unsigned long long);
+    const size_t guard = (size_t)(p.tile_w + 1) * cell_bytes;
+    if ((size_t)p.ng_chunk * p.strip_pix * p.Kp * sizeof(f32x4) >= guard &&
+        cell_bytes + (size_t)p.strip_pix * p.ng_chunk * 16 * sizeof(float) >= guard)
+      fast = p.tile_w_log2;
+  }
 #define GV_CASE(KPV)                                                                        \
   do {                                                                                      \
     if constexpr (kCanPack) {                                                               \
-      if (p.pack32 && fast) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, true, true>);  \
-      if (p.pack32 && r == 2 && cpl == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, true, false>);   \
-      if (p.pack32 && r == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, 8, true, false>);     \
-      if (p.pack32 && r == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, 8, true, false>);     \
+      if (p.pack32 && fast == 5) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, true, 5>);  \
+      if (p.pack32 && fast == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, true, 4>);  \
+      if (p.pack32 && fast == 3) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, true, 3>);  \
+      if (p.pack32 && r == 2 && cpl == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, true, 0>);   \
+      if (p.pack32 && r == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, 8, true, 0>);     \
+      if (p.pack32 && r == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, 8, true, 0>);     \
     }                                                                                       \
-    if (fast && !p.pack32) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, false, true>); \
-    if (r == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, 8, false, false>);                  \
-    if (r == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, 8, false, false>);                  \
-    if (cpl == 1) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 1, false, false>);                \
-    if (cpl == 2) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 2, false, false>);                \
-    if (cpl == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 4, false, false>);                \
-    return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, false, false>);                              \
+    if (!p.pack32 && fast == 5) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, false, 5>); \
+    if (!p.pack32 && fast == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, false, 4>); \
+    if (!p.pack32 && fast == 3) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, false, 3>); \
+    if (r == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 4, 8, false, 0>);                  \
+    if (r == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, 8, false, 0>);                  \
+    if (cpl == 1) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 1, false, 0>);                \
+    if (cpl == 2) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 2, false, 0>);                \
+    if (cpl == 4) return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 4, false, 0>);                \
+    return go(dcnv4_grad_value_kernel<Tag, KPV, 2, 8, false, 0>);                              \
   } while (0)
   if (k3 && !p.remove_center) GV_CASE(9);
   if (k3 && p.remove_center) GV_CASE(8);
