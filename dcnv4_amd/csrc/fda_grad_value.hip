@@ -17,9 +17,10 @@
 //   * fda_grad_value_kernel: persistent workgroups walk (tile, image, head) items, smallest level
 //     first.  An item collects its tile's slices of all chunk lists into LDS and applies them in
 //     batches: one lane per point rebuilds the position from sampling_loc_attn and, with the stored
-//     probability, the four corner weights; grad_out rows of the batch are parked in LDS (both
-//     requested one batch ahead, so the loads fly while the previous batch is applied); then a
-//     row of 8 lanes per point adds the contributions to the tile's accumulators with 64-bit integer
+//     probability, the four corner weights, while the previous batch is being applied (two record
+//     buffers, one barrier per batch; all loads are requested one batch ahead); then a row of 8 lanes
+//     per point, each holding its own channels of the point's grad_out row in registers, adds the
+//     contributions to the tile's accumulators with 64-bit integer
 //     LDS atomics on fixed-point values (normalised by max |grad_out|; probability * bilinear weight
 //     <= 1), so the result does not depend on the order of arrival and is bit-reproducible;
 //   * the finished tile is written to grad_value with plain stores in the tensor dtype.
@@ -207,10 +208,9 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
   const int D = p.D, LK = p.L * p.K, QK = p.Q * p.K;
   unsigned long long *acc = lds64;                            // [(kTileCells + 1) * DP], last cell = trash
   constexpr int n_acc = (kTileCells + 1) * DP;
-  f32x4 *rec_w = reinterpret_cast<f32x4 *>(lds64 + n_acc);    // [kBatch]
-  u32x2 *rec_meta = reinterpret_cast<u32x2 *>(rec_w + kBatch);   // [kBatch] four 7-bit cells
-  float *s_go = reinterpret_cast<float *>(rec_meta + kBatch); // [kBatch][DP]
-  uint32_t *s_list = reinterpret_cast<uint32_t *>(s_go + kBatch * DP);   // [kListCap]
+  f32x4 *rec_w = reinterpret_cast<f32x4 *>(lds64 + n_acc);    // [2][kBatch]: one batch is applied while the next is prepared
+  uint32_t *rec_meta = reinterpret_cast<uint32_t *>(rec_w + 2 * kBatch);   // [2][kBatch] four 7-bit cells
+  uint32_t *s_list = rec_meta + 2 * kBatch;                   // [kListCap]
   uint32_t *s_tab = s_list + kListCap;                        // [kTabCap] (offset | count << 16) of the item's tile per chunk
   uint32_t *s_pre = s_tab + kTabCap;                          // [kTabCap + 1] exclusive prefix of the counts
   __shared__ LevelPlan s_plan[kMaxLevels];
@@ -259,19 +259,21 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
     // Everything a batch needs is requested through range-checked buffer loads of raw words: no branches
     // around the loads, so they all fly together, and nothing is converted before it is needed.
     typedef typename RawWord<2 * Tag::kBytes>::type xy_t;      // (x, y) of a point are adjacent
-    typedef typename RawWord<4 * Tag::kBytes>::type go4_t;     // 4 channels of grad_out
     const __amdgpu_buffer_rsrc_t sla_rs = make_rsrc(reinterpret_cast<const elem_t *>(p.sla) + sla_bg,
                                                     (uint32_t)((size_t)p.Q * p.G * 3 * LK * Tag::kBytes));
     const __amdgpu_buffer_rsrc_t go_rs = make_rsrc(reinterpret_cast<const elem_t *>(p.grad_out) + go_bg,
                                                    (uint32_t)((size_t)p.Q * p.G * D * Tag::kBytes));
     const __amdgpu_buffer_rsrc_t pr_rs = make_rsrc(probs, (uint32_t)QK * 4u);
-    constexpr int kParts = DP / 4;                           // 4-channel pieces of a grad_out row
-    constexpr int kGoLoads = kBatch * kParts / kApplyThreads;
-    constexpr int kGoPerLane = kGoLoads > 0 ? kGoLoads : 1;
+    // A row of 8 lanes owns a listed point; lane c of the row owns the CPL consecutive channels from c * CPL, loads
+    // them itself and keeps them in registers until the point is applied.
+    typedef typename RawWord<CPL * Tag::kBytes>::type goN_t;
+    constexpr int kRowsPerLane = kBatch * kRowLanes / kApplyThreads;      // rows a lane serves per batch: 2
+    constexpr int kRowStep = kApplyThreads / kRowLanes;
+    const int row_in_block = tid / kRowLanes, c = tid & (kRowLanes - 1);
     struct Ahead {
       xy_t xy;                         // lanes < batch size: their point
       uint32_t pr;
-      go4_t go[kGoPerLane];
+      goN_t go[kRowsPerLane];
     };
     auto fetch = [&](uint32_t b0, int nb) {
       Ahead a;
@@ -284,16 +286,17 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
         a.pr = buffer_load<4>(pr_rs, live ? pt * 4u : kDropOffset);
       }
 #pragma unroll
-      for (int u = 0; u < kGoPerLane; ++u) {
-        const int i = tid + u * kApplyThreads, h = i / kParts, part = i - h * kParts;
-        const bool live = h < nb && i < kBatch * kParts && 4 * part < D;
+      for (int u = 0; u < kRowsPerLane; ++u) {
+        const int h = row_in_block + u * kRowStep;
+        const bool live = h < nb && c * CPL < D;
         const uint32_t q = s_list[b0 + min(h, max(nb - 1, 0))] / (uint32_t)p.K;
-        a.go[u] = buffer_load<4 * Tag::kBytes>(go_rs, live ? (q * (uint32_t)(p.G * D) + 4u * part) * Tag::kBytes : kDropOffset);
+        a.go[u] = buffer_load<CPL * Tag::kBytes>(go_rs, live ? (q * (uint32_t)(p.G * D) + (uint32_t)(c * CPL)) * Tag::kBytes : kDropOffset);
       }
       return a;
     };
-    auto park = [&](const Ahead &a, int nb) {
-      if (tid < nb) {          // one lane per point: corner weights and accumulator cells
+    // one lane per point: corner weights and accumulator cells, into record buffer `buf`
+    auto park = [&](const Ahead &a, int nb, int buf) {
+      if (tid < nb) {
         float xy[2];
         Pack<Tag, 2>::decode(a.xy, xy);
         const float x = sub_rn(mul_rn(xy[0], (float)lp.W), 0.5f);       // flash_deform_im2col_cuda.cuh:188-189
@@ -310,44 +313,51 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
           cells[cn] = ok ? (uint32_t)(cy * tw + cx) : (uint32_t)n_cells;
           w[cn] = ok ? ps * tp.w[cn] : 0.f;
         }
-        rec_w[tid] = f32x4{w[0], w[1], w[2], w[3]};
-        rec_meta[tid] = u32x2{cells[0] | (cells[1] << kCellBitsF) | (cells[2] << (2 * kCellBitsF)) | (cells[3] << (3 * kCellBitsF)), 0u};
-      }
-#pragma unroll
-      for (int u = 0; u < kGoPerLane; ++u) {      // grad_out rows, normalised to [-1, 1] (zeros past the head width)
-        const int i = tid + u * kApplyThreads, h = i / kParts, part = i - h * kParts;
-        if (h < nb && i < kBatch * kParts) {
-          float g4[4];
-          Pack<Tag, 4>::decode(a.go[u], g4);
-          *reinterpret_cast<f32x4 *>(s_go + h * DP + 4 * part) =
-              f32x4{ldexpf(g4[0], -e_go), ldexpf(g4[1], -e_go), ldexpf(g4[2], -e_go), ldexpf(g4[3], -e_go)};
-        }
+        rec_w[buf * kBatch + tid] = f32x4{w[0], w[1], w[2], w[3]};
+        rec_meta[buf * kBatch + tid] = cells[0] | (cells[1] << kCellBitsF) | (cells[2] << (2 * kCellBitsF)) | (cells[3] << (3 * kCellBitsF));
       }
     };
+    // Accumulator word of (lane c, slot j) is c + 8 j: the lanes of a row touch consecutive words.  The LDS takes a
+    // wave's 64-bit atomics half a wave at a time, four rows of eight lanes: row r visits its slots starting from
+    // slot r mod CPL, so with four slots the four rows of one instruction fill the 64 banks exactly once whatever
+    // their cells are.  The lane's channel values are rotated to that order once per point.
+    const int rot = row_in_block & (CPL - 1);
+    int slot_off[CPL];
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) slot_off[j] = kRowLanes * ((j + rot) & (CPL - 1));
     // applies the first n entries of s_list; called by every lane, ends past a barrier
     auto apply_list = [&](uint32_t n) {
       if (n == 0) return;
-      Ahead ahead = fetch(0, (int)min((uint32_t)kBatch, n));
+      int nb = (int)min((uint32_t)kBatch, n);
+      Ahead cur = fetch(0, nb);
+      park(cur, nb, 0);
+      __syncthreads();
+      int buf = 0;
       for (uint32_t b0 = 0; b0 < n; b0 += kBatch) {
-        const int nb = (int)min((uint32_t)kBatch, n - b0);
-        park(ahead, nb);
-        __syncthreads();
-        if (b0 + kBatch < n) ahead = fetch(b0 + kBatch, (int)min((uint32_t)kBatch, n - b0 - kBatch));
-        // a row of 8 lanes per point; row r starts its channel blocks at (r mod CPL), so the rows of one
-        // instruction spread over the banks
-        const int row_in_block = tid / kRowLanes, c = tid & (kRowLanes - 1);
-        for (int h = row_in_block; h < nb; h += kApplyThreads / kRowLanes) {
-          const f32x4 w = rec_w[h];
-          const uint32_t meta = rec_meta[h].x;
+        const int nb_next = b0 + kBatch < n ? (int)min((uint32_t)kBatch, n - b0 - kBatch) : 0;
+        Ahead nxt = cur;
+        if (nb_next > 0) nxt = fetch(b0 + kBatch, nb_next);      // flies while this batch is applied
+#pragma unroll
+        for (int u = 0; u < kRowsPerLane; ++u) {
+          const int h = row_in_block + u * kRowStep;
+          if (h >= nb) break;
+          const f32x4 w = rec_w[buf * kBatch + h];
+          const uint32_t meta = rec_meta[buf * kBatch + h];
           const uint32_t cells[4] = {meta & 127u, (meta >> kCellBitsF) & 127u, (meta >> (2 * kCellBitsF)) & 127u,
                                      (meta >> (3 * kCellBitsF)) & 127u};
           const float wv[4] = {w.x, w.y, w.z, w.w};
-          float gn[CPL];
-          int ch_off[CPL];
+          float g[CPL], gn[CPL];
+          Pack<Tag, CPL>::decode(cur.go[u], g);
 #pragma unroll
-          for (int j = 0; j < CPL; ++j) {
-            ch_off[j] = kRowLanes * ((j + row_in_block) & (CPL - 1));
-            gn[j] = s_go[h * DP + c + ch_off[j]];
+          for (int j = 0; j < CPL; ++j) g[j] = ldexpf(g[j], -e_go);      // normalised to [-1, 1]
+          if constexpr (CPL == 4) {          // gn[j] = g[(j + rot) & 3]
+            const bool r1 = rot & 1, r2 = rot & 2;
+            const float a0 = r1 ? g[1] : g[0], a1 = r1 ? g[2] : g[1], a2 = r1 ? g[3] : g[2], a3 = r1 ? g[0] : g[3];
+            gn[0] = r2 ? a2 : a0; gn[1] = r2 ? a3 : a1; gn[2] = r2 ? a0 : a2; gn[3] = r2 ? a1 : a3;
+          } else if constexpr (CPL == 2) {
+            gn[0] = rot ? g[1] : g[0]; gn[1] = rot ? g[0] : g[1];
+          } else {
+            gn[0] = g[0];
           }
 #pragma unroll
           for (int cn = 0; cn < 4; ++cn) {
@@ -356,20 +366,24 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
               const double wd = (double)wv[cn];
 #pragma unroll
               for (int j = 0; j < CPL; ++j)
-                __hip_atomic_fetch_add(dst + ch_off[j], fixed_product((double)gn[j], wd), __ATOMIC_RELAXED,
+                __hip_atomic_fetch_add(dst + slot_off[j], fixed_product((double)gn[j], wd), __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_WORKGROUP);
             } else {
               // 16-bit tensors carry 8-11 significant bits: terms below 2^31 (fix_bits <= 30), truncated
 #pragma unroll
               for (int j = 0; j < CPL; ++j) {
                 const int t = (int)(gn[j] * wv[cn]);
-                __hip_atomic_fetch_add(dst + ch_off[j], ((unsigned long long)(uint32_t)(t >> 31) << 32) | (uint32_t)t,
+                __hip_atomic_fetch_add(dst + slot_off[j], ((unsigned long long)(uint32_t)(t >> 31) << 32) | (uint32_t)t,
                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
               }
             }
           }
         }
+        if (nb_next > 0) park(nxt, nb_next, buf ^ 1);
         __syncthreads();
+        cur = nxt;
+        nb = nb_next;
+        buf ^= 1;
       }
     };
 
@@ -423,7 +437,7 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
     for (int i = tid; i < n_cells * D; i += kApplyThreads) {
       const int cell = i / D, ch = i - cell * D;
       const int cy = cell / tw, cx = cell - cy * tw;
-      const unsigned long long a = acc[cell * DP + ch];
+      const unsigned long long a = acc[cell * DP + ch / CPL + kRowLanes * (ch % CPL)];
       const double v = ldexp((double)(int)(a >> 32) * 4294967296.0 + (double)(uint32_t)a, e_out);
       const float f[1] = {(float)v};
       gv[(((size_t)b * p.N + lp.start + (size_t)(ty0 + cy) * lp.W + tx0 + cx) * p.G + g) * D + ch] = Pack<Tag, 1>::encode(f);
@@ -469,8 +483,8 @@ hipError_t launch_t(const FdaLaunch &p, hipStream_t stream) {
 
 size_t fda_grad_value_lds_bytes(const FdaLaunch &p) {
   const size_t dp = (size_t)fda_padded_channels(p.D);
-  return ((size_t)kTileCells + 1) * dp * sizeof(unsigned long long) + kBatch * (sizeof(f32x4) + sizeof(u32x2)) +
-         kBatch * dp * sizeof(float) + ((size_t)kListCap + 2 * kTabCap + 4) * sizeof(uint32_t);
+  return ((size_t)kTileCells + 1) * dp * sizeof(unsigned long long) + 2 * kBatch * (sizeof(f32x4) + sizeof(uint32_t)) +
+         ((size_t)kListCap + 2 * kTabCap + 4) * sizeof(uint32_t);
 }
 
 hipError_t launch_fda_grad_value(int dtype, const FdaLaunch &p, hipStream_t stream) {
