@@ -38,6 +38,13 @@ constexpr int kTiledThreads = 512;      // lanes per workgroup at most: leaves e
 __device__ __forceinline__ float rcp(float d) { return __builtin_amdgcn_rcpf(d); }
 __device__ __forceinline__ int fdiv(int n, float inv) { return (int)(((float)n + 0.5f) * inv); }
 
+// a.lo * b.lo + a.hi * b.hi + c for two packed 16-bit elements per word, products and sum in fp32
+template <typename Tag>
+__device__ __forceinline__ float dot2_pair(uint32_t a, uint32_t b, float c) {
+  if constexpr (Tag::kCode == F16::kCode) return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+  else return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+}
+
 template <typename Tag>
 __device__ __forceinline__ float lds_elem(const typename RawWord<Tag::kBytes>::type *p, int i) {
   float f[1];
@@ -490,12 +497,28 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
 #pragma unroll
       for (int cn = 0; cn < 4; ++cn) {
         float acc = 0.f;
+        if constexpr (Tag::kBytes == 2) {
+          // 16-bit tensors: two channels per instruction straight from the raw words, products and sums in fp32;
+          // two running sums, so that consecutive instructions do not wait for each other
+          float acc1 = 0.f;
 #pragma unroll
-        for (int v = 0; v < NV; ++v) {
-          float f[EPV];
-          pack::decode(raw[cn][v], f);
+          for (int v = 0; v < NV; ++v) {
+            const u32x4 a = raw[cn][v], g = go_raw[v];
+            const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, gw[4] = {g.x, g.y, g.z, g.w};
+            acc = dot2_pair<Tag>(aw[0], gw[0], acc);
+            acc1 = dot2_pair<Tag>(aw[1], gw[1], acc1);
+            acc = dot2_pair<Tag>(aw[2], gw[2], acc);
+            acc1 = dot2_pair<Tag>(aw[3], gw[3], acc1);
+          }
+          acc += acc1;
+        } else {
 #pragma unroll
-          for (int c = 0; c < EPV; ++c) acc = fmaf(f[c], go[v][c], acc);
+          for (int v = 0; v < NV; ++v) {
+            float f[EPV];
+            pack::decode(raw[cn][v], f);
+#pragma unroll
+            for (int c = 0; c < EPV; ++c) acc = fmaf(f[c], go[v][c], acc);
+          }
         }
         d[cn] = pair ? acc + dpp_quad_xor1(acc) : acc;
       }
