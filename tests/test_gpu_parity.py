@@ -37,6 +37,14 @@ DCN_CASES = {
     "d64": (1, 8, 9, 2, 64, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
     "far_offsets_mostly_outside": (1, 5, 5, 4, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 9.0),
     "single_pixel": (1, 1, 1, 1, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 1.0),
+    # 32-wide grad_value tiles, one group per workgroup: a one-pixel remainder tile in both directions
+    "edge_33x33_g2": (1, 33, 33, 2, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 3.0),
+    # ... a tile two rows high, whose corners above and below land outside the accumulators
+    "wide_short_2x40_g3": (2, 2, 40, 3, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 3.0),
+    # ... and a tall image only 8 pixels wide (narrow tiles keep the general accumulation)
+    "tall_narrow_40x8_g2": (1, 40, 8, 2, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 3.0),
+    # 16-wide tiles with four groups per workgroup and a last chunk of one group
+    "g5_16x12": (2, 16, 12, 5, 16, (3, 3, 1, 1, 1, 1, 1, 1), 1, 1.0, 3.0),
 }
 
 
