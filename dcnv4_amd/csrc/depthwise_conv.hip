@@ -192,10 +192,19 @@ __global__ void __launch_bounds__(kDwThreads) dwconv_grad_weight_kernel(const Dw
       raw_t win[KW][KH];
 #pragma unroll
       for (int j = 0; j < KW - 1; ++j) column(x_begin + j - p.pw, win[j]);
+      // the next pixel's input column and grad_out vector are requested before this pixel's sums
+      raw_t col_next[KH], go_next;
+      column(x_begin + KW - 1 - p.pw, col_next);
+      go_next = buffer_load<kVecBytes>(go_rs, go_row + (uint32_t)x_begin * pix_bytes);
       for (int x = x_begin; x < x_end; ++x) {
-        column(x + KW - 1 - p.pw, win[KW - 1]);
+#pragma unroll
+        for (int i = 0; i < KH; ++i) win[KW - 1][i] = col_next[i];
         float g[V];
-        load_vec<Tag, V>(go_rs, go_row + (uint32_t)x * pix_bytes, g);
+        Pack<Tag, V>::decode(go_next, g);
+        if (x + 1 < x_end) {
+          column(x + KW - p.pw, col_next);
+          go_next = buffer_load<kVecBytes>(go_rs, go_row + (uint32_t)(x + 1) * pix_bytes);
+        }
 #pragma unroll
         for (int j = 0; j < KW; ++j)
 #pragma unroll
@@ -300,10 +309,9 @@ hipError_t grad_weight_v(const DwLaunch &p, hipStream_t stream) {
 template <typename Tag>
 hipError_t grad_weight_t(const DwLaunch &p, hipStream_t stream) {
   constexpr int kFull = 16 / Tag::kBytes;
-  switch (depthwise_grad_weight_vector(Tag::kBytes, p.C, p.kh)) {
-    case kFull: return grad_weight_v<Tag, kFull>(p, stream);
-    case 2: return grad_weight_v<Tag, 2>(p, stream);
-  }
+  const int v = depthwise_grad_weight_vector(Tag::kBytes, p.C, p.kh);
+  if (v == kFull) return grad_weight_v<Tag, kFull>(p, stream);
+  if (v == 2) return grad_weight_v<Tag, 2>(p, stream);
   return grad_weight_v<Tag, 1>(p, stream);
 }
 
@@ -317,9 +325,12 @@ hipError_t reduce_t(const DwLaunch &p, hipStream_t stream) {
 
 }  // namespace
 
-// narrow vectors keep the register footprint of (taps + 1) * V sums in bounds for the larger kernels
+// Narrow vectors keep the register footprint of (taps + 1) * V sums in bounds: the kernel waits on its loads every
+// pixel, so waves per SIMD count for more than bytes per load.  16-bit tensors: two channels per lane (measured
+// 128x56x56x112 fp16: 103 us with 8 channels per lane, 68 us with 2); fp32: no difference between 4, 2 and 1.
 int depthwise_grad_weight_vector(int elem_bytes, int C, int k) {
   const int full = 16 / elem_bytes;
+  if (k <= 3 && elem_bytes == 2 && C % 2 == 0) return 2;
   if (k <= 3 && C % full == 0) return full;
   return C % 2 == 0 ? 2 : 1;
 }
