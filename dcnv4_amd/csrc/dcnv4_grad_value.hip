@@ -70,6 +70,12 @@ __host__ __device__ inline int acc_words_per_cell(int ng_chunk, int D, bool pack
 template <typename Tag, int KP, int R, int CPL, bool PACK, int FAST>
 __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const DcnLaunch p) {
   extern __shared__ unsigned long long lds64[];
+  // Packed sums, one group per workgroup: a cell is 64 bytes, half of what the LDS takes in one pass of eight
+  // records (16 lanes x 8 bytes over 32 banks), so two records on the same unit collide when their cells' columns
+  // have the same parity.  The hit list is therefore kept in two parts - even first columns from the front, odd
+  // ones from the back - and the rows of a wave draw from them alternately: every pass then holds four records of
+  // each parity on four different units, for all four corners (the other corners shift every record alike).
+  constexpr bool kTwoEnded = PACK && FAST == 5;
   const int Kp = p.Kp, D = p.D, C = p.G * p.D;
   const int n_chunks = (p.G + p.ng_chunk - 1) / p.ng_chunk;
   const int nty = (p.H + p.tile_h - 1) >> p.tile_h_log2, ntx = (p.W + p.tile_w - 1) >> p.tile_w_log2;
@@ -298,6 +304,24 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
             meta = (uint32_t)(ly + 1) | ((uint32_t)(lx + 1) << kMetaPosBits) | (valid << (2 * kMetaPosBits)) | ((uint32_t)it.px << 16);
           }
         }
+        if constexpr (kTwoEnded) {
+          // records whose first cell has an even column grow the list from its front, the others from its back
+          const bool odd = (meta >> kMetaPosBits) & 1u ? false : true;      // the field holds column + 1
+          const uint64_t mask_e = __builtin_amdgcn_ballot_w64(hit && !odd), mask_o = __builtin_amdgcn_ballot_w64(hit && odd);
+          if ((mask_e | mask_o) != 0) {
+            uint32_t base = 0;
+            if (lane < 2) base = atomicAdd(&count[lane], (uint32_t)__builtin_popcountll(lane == 0 ? mask_e : mask_o));
+            const uint32_t base_e = (uint32_t)__builtin_amdgcn_readlane((int)base, 0), base_o = (uint32_t)__builtin_amdgcn_readlane((int)base, 1);
+            if (hit) {
+              const uint64_t mine = odd ? mask_o : mask_e;
+              const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(mine >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mine, 0u));
+              const uint32_t slot = odd ? (uint32_t)list_cap - 1u - (base_o + rank) : base_e + rank;
+              hit_w[slot] = w;
+              hit_meta[slot] = meta;
+            }
+          }
+          continue;
+        }
       // append the wave's hits to its group's list: one LDS counter bump per wave
         const uint64_t mask = __builtin_amdgcn_ballot_w64(hit);
         if (mask != 0) {
@@ -356,9 +380,19 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
         const float *go_row = s_go + lane_group * 16 + c * CPL;
         const f32x4 *w_list = hit_w + lane_group * list_cap;
         const HitMeta *meta_list = hit_meta + lane_group * list_cap;
-        for (uint32_t i0 = wave * rows_per_group; i0 < n_max; i0 += kWaves * rows_per_group) {
-          const uint32_t i = i0 + my_slot;
-          if (i >= n_mine) continue;
+        // two-ended list: rows 2j and 2j + 1 of a wave take the j-th even and the j-th odd record of the pass
+        const uint32_t n_two = kTwoEnded ? ((my_slot & 1) ? count[1] : count[0]) : 0u;
+        const uint32_t bound = kTwoEnded ? max(count[0], count[1]) : n_max;
+        const uint32_t lane_step = kTwoEnded ? (uint32_t)(my_slot >> 1) : (uint32_t)my_slot;
+        const uint32_t wave_rows = kTwoEnded ? (uint32_t)(kWave / R / 2) : (uint32_t)rows_per_group;
+        if constexpr (kTwoEnded) {
+#pragma unroll
+          for (int u = 0; u < kUnits; ++u) unit_of[u] = (u + (my_slot >> 1)) & (kUnits - 1);
+        }
+        for (uint32_t i0 = wave * wave_rows; i0 < bound; i0 += kWaves * wave_rows) {
+          uint32_t i = i0 + lane_step;
+          if (i >= (kTwoEnded ? n_two : n_mine)) continue;
+          if (kTwoEnded && (my_slot & 1)) i = (uint32_t)list_cap - 1u - i;
           const f32x4 w = w_list[i];
           const HitMeta meta = meta_list[i];
           const float *go_px = go_row + (meta >> 16) * (kGroups * 16);
