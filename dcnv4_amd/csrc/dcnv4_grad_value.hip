@@ -19,8 +19,8 @@
 //          lanes per record keep the per-record work (reading and unpacking it) small next to the
 //          adds.  The 64 / R rows of a wave are dealt evenly to the groups of the chunk, and the n-th
 //          row of a group starts its walk over the lane's channels at the n-th, so the rows of one
-//          ds_add_u64 instruction spread evenly over the banks: two bank sweeps, the least 64 lanes of
-//          8 bytes can take;
+//          ds_add_u64 instruction spread evenly over the banks (32 banks of 4 bytes; a 64-bit operation is
+//          served 16 lanes per pass): four passes, the least 64 lanes of 8 bytes can take;
 //   * fixed point: contributions are normalised by the global maxima of |grad_out| and
 //     |modulation| (GradState, produced by the grad_offset_mask kernel that runs first) and carry
 //     `fix_bits` fractional bits (up to 50; each product is exact in double precision and rounded
@@ -353,9 +353,10 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
       int my_group = row_in_wave / rows_per_group, my_slot = row_in_wave - my_group * rows_per_group;
       int first_unit = my_slot;
       if (PACK && R == 2 && p.ng_chunk == 4 && group_words == 8) {
-        // A cell of packed sums is 32 words, one bank sweep, and the LDS takes a wave's 64-bit atomics half a wave
-        // at a time: deal the 16 rows of each half-wave as 4 groups x 4 starting units, so that a half-wave touches
-        // 32 distinct words (groups in consecutive rows would put two rows of a half-wave on every word).
+        // A cell of packed sums is 32 words, 8 per group, and the LDS serves a wave's 64-bit atomics 16 lanes (8 rows)
+        // per pass over 16 word slots: deal each run of 8 rows as 2 groups x 4 starting units (16 rows: 4 groups), so
+        // that the rows of a pass touch different slots whatever their cells are (groups in consecutive rows would
+        // put rows of groups g and g + 2 on the same slots).
         const int half = row_in_wave >> 4, i = row_in_wave & 15;
         my_group = i >> 2;
         first_unit = i & 3;

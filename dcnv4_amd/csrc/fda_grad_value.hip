@@ -317,10 +317,11 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
         rec_meta[buf * kBatch + tid] = cells[0] | (cells[1] << kCellBitsF) | (cells[2] << (2 * kCellBitsF)) | (cells[3] << (3 * kCellBitsF));
       }
     };
-    // Accumulator word of (lane c, slot j) is c + 8 j: the lanes of a row touch consecutive words.  The LDS takes a
-    // wave's 64-bit atomics half a wave at a time, four rows of eight lanes: row r visits its slots starting from
-    // slot r mod CPL, so with four slots the four rows of one instruction fill the 64 banks exactly once whatever
-    // their cells are.  The lane's channel values are rotated to that order once per point.
+    // Accumulator word of (lane c, slot j) is c + 8 j: the lanes of a row touch consecutive words.  The LDS serves a
+    // wave's 64-bit atomics 16 lanes per pass over its 32 banks, two rows of eight lanes: row r visits its slots
+    // starting from slot r mod CPL, so neighbouring rows are on slots of different parity and the two rows of a pass
+    // fill the banks exactly once whatever their cells are.  The lane's channel values are rotated to that order
+    // once per point.
     const int rot = row_in_block & (CPL - 1);
     int slot_off[CPL];
 #pragma unroll
