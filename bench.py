@@ -70,6 +70,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--offset-range", type=float, default=None,
+                    help="with --only-op dcnv4_*: offsets uniform in +-this many pixels instead of the benchmark's +-3 (+-4 for the dense shapes)")
     ap.add_argument("--op-iters", type=int, default=100, help="timed launches per operator in the detail table")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-detail", action="store_true", help="skip per-operator timings other than the step's own")
@@ -192,7 +194,7 @@ def main():
             for name, B, H, W, C, G in table:
                 if name != shape_name:
                     continue
-                t = dcn_inputs(B, H, W, C, G, dtype, off)
+                t = dcn_inputs(B, H, W, C, G, dtype, off if args.offset_range is None else args.offset_range)
                 fn = (lambda: dcn_fwd(t, G, C)) if op == "dcnv4_fwd" else (lambda: dcn_bwd(t, G, C))
                 ms = time_op(fn, args.steps, warm=args.warmup)
                 nbytes = dcn_bytes(t[0].element_size(), B, H, W, C, G)[0 if op == "dcnv4_fwd" else 1]
