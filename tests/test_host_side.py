@@ -229,3 +229,43 @@ def test_tuner_candidates_are_valid_hints_and_start_with_the_library_choice():
         bwd = tune.candidates(G, D, es, "bwd")
         assert bwd[0] == ("library", {}, 0, 0) and {"scatter": "atomic"} in [c[1] for c in bwd]
     assert set(tune.SHAPES) == {"t", "b", "dense"} and all(len(v) == 4 for v in tune.SHAPES.values())
+
+
+def test_module_initial_values_follow_the_reference_recipe():
+    """Xavier-uniform projections with zero biases, zero offset / modulation / attention projections, and the
+    attention offsets' bias on a square ring (DCNv4_op/DCNv4/modules/dcnv4.py:95-103, flash_deform_attn.py:64-82)."""
+    import math
+    from dcnv4_amd import DCNv4, FlashDeformAttn
+    torch.manual_seed(0)
+    dcn = DCNv4(channels=128, group=8)
+    att = FlashDeformAttn(d_model=128, n_levels=3, n_heads=8, n_points=4)
+    for proj in (dcn.value_proj, dcn.output_proj, att.value_proj, att.output_proj):
+        bound = math.sqrt(6.0 / (proj.in_features + proj.out_features))
+        w = proj.weight.detach()
+        assert w.abs().max() <= bound and w.abs().max() > 0.95 * bound          # uniform on [-bound, bound]
+        assert abs(float(w.std()) - bound / math.sqrt(3.0)) < 0.03 * bound
+        assert proj.bias.abs().sum() == 0
+    for lin in (dcn.offset_mask, att.attention_weights):
+        assert lin.weight.abs().sum() == 0 and lin.bias.abs().sum() == 0
+    assert att.sampling_offsets.weight.abs().sum() == 0
+    bias = att.sampling_offsets.bias.detach().view(8, 3, 4, 2)
+    for h in range(8):
+        theta = 2 * math.pi * h / 8
+        d = torch.tensor([math.cos(theta), math.sin(theta)])
+        d = d / d.abs().max()
+        for k in range(4):
+            assert torch.allclose(bias[h, :, k], (d * (k + 1)).expand(3, 2), atol=1e-6)
+
+
+def test_center_feature_blend_matches_the_reference_expression():
+    """out = y (1 - s) + x s with s = sigmoid(W y + b) repeated over each group's channels
+    (DCNv4_op/DCNv4/modules/dcnv4.py:142-147), on the CPU-capable part of the module."""
+    from dcnv4_amd.functions import center_feature_func
+    g = torch.Generator().manual_seed(1)
+    y, x = torch.randn(2, 3, 4, 32, generator=g), torch.randn(2, 3, 4, 32, generator=g)
+    w, b = torch.randn(2, 32, generator=g), torch.randn(2, generator=g)
+    s = torch.sigmoid(torch.nn.functional.linear(y, w, b))
+    s = s[..., None].repeat(1, 1, 1, 1, 16).flatten(-2)
+    want = y * (1 - s) + x * s
+    got = center_feature_func.blend_reference(y, x, w, b)
+    assert torch.allclose(got, want, atol=1e-6)
