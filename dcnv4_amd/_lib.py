@@ -10,7 +10,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libdcnv4_gfx950.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 OK, ERR_INVALID_ARGUMENT, ERR_RUNTIME = 0, 1, 2
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 
@@ -21,6 +21,7 @@ SIGNATURES = {
     "dcnv4_gfx950_abi_version": (_i, []),
     "dcnv4_gfx950_last_error": (ctypes.c_char_p, []),
     "dcnv4_gfx950_set_launch_option": (_i, [ctypes.c_char_p, _i]),
+    "dcnv4_gfx950_get_launch_option": (_i, [ctypes.c_char_p, ctypes.POINTER(_i)]),
     "dcnv4_gfx950_forward": (_i, [_vp, _vp, _vp, _i] + [_i] * 13 + [_f] + [_i] * 6 + [_vp]),
     "dcnv4_gfx950_backward_workspace_bytes": (_sz, [_i] * 6),
     "dcnv4_gfx950_backward": (_i, [_vp] * 6 + [_sz, _i] + [_i] * 13 + [_f] + [_i] * 6 + [_vp]),

@@ -119,31 +119,23 @@ __global__ void init_state_kernel(GradState *st) {
 }
 
 constexpr size_t kStateBytes = 256;     // GradState, padded
-constexpr int kTiledMaxGroupChannels = 64;
+constexpr int kMaxBackwardGroupChannels = 512;    // widest group of the backward: 64 lanes of 16 bytes in the gather, 16 lanes of 32 channels per slot
 
-// Per-thread launch options (dcnv4_gfx950_set_launch_option); 0 = not set: the environment variable of the
-// same purpose decides, then the library's default.
+// Per-thread launch options (dcnv4_gfx950_set_launch_option).  They choose between kernels that compute the same
+// result; nothing else in the library reads the environment or any other hidden state.
 enum { kOptAuto = 0, kOptTiled = 1, kOptPlain = 2 };
-thread_local int g_opt_gather = kOptAuto;       // LDS-tiled / direct gathers (forward, grad_offset_mask)
-thread_local int g_opt_scatter = kOptAuto;      // tiled LDS accumulation / global atomics (grad_value)
-thread_local int g_opt_reach = 0;               // 0 = not set, else reach + 1
+struct LaunchOptions {
+  int gather = kOptAuto;       // LDS-tiled / direct gathers (DCNv4 forward, grad_offset_mask)
+  int scatter = kOptAuto;      // attention grad_value: binned LDS accumulation / global atomics
+  int reach = -1;              // input pixels around a reference point that the tiled gathers stage; -1: default
+  int tile = 0;                // largest side of a grad_value tile (8, 16, 32); 0: default
+  int fda_order = kOptAuto;    // attention forward: 1 whole query rows per workgroup, 2 one head per workgroup
+};
+thread_local LaunchOptions g_opt;
 
-bool tiled_grad_value(int D) { return D <= kTiledMaxGroupChannels && g_opt_scatter != kOptPlain; }
+constexpr int kDefaultReach = 5;
 
-// Tuning override, read on every call: DCNV4_GFX950_REACH = distance (input pixels) from an output
-// pixel's reference point that the tiled kernels cover; sampling points beyond it take the
-// global-memory paths.  Default 5.
-// Tuning override, read on every call: DCNV4_GFX950_TILE=16 keeps the tiled grad_value kernel on 16x16 tiles.
-bool large_tiles_enabled() {
-  const char *e = getenv("DCNV4_GFX950_TILE");
-  return !(e && strcmp(e, "16") == 0);
-}
-
-int reach_setting() {
-  const char *e = getenv("DCNV4_GFX950_REACH");
-  const int r = g_opt_reach > 0 ? g_opt_reach - 1 : (e ? atoi(e) : 5);
-  return r < 0 ? 0 : (r > 64 ? 64 : r);
-}
+int reach_setting() { return g_opt.reach < 0 ? kDefaultReach : std::min(g_opt.reach, 64); }
 
 // Flash attention backward: head widths the tiled grad_value kernel handles (8 lanes x up to 4 channels,
 // whole 8-channel blocks), with point counts that fit its 32-bit point ids.
@@ -153,77 +145,42 @@ bool fda_tiled_shape(int D, int L, int Q, int K) {
 
 constexpr size_t kL2BytesPerXcd = 4u << 20;
 
-// Tuning override, read on every call: DCNV4_GFX950_FDA_ORDER=rows keeps the attention forward on whole rows
-// (all heads of a query in one workgroup) whatever the sizes.
-bool fda_head_major_enabled() {
-  const char *e = getenv("DCNV4_GFX950_FDA_ORDER");
-  return !(e && strcmp(e, "rows") == 0);
-}
+bool fda_tiled_enabled() { return g_opt.scatter != kOptPlain; }
 
-// Tuning override, read on every call: DCNV4_GFX950_FDA_SCATTER=atomic keeps the fp32 atomic scatter.
-bool fda_tiled_enabled() {
-  if (g_opt_scatter != kOptAuto) return g_opt_scatter == kOptTiled;
-  const char *e = getenv("DCNV4_GFX950_FDA_SCATTER");
-  return !(e && strcmp(e, "atomic") == 0);
-}
-
-// Tile, channel chunk and strip of the tiled grad_value kernel such that its LDS footprint fits.
-int plan_grad_value_tiles(DcnLaunch *L, int elem_bytes_of_launch) {
+// Tile, group chunk, lanes per slot and strip of the tiled grad_value kernel such that a workgroup of 1024 lanes has
+// at most one (cell, group, channel part) per lane and its LDS footprint fits.
+int plan_grad_value_tiles(DcnLaunch *L, int dtype) {
   const int D = L->D;
-  L->reach = reach_setting();
-  L->ng_chunk = std::max(1, std::min(L->G, kTiledMaxGroupChannels / std::max(D, 16)));   // <= 4
-  // 16-bit tensors: two 32-bit fixed-point sums per accumulator word when that leaves at least 18
-  // fractional bits.  A cell collects at most one corner per tap from the (2*reach+1)^2 output pixels
-  // around it, each of magnitude <= 2^fix_bits, and the sum must stay below 2^31.
-  const long long per_cell = (long long)(2 * L->reach + 1) * (2 * L->reach + 1) * L->Kp;
-  const int fix32 = 31 - ceil_log2((int)std::min<long long>(per_cell, 1 << 30));
-  L->pack32 = (elem_bytes_of_launch == 2 && D > 8 && fix32 >= 18) ? 1 : 0;
-  // Power-of-two tiles (the reach rule uses shifts); shrink until the LDS footprint fits.  Images wider or taller
-  // than 16 pixels first try 32x32 tiles with ONE group per workgroup: the accumulators take the same LDS as four
-  // groups of a 16x16 tile, the workgroup count is the same, but a tile visits (32 + 2 reach)^2 / 32^2 = 1.7 output
-  // pixels per input pixel instead of 2.6 (1.0 when the tile covers the whole image), and every sampling point
-  // belongs to exactly one group, so nothing is evaluated twice.
-  auto visited = [&](int tile, int stride) { return (tile + 2 * L->reach + stride - 1) / stride + 1; };
-  auto plan = [&](int max_log2, int groups) {
-    L->ng_chunk = groups;
-    L->tile_h_log2 = L->tile_w_log2 = max_log2;
-    while (L->tile_h_log2 > 0 && (1 << (L->tile_h_log2 - 1)) >= L->H) --L->tile_h_log2;
-    while (L->tile_w_log2 > 0 && (1 << (L->tile_w_log2 - 1)) >= L->W) --L->tile_w_log2;
-    for (;;) {
-      L->tile_h = 1 << L->tile_h_log2;
-      L->tile_w = 1 << L->tile_w_log2;
-      const int row = visited(L->tile_w, L->sw);
-      for (int rows = 8; rows >= 1; --rows) {                // up to 8 visited rows per strip: every strip costs two barriers
-        L->strip_pix = std::min(rows * row, 1023);           // pixel index field of a hit record
-        if (dcnv4_grad_value_lds_bytes(*L) <= kMaxLdsPerWorkgroup - 256) return true;
-      }
-      if (max_log2 > 4) return false;                        // the large-tile plan is all or nothing
-      if (L->tile_h_log2 > 0 && L->tile_h_log2 >= L->tile_w_log2) --L->tile_h_log2;
-      else if (L->tile_w_log2 > 0) --L->tile_w_log2;
-      else return false;
+  L->gv_cw = D <= 8 ? 8 : (D <= 16 ? 16 : 32);
+  L->gv_lps_log2 = 0;
+  while ((L->gv_cw << L->gv_lps_log2) < D) ++L->gv_lps_log2;
+  const int max_slots = 1024 >> L->gv_lps_log2;
+  const int cap_log2 = g_opt.tile == 8 ? 3 : (g_opt.tile == 16 ? 4 : 5);
+  L->tile_h_log2 = L->tile_w_log2 = cap_log2;
+  while (L->tile_h_log2 > 0 && (1 << (L->tile_h_log2 - 1)) >= L->H) --L->tile_h_log2;
+  while (L->tile_w_log2 > 0 && (1 << (L->tile_w_log2 - 1)) >= L->W) --L->tile_w_log2;
+  while ((1 << (L->tile_h_log2 + L->tile_w_log2)) > max_slots) {
+    if (L->tile_h_log2 >= L->tile_w_log2) --L->tile_h_log2; else --L->tile_w_log2;
+  }
+  L->tile_h = 1 << L->tile_h_log2;
+  L->tile_w = 1 << L->tile_w_log2;
+  const int cells = L->tile_h * L->tile_w;
+  const int max_items = dcnv4_grad_value_rounds(L->gv_cw) * 1024;
+  const int park_bytes = dtype == DCNV4_DTYPE_F16 ? 2 : 4;
+  for (int ng = std::min({L->G, max_slots / cells, 63, max_items / L->Kp}); ng >= 1; --ng) {
+    L->ng_chunk = ng;
+    int units = (ng * (L->gv_cw << L->gv_lps_log2) * park_bytes + 15) / 16;
+    units |= 1;                                     // an odd number of 16-byte units spreads the rows over the LDS banks
+    L->gv_go_stride = units * 16;
+    for (int s = std::min(1023, max_items / (L->Kp * ng)); s >= 1; s = s > 64 ? s - 16 : s - 1) {
+      L->strip_pix = s;
+      if (dcnv4_grad_value_lds_bytes(*L) <= kMaxLdsPerWorkgroup - 512) return DCNV4_OK;
     }
-  };
-  const int groups16 = L->ng_chunk;
-  const bool large = (L->H > 16 || L->W > 16) && large_tiles_enabled() && plan(5, 1);
-  if (!large && !plan(4, groups16))
-    return fail(DCNV4_ERR_RUNTIME, "kernel with %d taps and %d group channels does not fit the tiled backward", L->Kp, D);
-  const long long contributions = (long long)visited(L->tile_h, L->sh) * visited(L->tile_w, L->sw) * L->Kp;
-  // a term must stay below 2^51 (the conversion's range), a sum below 2^62
-  L->fix_bits = std::min(50, 62 - ceil_log2((int)std::min<long long>(contributions, 1 << 30)));
-  if (L->pack32) L->fix_bits = std::min(fix32, 22);                         // the rounding trick of the packed path needs |term| < 2^22
-  // the tiled kernel addresses one image's offset_mask and grad_out with 32-bit element offsets
-  if (L->Q >= (1 << 24) || (uint64_t)L->Q * (uint64_t)L->P_pad >= (1ull << 31) || (uint64_t)L->Q * (uint64_t)(L->G * L->D) >= (1ull << 31))
-    return fail(DCNV4_ERR_RUNTIME, "one image of %d output pixels is too large for the tiled backward", L->Q);
-  return DCNV4_OK;
+  }
+  return fail(DCNV4_ERR_RUNTIME, "kernel with %d taps and %d group channels does not fit the tiled backward", L->Kp, D);
 }
 
-// Tuning override, read on every call: DCNV4_GFX950_GATHER=direct keeps the gathers on the
-// global-memory kernels.
-bool tiled_gather_enabled() {
-  if (g_opt_gather != kOptAuto) return g_opt_gather == kOptTiled;
-  const char *e = getenv("DCNV4_GFX950_GATHER");
-  return !(e && strcmp(e, "direct") == 0);
-}
+bool tiled_gather_enabled() { return g_opt.gather != kOptPlain; }
 
 // Output tile, group chunk and input window of the LDS-tiled gather kernels.  Returns false (and
 // leaves gt_h = 0) when the shape does not suit them: group width not a power-of-two number of
@@ -315,11 +272,11 @@ int dcn_prepare(DcnProblem *pr, bool backward, int dtype, int batch, int H, int 
 
   DcnLaunch &L = pr->launch;
   L = DcnLaunch{};
-  if (int rc = choose_lanes(D, s, d_stride, backward, &L.lanes)) return rc;
+  if (int rc = choose_lanes(D, s, d_stride, false, &L.lanes)) return rc;
   const int width = 1 << L.lanes.tpgp_log2;
-  if (backward && width > kWave)
-    return fail(DCNV4_ERR_INVALID_ARGUMENT, "backward needs group_channels/%d <= 64 lanes per group, got %d",
-                L.lanes.cpt, L.lanes.tpg);
+  if (backward && (width > kWave || D > kMaxBackwardGroupChannels))
+    return fail(DCNV4_ERR_INVALID_ARGUMENT, "backward takes groups of up to %d channels in at most 64 lanes of 16 bytes, got %d channels",
+                kMaxBackwardGroupChannels, D);
   L.Q = Ho * Wo; L.Wo = Wo; L.H = H; L.W = W; L.G = G; L.D = D;
   L.kh = kh; L.kw = kw; L.sh = sh; L.sw = sw; L.ph = ph; L.pw = pw; L.dh = dh; L.dw = dw;
   L.Kp = Kp; L.P_pad = P_pad; L.remove_center = remove_center; L.softmax = softmax ? 1 : 0;
@@ -398,7 +355,8 @@ void fda_choose_order(FdaLaunch *F, const FdaProblem &pr, int N, int G, int D, i
   const size_t lines_per_pixel = (std::max(head_bytes, line) + line - 1) / line;      // cache lines a head touches per pixel
   const size_t head_footprint = (size_t)N * lines_per_pixel * line;
   F->head_major = 0;
-  if (!fda_head_major_enabled() || G <= 1 || pr.img_elems * pr.s <= kL2BytesPerXcd / 2 || head_footprint > kL2BytesPerXcd) return;
+  if (g_opt.fda_order == 1 || G <= 1) return;
+  if (g_opt.fda_order != 2 && (pr.img_elems * pr.s <= kL2BytesPerXcd / 2 || head_footprint > kL2BytesPerXcd)) return;
   F->head_major = 1;
   const int width = 1 << F->lanes.tpgp_log2;
   const size_t lds_per_row = (size_t)3 * L * K * sizeof(float) * (backward ? 2 : 1);
@@ -496,13 +454,32 @@ int dcnv4_gfx950_abi_version(void) { return DCNV4_GFX950_ABI_VERSION; }
 
 const char *dcnv4_gfx950_last_error(void) { return g_error; }
 
+static int *launch_option_slot(const char *name) {
+  if (name == nullptr) return nullptr;
+  if (std::strcmp(name, "gather") == 0) return &g_opt.gather;
+  if (std::strcmp(name, "scatter") == 0) return &g_opt.scatter;
+  if (std::strcmp(name, "reach") == 0) return &g_opt.reach;
+  if (std::strcmp(name, "tile") == 0) return &g_opt.tile;
+  if (std::strcmp(name, "fda_order") == 0) return &g_opt.fda_order;
+  return nullptr;
+}
+
 int dcnv4_gfx950_set_launch_option(const char *name, int value) {
-  if (name == nullptr) return fail(DCNV4_ERR_INVALID_ARGUMENT, "null option name");
+  int *slot = launch_option_slot(name);
+  if (slot == nullptr) return fail(DCNV4_ERR_INVALID_ARGUMENT, "unknown launch option %s", name ? name : "(null)");
   const bool family = value == kOptAuto || value == kOptTiled || value == kOptPlain;
-  if (std::strcmp(name, "gather") == 0 && family) g_opt_gather = value;
-  else if (std::strcmp(name, "scatter") == 0 && family) g_opt_scatter = value;
-  else if (std::strcmp(name, "reach") == 0 && value >= -1 && value <= 64) g_opt_reach = value + 1;
-  else return fail(DCNV4_ERR_INVALID_ARGUMENT, "unknown launch option %s = %d", name, value);
+  const bool ok = slot == &g_opt.reach ? (value >= -1 && value <= 64)
+                  : slot == &g_opt.tile ? (value == 0 || value == 8 || value == 16 || value == 32)
+                                        : family;
+  if (!ok) return fail(DCNV4_ERR_INVALID_ARGUMENT, "launch option %s does not take the value %d", name, value);
+  *slot = value;
+  return DCNV4_OK;
+}
+
+int dcnv4_gfx950_get_launch_option(const char *name, int *value) {
+  const int *slot = launch_option_slot(name);
+  if (slot == nullptr || value == nullptr) return fail(DCNV4_ERR_INVALID_ARGUMENT, "unknown launch option %s", name ? name : "(null)");
+  *value = *slot;
   return DCNV4_OK;
 }
 
@@ -538,17 +515,15 @@ size_t dcnv4_gfx950_backward_workspace_bytes(int dtype, int batch, int height_in
                                              int group_channels) {
   if (elem_bytes(dtype) == 0 || batch <= 0 || height_in <= 0 || width_in <= 0 || group <= 0 || group_channels <= 0)
     return 0;
-  if (tiled_grad_value(group_channels)) return kStateBytes;
-  if (elem_bytes(dtype) != 2) return 0;
-  return round16((size_t)batch * height_in * width_in * group * group_channels * sizeof(float));
+  return kStateBytes;      // a function of nothing: in particular not of the launch options
 }
 
-int dcnv4_gfx950_backward(const void *value, const void *offset_mask, const void *grad_output, void *grad_value,
-                          void *grad_offset_mask, void *workspace, size_t workspace_bytes, int dtype, int batch,
-                          int height_in, int width_in, int group, int group_channels, int kernel_h, int kernel_w,
-                          int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w,
-                          float offset_scale, int im2col_step, int remove_center, int padded_offset_dim,
-                          int softmax, int d_stride, int block_thread, void *stream) {
+static int dcn_backward_impl(const void *value, const void *offset_mask, const void *grad_output, void *grad_value,
+                             void *grad_offset_mask, void *workspace, size_t workspace_bytes, int dtype, int batch,
+                             int height_in, int width_in, int group, int group_channels, int kernel_h, int kernel_w,
+                             int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w,
+                             float offset_scale, int im2col_step, int remove_center, int padded_offset_dim,
+                             int softmax, int d_stride, int block_thread, void *stream) {
   DcnProblem pr;
   if (int rc = dcn_prepare(&pr, true, dtype, batch, height_in, width_in, group, group_channels, kernel_h,
                            kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, offset_scale,
@@ -561,67 +536,51 @@ int dcnv4_gfx950_backward(const void *value, const void *offset_mask, const void
       return fail(DCNV4_ERR_RUNTIME, "workspace of %zu bytes needed, got %zu at %p", need, workspace_bytes, workspace);
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const size_t total = (size_t)batch * pr.img_elems;
 
-  if (tiled_grad_value(group_channels)) {
-    // 1. grad_offset_mask + statistics  2. tiled grad_value (plain stores)  3. fallback scatter
-    //    for corners beyond the reach / non-finite statistics (returns at once otherwise)
-    DcnLaunch base = pr.launch;
-    if (int rc = plan_grad_value_tiles(&base, pr.s)) return rc;
-    const bool gather_tiled = plan_gather_tiles(&base, pr.s);
-    base.state = static_cast<GradState *>(workspace);
-    hipLaunchKernelGGL(init_state_kernel, dim3(1), dim3(64), 0, st, base.state);
-    if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);
-    const int per = images_per_launch(pr, false);
-    for (int pass = 0; pass < 3; ++pass) {
-      for (int b0 = 0; b0 < batch; b0 += per) {
-        const int nb = std::min(per, batch - b0);
-        DcnLaunch L = base;
-        L.value = at(value, b0 * pr.img_elems, pr.s);
-        L.offset_mask = at(offset_mask, b0 * pr.img_om_elems, pr.s);
-        L.grad_out = at(grad_output, b0 * pr.img_out_elems, pr.s);
-        L.grad_value = at(grad_value, b0 * pr.img_elems, pr.s);
-        L.grad_offset_mask = at(grad_offset_mask, b0 * pr.img_om_elems, pr.s);
-        L.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
-        L.n_pix = nb * L.Q;
-        L.n_img = nb;
-        hipError_t e = hipSuccess;
-        if (pass == 0 && gather_tiled) {
-          e = launch_dcnv4_offset_mask_grad_tiled(dtype, L, st);
-        } else if (pass == 0) {
-          // gathers want 16-byte lanes; the lane map chosen for scatter is only used by pass 2
-          if (int rc = choose_lanes(group_channels, pr.s, 0, false, &L.lanes)) return rc;
-          if (int rc = choose_block_pixels(&L, 0, true)) return rc;
-          e = launch_dcnv4_backward(dtype, L, kBwdOffsetMask, st);
-        } else if (pass == 1) {
-          e = launch_dcnv4_grad_value(dtype, L, st);
-        } else {
-          e = launch_dcnv4_backward(dtype, L, kBwdFallback, st);
-        }
-        if (e) return hip_fail("dcnv4 backward launch", e);
-      }
+  // state reset, then 1. grad_offset_mask + the reach the sampling points need  2. tiled grad_value (plain stores)
+  DcnLaunch base = pr.launch;
+  if (int rc = plan_grad_value_tiles(&base, dtype)) return rc;
+  // the grad_value kernel addresses one image's offset_mask and grad_out with 32-bit element offsets
+  if (base.Q >= (1 << 24) || (uint64_t)base.Q * (uint64_t)base.P_pad >= (1ull << 31) ||
+      (uint64_t)base.Q * (uint64_t)(base.G * base.D) >= (1ull << 31))
+    return fail(DCNV4_ERR_RUNTIME, "one image of %d output pixels is too large for the backward", base.Q);
+  const bool gather_tiled = plan_gather_tiles(&base, pr.s);
+  base.state = static_cast<GradState *>(workspace);
+  hipLaunchKernelGGL(init_state_kernel, dim3(1), dim3(64), 0, st, base.state);
+  if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);
+  const int per = images_per_launch(pr, false);
+  for (int pass = 0; pass < 2; ++pass) {
+    for (int b0 = 0; b0 < batch; b0 += per) {
+      const int nb = std::min(per, batch - b0);
+      DcnLaunch L = base;
+      L.value = at(value, b0 * pr.img_elems, pr.s);
+      L.offset_mask = at(offset_mask, b0 * pr.img_om_elems, pr.s);
+      L.grad_out = at(grad_output, b0 * pr.img_out_elems, pr.s);
+      L.grad_value = at(grad_value, b0 * pr.img_elems, pr.s);
+      L.grad_offset_mask = at(grad_offset_mask, b0 * pr.img_om_elems, pr.s);
+      L.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
+      L.n_pix = nb * L.Q;
+      L.n_img = nb;
+      hipError_t e = hipSuccess;
+      if (pass == 0 && gather_tiled) e = launch_dcnv4_offset_mask_grad_tiled(dtype, L, st);
+      else if (pass == 0) e = launch_dcnv4_offset_mask_grad(dtype, L, st);
+      else e = launch_dcnv4_grad_value(dtype, L, st);
+      if (e) return hip_fail("dcnv4 backward launch", e);
     }
-    return DCNV4_OK;
   }
-
-  float *acc = need > 0 ? static_cast<float *>(workspace) : static_cast<float *>(grad_value);
-  if (hipError_t e = clear_async(acc, total, st)) return hip_fail("clear launch", e);
-  const int per = images_per_launch(pr, true);
-  for (int b0 = 0; b0 < batch; b0 += per) {
-    const int nb = std::min(per, batch - b0);
-    DcnLaunch L = pr.launch;
-    L.value = at(value, b0 * pr.img_elems, pr.s);
-    L.offset_mask = at(offset_mask, b0 * pr.img_om_elems, pr.s);
-    L.grad_out = at(grad_output, b0 * pr.img_out_elems, pr.s);
-    L.grad_value_acc = acc + b0 * pr.img_elems;
-    L.grad_offset_mask = at(grad_offset_mask, b0 * pr.img_om_elems, pr.s);
-    L.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
-    L.n_pix = nb * L.Q;
-    if (hipError_t e = launch_dcnv4_backward(dtype, L, kBwdFull, st)) return hip_fail("dcnv4 backward launch", e);
-  }
-  if (need > 0)
-    if (hipError_t e = narrow_async(dtype, acc, grad_value, total, st)) return hip_fail("cast launch", e);
   return DCNV4_OK;
+}
+
+int dcnv4_gfx950_backward(const void *value, const void *offset_mask, const void *grad_output, void *grad_value,
+                          void *grad_offset_mask, void *workspace, size_t workspace_bytes, int dtype, int batch,
+                          int height_in, int width_in, int group, int group_channels, int kernel_h, int kernel_w,
+                          int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w,
+                          float offset_scale, int im2col_step, int remove_center, int padded_offset_dim,
+                          int softmax, int d_stride, int block_thread, void *stream) {
+  return dcn_backward_impl(value, offset_mask, grad_output, grad_value, grad_offset_mask, workspace, workspace_bytes, dtype,
+                           batch, height_in, width_in, group, group_channels, kernel_h, kernel_w, stride_h, stride_w, pad_h,
+                           pad_w, dilation_h, dilation_w, offset_scale, im2col_step, remove_center, padded_offset_dim,
+                           softmax, d_stride, block_thread, stream);
 }
 
 int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_shapes,

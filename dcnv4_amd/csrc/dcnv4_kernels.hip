@@ -113,45 +113,24 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_forward_kernel(const DcnL
 }
 
 // ------------------------------------------------------------------------------- backward
-// One kernel body, three roles (BackwardMode):
-//   kBwdFull        grad_offset_mask, and grad_value scattered with fp32 buffer atomics into a
-//                   cleared fp32 image (any group width; the generic path)
-//   kBwdOffsetMask  grad_offset_mask only, plus the statistics the tiled grad_value kernel needs
-//                   (max |grad_out|, max |modulation|, the reach the scatter needs)
-//   kBwdFallback    no gradients of offsets; scatters into grad_value, in its own dtype, the
-//                   corners the tiled kernel does not cover: the far ones, or all of them when the
-//                   statistics are not finite.  Exits at once when there is nothing to do.
-template <typename Tag, int CPT, int KP, int MODE>
-__global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const DcnLaunch p) {
+// grad_offset_mask for any group width (the part of dcnv4_col2im_cuda.cuh:280-350 and common.h:188-211 that does not
+// scatter), plus the reach the grad_value kernel has to cover.
+template <typename Tag, int CPT, int KP>
+__global__ void __launch_bounds__(kBlockThreads) dcnv4_offset_mask_grad_kernel(const DcnLaunch p) {
   extern __shared__ float lds[];
   typedef Pack<Tag, CPT> pack;
-  bool scatter_all = false;
-  if constexpr (MODE == kBwdFallback) {
-    const uint32_t gmax = p.state->go_max_bits, mmax = p.state->mask_max_bits;
-    scatter_all = gmax >= 0x7f800000u || mmax >= 0x7f800000u;
-    if (!scatter_all && p.state->reach_needed <= (uint32_t)p.reach) return;
-  }
-  // The fallback role is launched with a small grid (its usual job is to find out that there is nothing
-  // to do) and strides over the pixel blocks; the other roles own exactly one block.
-  const uint32_t n_blocks = (uint32_t)((p.n_pix + p.npix_block - 1) / p.npix_block);
-  uint32_t block_index = blockIdx.x;
-  int pix0 = 0, npix = 0;
   const bool vec16 = (p.P_pad * Tag::kBytes) % 16 == 0;
   float *s_om = lds, *s_grad = lds + p.npix_block * p.P_pad;
-  uint32_t go_max = 0, mask_max = 0, reach_needed = 0;
-  for (;;) {
-  const uint32_t blk = MODE == kBwdFallback ? block_index : xcd_contiguous_block(block_index, gridDim.x);
-  pix0 = (int)blk * p.npix_block;
-  npix = min(p.npix_block, p.n_pix - pix0);
+  uint32_t reach_needed = 0;
+  const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
+  const int pix0 = (int)blk * p.npix_block;
+  const int npix = min(p.npix_block, p.n_pix - pix0);
   stage_rows_to_lds<Tag>(s_om, (const char *)p.offset_mask + (size_t)pix0 * p.P_pad * Tag::kBytes,
                          npix * p.P_pad, vec16);
-  if constexpr (MODE != kBwdFallback)
-    for (int i = threadIdx.x; i < npix * p.P_pad; i += blockDim.x) s_grad[i] = 0.f;
+  for (int i = threadIdx.x; i < npix * p.P_pad; i += blockDim.x) s_grad[i] = 0.f;
   __syncthreads();
 
   const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
-  // fp32 accumulation image of value: same element offsets, 4-byte elements
-  const __amdgpu_buffer_rsrc_t gacc = make_rsrc(p.grad_value_acc, p.value_bytes / Tag::kBytes * 4);
   const int tpgp_log2 = p.lanes.tpgp_log2, width = 1 << tpgp_log2;
   const int items = (npix * p.G) << tpgp_log2;
   const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
@@ -169,16 +148,9 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
     float *gom = s_grad + lp * p.P_pad + g * 3 * Kp;
     float mx = 0.f, inv = 1.f;
     if (p.softmax) softmax_stats(om + 2 * Kp, Kp, mx, inv);
-    // reference point of this output pixel (centre tap at zero offset) and the box the tiled scatter covers
-    NearBox box = {0, 0, 0, 0};
-    int p0y = 0, p0x = 0;
-    if constexpr (MODE != kBwdFull) {
-      const int q = pix % p.Q;
-      p0y = half_h - p.ph + (q / p.Wo) * p.sh;
-      p0x = half_w - p.pw + (q % p.Wo) * p.sw;
-      box = near_box(p0y, p0x, p.tile_h_log2, p.tile_w_log2, p.reach);
-    }
-    const size_t img_elem0 = (size_t)(pix / p.Q) * (size_t)(p.H * p.W) * (size_t)(p.G * p.D);
+    // reference point of this output pixel (centre tap at zero offset)
+    const int q = pix % p.Q;
+    const int p0y = half_h - p.ph + (q / p.Wo) * p.sh, p0x = half_w - p.pw + (q % p.Wo) * p.sw;
 
     float go[CPT];
     {
@@ -188,10 +160,6 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
       if (!active) {
 #pragma unroll
         for (int c = 0; c < CPT; ++c) go[c] = 0.f;
-      }
-      if constexpr (MODE == kBwdOffsetMask) {
-#pragma unroll
-        for (int c = 0; c < CPT; ++c) go_max = max(go_max, __builtin_bit_cast(uint32_t, fabsf(go[c])));
       }
     }
     float dot_pg = 0.f;     // sum_k p_k * gz_k, softmax Jacobian only
@@ -207,21 +175,7 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
 #pragma unroll
         for (int cn = 0; cn < 4; ++cn) t.off[cn] = kDropOffset;
       }
-      if constexpr (MODE == kBwdFallback) {
-#pragma unroll
-        for (int cn = 0; cn < 4; ++cn) {
-          if (!(t.valid & (1u << cn))) continue;
-          const int cy = t.y0 + (cn >> 1), cx = t.x0 + (cn & 1);
-          if (!scatter_all && corner_is_near(box, cy, cx)) continue;
-          const float w = m * t.w[cn];
-          const size_t e0 = img_elem0 + (size_t)(cy * p.W + cx) * (p.G * p.D) + g * p.D + chunk * CPT;
-#pragma unroll
-          for (int c = 0; c < CPT; ++c) atomic_add_element<Tag>(p.grad_value, e0 + c, go[c] * w);
-        }
-        return;
-      }
-      if constexpr (MODE == kBwdOffsetMask) {
-        mask_max = max(mask_max, __builtin_bit_cast(uint32_t, fabsf(m)));
+      {
         if (t.valid != 0) {     // distance of the in-image part of the 2x2 corner block from the reference point;
           // a far row or column whose bilinear weight is exactly zero (integer coordinate) adds nothing and is left out
           const int y1 = t.y0 + (t.ly > 0.f ? 1 : 0), x1 = t.x0 + (t.lx > 0.f ? 1 : 0);
@@ -242,14 +196,6 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
 #pragma unroll
         for (int c = 0; c < CPT; ++c) d = fmaf(v[c], go[c], d);
         dots[cn] = d;
-        if constexpr (MODE == kBwdFull) {
-          // scatter: grad_value[corner] += grad_out * m * w   (common.h:153,164,174,184)
-          const float w = m * t.w[cn];
-          const uint32_t aoff = (t.off[cn] == kDropOffset) ? kDropOffset : t.off[cn] * (4 / Tag::kBytes);
-#pragma unroll
-          for (int c = 0; c < CPT; ++c)
-            __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(go[c] * w, gacc, aoff + 4 * c, 0, 0);
-        }
       }
       const float hy = 1.f - t.ly, hx = 1.f - t.lx;
       float gx = hy * (dots[1] - dots[0]) + t.ly * (dots[3] - dots[2]);   // common.h:188-201
@@ -282,38 +228,25 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_backward_kernel(const Dcn
           ++k;
         }
     }
-    if constexpr (MODE != kBwdFallback) {
-      if (p.softmax && chunk == 0) {      // p_k (g_k - sum_j p_j g_j), dcnv4_col2im_cuda.cuh:352-365
-        for (int k = 0; k < Kp; ++k) {
-          const float pk = __expf(om[2 * Kp + k] - mx) * inv;
-          gom[2 * Kp + k] = pk * (gom[2 * Kp + k] - dot_pg);
-        }
+    if (p.softmax && chunk == 0) {      // p_k (g_k - sum_j p_j g_j), dcnv4_col2im_cuda.cuh:352-365
+      for (int k = 0; k < Kp; ++k) {
+        const float pk = __expf(om[2 * Kp + k] - mx) * inv;
+        gom[2 * Kp + k] = pk * (gom[2 * Kp + k] - dot_pg);
       }
     }
   }
-  if constexpr (MODE != kBwdFallback) break;
-  block_index += gridDim.x;
-  if (block_index >= n_blocks) return;
-  __syncthreads();        // the staged rows are replaced next
-  }
-  if constexpr (MODE == kBwdOffsetMask) {
-    // Same-address atomics retire slowly at the memory side: fold the workgroup's statistics in
-    // LDS first and only touch the global word when it would actually grow.
-    __shared__ uint32_t s_stat[3];
-    if (threadIdx.x < 3) s_stat[threadIdx.x] = 0u;
+  {
+    // Same-address atomics retire slowly at the memory side: fold the workgroup's value in LDS first and only
+    // touch the global word when it would actually grow.
+    __shared__ uint32_t s_reach;
+    if (threadIdx.x == 0) s_reach = 0u;
     __syncthreads();
-    go_max = wave_max_u32(go_max);
-    mask_max = wave_max_u32(mask_max);
     reach_needed = wave_max_u32(reach_needed);
-    if ((threadIdx.x & (kWave - 1)) == 0) {
-      atomicMax(&s_stat[0], go_max);
-      atomicMax(&s_stat[1], mask_max);
-      atomicMax(&s_stat[2], reach_needed);
-    }
+    if ((threadIdx.x & (kWave - 1)) == 0 && reach_needed != 0) atomicMax(&s_reach, reach_needed);
     __syncthreads();
-    if (threadIdx.x < 3) {
-      uint32_t *dst = &p.state->go_max_bits + threadIdx.x;
-      const uint32_t mine = s_stat[threadIdx.x];
+    if (threadIdx.x == 0) {
+      uint32_t *dst = &p.state->reach_needed;
+      const uint32_t mine = s_reach;
       if (mine > __hip_atomic_load(dst, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(dst, mine);
     }
   }
@@ -331,25 +264,24 @@ hipError_t launch_fwd_k(const DcnLaunch &p, hipStream_t stream, dim3 grid, dim3 
   return hipGetLastError();
 }
 
-template <typename Tag, int CPT, int MODE>
+template <typename Tag, int CPT>
 hipError_t launch_bwd_k(const DcnLaunch &p, hipStream_t stream, dim3 grid, dim3 block, size_t lds) {
   const bool k3 = p.kh == 3 && p.kw == 3;
-  if (k3 && !p.remove_center) hipLaunchKernelGGL((dcnv4_backward_kernel<Tag, CPT, 9, MODE>), grid, block, lds, stream, p);
-  else if (k3 && p.remove_center) hipLaunchKernelGGL((dcnv4_backward_kernel<Tag, CPT, 8, MODE>), grid, block, lds, stream, p);
-  else hipLaunchKernelGGL((dcnv4_backward_kernel<Tag, CPT, 0, MODE>), grid, block, lds, stream, p);
+  if (k3 && !p.remove_center) hipLaunchKernelGGL((dcnv4_offset_mask_grad_kernel<Tag, CPT, 9>), grid, block, lds, stream, p);
+  else if (k3 && p.remove_center) hipLaunchKernelGGL((dcnv4_offset_mask_grad_kernel<Tag, CPT, 8>), grid, block, lds, stream, p);
+  else hipLaunchKernelGGL((dcnv4_offset_mask_grad_kernel<Tag, CPT, 0>), grid, block, lds, stream, p);
   return hipGetLastError();
 }
 
-// MODE < 0 selects the forward kernel.
-template <typename Tag, int MODE>
+template <typename Tag, bool BWD>
 hipError_t launch_by_cpt(const DcnLaunch &p, hipStream_t stream) {
   const unsigned n_blocks = (unsigned)((p.n_pix + p.npix_block - 1) / p.npix_block);
-  const dim3 grid(MODE == kBwdFallback ? std::min(n_blocks, 1024u) : n_blocks), block(kBlockThreads);
-  const size_t lds = MODE >= 0 ? dcnv4_backward_lds_bytes(p) : dcnv4_forward_lds_bytes(p);
+  const dim3 grid(n_blocks), block(kBlockThreads);
+  const size_t lds = BWD ? dcnv4_backward_lds_bytes(p) : dcnv4_forward_lds_bytes(p);
 #define DCN_CASE(N)                                                              \
   case N:                                                                        \
     if constexpr (N * Tag::kBytes <= 16) {                                       \
-      if constexpr (MODE >= 0) return launch_bwd_k<Tag, N, MODE>(p, stream, grid, block, lds); \
+      if constexpr (BWD) return launch_bwd_k<Tag, N>(p, stream, grid, block, lds); \
       else return launch_fwd_k<Tag, N>(p, stream, grid, block, lds);             \
     }                                                                            \
     break;
@@ -360,11 +292,11 @@ hipError_t launch_by_cpt(const DcnLaunch &p, hipStream_t stream) {
   return hipErrorInvalidValue;
 }
 
-template <int MODE> hipError_t launch_by_dtype(int dtype, const DcnLaunch &p, hipStream_t stream) {
+template <bool BWD> hipError_t launch_by_dtype(int dtype, const DcnLaunch &p, hipStream_t stream) {
   switch (dtype) {
-    case F32::kCode: return launch_by_cpt<F32, MODE>(p, stream);
-    case F16::kCode: return launch_by_cpt<F16, MODE>(p, stream);
-    case BF16::kCode: return launch_by_cpt<BF16, MODE>(p, stream);
+    case F32::kCode: return launch_by_cpt<F32, BWD>(p, stream);
+    case F16::kCode: return launch_by_cpt<F16, BWD>(p, stream);
+    case BF16::kCode: return launch_by_cpt<BF16, BWD>(p, stream);
   }
   return hipErrorInvalidValue;
 }
@@ -375,15 +307,10 @@ size_t dcnv4_forward_lds_bytes(const DcnLaunch &p) { return (size_t)p.npix_block
 size_t dcnv4_backward_lds_bytes(const DcnLaunch &p) { return 2 * dcnv4_forward_lds_bytes(p); }
 
 hipError_t launch_dcnv4_forward(int dtype, const DcnLaunch &p, hipStream_t stream) {
-  return launch_by_dtype<-1>(dtype, p, stream);
+  return launch_by_dtype<false>(dtype, p, stream);
 }
-hipError_t launch_dcnv4_backward(int dtype, const DcnLaunch &p, int mode, hipStream_t stream) {
-  switch (mode) {
-    case kBwdFull: return launch_by_dtype<kBwdFull>(dtype, p, stream);
-    case kBwdOffsetMask: return launch_by_dtype<kBwdOffsetMask>(dtype, p, stream);
-    case kBwdFallback: return launch_by_dtype<kBwdFallback>(dtype, p, stream);
-  }
-  return hipErrorInvalidValue;
+hipError_t launch_dcnv4_offset_mask_grad(int dtype, const DcnLaunch &p, hipStream_t stream) {
+  return launch_by_dtype<true>(dtype, p, stream);
 }
 
 }  // namespace dcn

@@ -408,7 +408,7 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_forward_tiled_kernel(cons
 // so nothing is reduced across lanes.  The gradients replace the lane's own offset_mask slice in
 // LDS (each slot is read before it is overwritten) and the slices go back to memory as rows;
 // the workgroup that owns the last groups also clears the padding tail of its rows.  The kernel
-// also folds the statistics the tiled grad_value kernel needs into GradState.
+// also folds the reach the grad_value kernel has to cover into GradState.
 template <typename Tag, int NV, int KP>
 __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_kernel(const DcnLaunch p) {
   extern __shared__ u32x4 lds128[];
@@ -420,8 +420,8 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
   const int cell_stride = p.gt_ng * p.D * Tag::kBytes + GT_PAD;
   char *s_win = reinterpret_cast<char *>(lds128);
   elem_t *s_om = reinterpret_cast<elem_t *>(s_win + (size_t)(p.gt_wh * p.gt_ww + p.gt_ww + 2) * cell_stride);
-  __shared__ uint32_t s_stat[3];
-  if (threadIdx.x < 3) s_stat[threadIdx.x] = 0u;
+  __shared__ uint32_t s_reach;
+  if (threadIdx.x == 0) s_reach = 0u;
 
   // lane -> (tile pixel, group of the chunk); its grad_out vector is requested before the staging
   const int part = threadIdx.x & (p.gt_lpg - 1), unit = threadIdx.x >> (p.gt_lpg - 1);
@@ -440,15 +440,11 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
   stage_tile<Tag, NV>(p, t, s_win, s_om, cell_stride);
   __syncthreads();
 
-  uint32_t go_max = 0, mask_max = 0, reach_needed = 0;
+  uint32_t reach_needed = 0;
   if (active) {
     float go[NV][EPV];
 #pragma unroll
-    for (int v = 0; v < NV; ++v) {
-      pack::decode(go_raw[v], go[v]);
-#pragma unroll
-      for (int c = 0; c < EPV; ++c) go_max = max(go_max, __builtin_bit_cast(uint32_t, fabsf(go[v][c])));
-    }
+    for (int v = 0; v < NV; ++v) pack::decode(go_raw[v], go[v]);
     const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
     const int p0y = half_h - p.ph + ho * p.sh, p0x = half_w - p.pw + wo * p.sw;      // reference point
     const float x_base = sub_rn((float)p0x, mul_rn((float)half_w, p.offset_scale));
@@ -477,7 +473,6 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
       const float x = add_rn(x_base, mul_rn(add_rn((float)(i * p.dw), lds_elem<Tag>(om, 2 * k)), p.offset_scale));
       const float y = add_rn(y_base, mul_rn(add_rn((float)(j * p.dh), lds_elem<Tag>(om, 2 * k + 1)), p.offset_scale));
       const float m = lds_elem<Tag>(om, 2 * Kp + k);
-      mask_max = max(mask_max, __builtin_bit_cast(uint32_t, fabsf(m)));
       const WinTap wt = window_tap(y, x, p.H, p.W, t, cell_stride, lane_bytes, zero_base);
       far_mask |= (mask_t)(wt.inside && !wt.ok) << k;
       if (wt.inside) {      // distance of the weighted, in-image part of the 2x2 corner block from the reference point
@@ -582,20 +577,14 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
     }
   }
 
-  // statistics: fold in LDS, then touch the global words only when they would grow (same-address
-  // global atomics retire slowly)
-  go_max = wave_max_u32(go_max);
-  mask_max = wave_max_u32(mask_max);
+  // the reach the grad_value kernel has to cover: fold in LDS, then touch the global word only when it would grow
+  // (same-address global atomics retire slowly)
   reach_needed = wave_max_u32(reach_needed);
-  if ((threadIdx.x & (kWave - 1)) == 0) {
-    atomicMax(&s_stat[0], go_max);
-    atomicMax(&s_stat[1], mask_max);
-    atomicMax(&s_stat[2], reach_needed);
-  }
+  if ((threadIdx.x & (kWave - 1)) == 0 && reach_needed != 0) atomicMax(&s_reach, reach_needed);
   __syncthreads();
-  if (threadIdx.x < 3) {
-    uint32_t *dst = &p.state->go_max_bits + threadIdx.x;
-    const uint32_t mine = s_stat[threadIdx.x];
+  if (threadIdx.x == 0) {
+    uint32_t *dst = &p.state->reach_needed;
+    const uint32_t mine = s_reach;
     if (mine > __hip_atomic_load(dst, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(dst, mine);
   }
   unstage_tile_grads<Tag>(p, t, s_om);
@@ -605,13 +594,8 @@ template <typename Tag, int NV, bool BWD>
 hipError_t launch_nv(const DcnLaunch &p, hipStream_t stream, dim3 grid, dim3 block, size_t lds) {
   const bool k3 = p.kh == 3 && p.kw == 3;
   auto go = [&](auto kernel) -> hipError_t {
-    static bool raised = false;        // per kernel instantiation: dynamic LDS above 64 KB needs the attribute
-    if (!raised) {
-      if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLdsPerWorkgroup - 1024))   // leaves room for static LDS
-        return e;
-      raised = true;
-    }
+    // leaves room for the kernels' static LDS
+    if (hipError_t e = ensure_dynamic_lds_limit(reinterpret_cast<const void *>(kernel), kMaxLdsPerWorkgroup - 1024)) return e;
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
     return hipGetLastError();
   };

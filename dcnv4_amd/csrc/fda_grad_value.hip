@@ -462,13 +462,7 @@ hipError_t launch_t(const FdaLaunch &p, hipStream_t stream) {
   const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(4, (kMaxLdsPerWorkgroup - 4096) / (lds + 1024)));
   const dim3 grid((unsigned)(cus * per_cu)), block(kApplyThreads);
   auto go = [&](auto kernel) -> hipError_t {
-    static bool raised = false;
-    if (!raised) {
-      if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLdsPerWorkgroup - 2048))
-        return e;
-      raised = true;
-    }
+    if (hipError_t e = ensure_dynamic_lds_limit(reinterpret_cast<const void *>(kernel), kMaxLdsPerWorkgroup - 2048)) return e;
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
     return hipGetLastError();
   };

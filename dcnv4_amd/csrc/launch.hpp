@@ -4,6 +4,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+#include <unordered_set>
+
 namespace dcn {
 
 // Largest span (bytes) one launch may address through a 32-bit buffer offset.  Value tensors
@@ -17,17 +20,30 @@ constexpr size_t kMaxLdsPerWorkgroup = 160 * 1024;  // gfx950
 
 // Device-side scratch word block shared by the kernels of one backward call (16 bytes).
 struct GradState {
-  uint32_t go_max_bits;    // max |grad_out| as IEEE bits (ordered like unsigned ints for x >= 0; NaN sorts last)
-  uint32_t mask_max_bits;  // max |modulation| (after softmax when enabled)
-  uint32_t reach_needed;   // largest Chebyshev distance (pixels) of an in-image corner of non-zero weight from its output pixel's reference point
-  uint32_t reserved;
+  uint32_t go_max_bits;    // attention backward: max |grad_out| as IEEE bits (ordered like unsigned ints for x >= 0; NaN sorts last)
+  uint32_t unused;
+  uint32_t reach_needed;   // DCNv4: largest Chebyshev distance (pixels) of an in-image corner of non-zero weight from its output pixel's reference point
+  uint32_t reserved;       // attention backward: set when a level has more tiles than the binning kernel can count
 };
 
-enum BackwardMode {
-  kBwdFull = 0,        // grad_offset_mask + fp32 atomic scatter of grad_value (generic path)
-  kBwdOffsetMask = 1,  // grad_offset_mask + GradState statistics, no scatter
-  kBwdFallback = 2,    // scatter of the corners the tiled kernel skipped, atomics in the tensor dtype
-};
+// Dynamic LDS above 64 KB needs hipFuncAttributeMaxDynamicSharedMemorySize on the kernel, on every device that runs
+// it (the reference sets it on every launch, DCNv4_op/src/cuda/dcnv4_col2im_cuda.cuh:454).  Set once per (kernel,
+// device); safe from concurrent host threads.
+inline hipError_t ensure_dynamic_lds_limit(const void *kernel, size_t bytes) {
+  static std::mutex mu;
+  static std::unordered_set<uint64_t> done;
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev)) return e;
+  const uint64_t key = (uint64_t)reinterpret_cast<uintptr_t>(kernel) * 64u + (uint64_t)(dev & 63);
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (done.count(key)) return hipSuccess;
+  }
+  if (hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes)) return e;
+  std::lock_guard<std::mutex> lock(mu);
+  done.insert(key);
+  return hipSuccess;
+}
 
 struct LaneMap {
   int cpt;          // channels per lane (power of two, cpt * elem_bytes <= 16)
@@ -41,7 +57,6 @@ struct DcnLaunch {
   const void *offset_mask;  // [n_pix, P_pad]
   const void *grad_out;     // [n_pix, G*D]            (backward)
   void *out;                // [n_pix, G*D]            (forward)
-  float *grad_value_acc;    // [n_img, H, W, G*D] fp32, zeroed (backward)
   void *grad_offset_mask;   // [n_pix, P_pad]          (backward)
   uint32_t value_bytes;
   int n_pix;                // images in this launch * Ho * Wo
@@ -57,11 +72,11 @@ struct DcnLaunch {
   int n_img;
   int tile_h, tile_w;       // input-space tile one workgroup owns (powers of two)
   int tile_h_log2, tile_w_log2;
-  int reach;                // cap on the reach the tiled scatter covers; it uses min(reach, GradState::reach_needed)
   int ng_chunk;             // groups per workgroup (channel chunk = ng_chunk * D)
   int strip_pix;            // output pixels staged per strip
-  int fix_bits;             // fractional bits of the fixed-point accumulators
-  int pack32;               // 16-bit tensors: two 32-bit sums per accumulator word instead of one 64-bit sum
+  int gv_cw;                // channels a lane accumulates: 8, 16 or 32
+  int gv_lps_log2;          // log2 of the lanes that share one (cell, group): group width / gv_cw, rounded up to a power of two
+  int gv_go_stride;         // bytes between the parked grad_out rows of consecutive pixels (an odd number of 16-byte units)
   // LDS-tiled gather path (forward and grad_offset_mask); gt_h == 0: not planned
   int gt_h, gt_w;           // output tile one workgroup owns
   int gt_ng;                // groups per workgroup
@@ -69,6 +84,10 @@ struct DcnLaunch {
   int gt_wh, gt_ww;         // largest input window (rows, columns of cells) a tile stages
   int gt_reach;             // input pixels around an output pixel's reference point that the window covers
 };
+
+// Sampling points a lane of the tiled grad_value kernel handles per strip, at most (it keeps them in registers next to
+// cw running sums): a strip holds at most 1024 * rounds of them.
+constexpr int dcnv4_grad_value_rounds(int cw) { return cw <= 16 ? 4 : 2; }
 
 // Flash deformable attention (reference: DCNv4_op/src/cuda/flash_deform_im2col_cuda.cuh:211-272)
 struct FdaLaunch {
@@ -159,7 +178,7 @@ int depthwise_grad_weight_pixel_lanes(int elem_bytes, int C, int k);
 hipError_t launch_depthwise_grad_weight_partials(int dtype, const DwLaunch &p, hipStream_t stream);
 hipError_t launch_depthwise_grad_weight_reduce(int dtype, const DwLaunch &p, hipStream_t stream);
 hipError_t launch_dcnv4_forward(int dtype, const DcnLaunch &p, hipStream_t stream);
-hipError_t launch_dcnv4_backward(int dtype, const DcnLaunch &p, int mode, hipStream_t stream);
+hipError_t launch_dcnv4_offset_mask_grad(int dtype, const DcnLaunch &p, hipStream_t stream);
 hipError_t launch_dcnv4_grad_value(int dtype, const DcnLaunch &p, hipStream_t stream);
 size_t dcnv4_grad_value_lds_bytes(const DcnLaunch &p);
 hipError_t launch_dcnv4_forward_tiled(int dtype, const DcnLaunch &p, hipStream_t stream);

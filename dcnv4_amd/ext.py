@@ -41,25 +41,44 @@ def _hint(v):
 
 
 _FAMILY = {"auto": 0, "tiled": 1, "direct": 2, "atomic": 2}
+_ORDER = {"auto": 0, "rows": 1, "heads": 2}
 
 
 class launch_options:
     """Context manager over the calling thread's launch options (include/dcnv4_gfx950.h,
     ``dcnv4_gfx950_set_launch_option``): ``gather`` in auto / tiled / direct, ``scatter`` in auto / tiled / atomic,
-    ``reach`` an int or None.  Used by the tuner and by dispatch-table entries that carry options; the options are
-    back at the library's choice on exit.  Results do not depend on them beyond the rounding of sums."""
+    ``reach`` an int or None, ``tile`` 8 / 16 / 32 or None, ``fda_order`` in auto / rows / heads.  Used by the tuner,
+    by dispatch-table entries that carry options and by tests that force a kernel family; on exit every option is
+    back at the value it had on entry, so contexts nest.  Results do not depend on the options beyond the rounding
+    of sums."""
 
-    def __init__(self, gather="auto", scatter="auto", reach=None):
-        self.values = {"gather": _FAMILY[gather], "scatter": _FAMILY[scatter], "reach": -1 if reach is None else int(reach)}
+    def __init__(self, gather=None, scatter=None, reach=None, tile=None, fda_order=None):
+        self.values = {}
+        if gather is not None:
+            self.values["gather"] = _FAMILY[gather]
+        if scatter is not None:
+            self.values["scatter"] = _FAMILY[scatter]
+        if reach is not None:
+            self.values["reach"] = int(reach)
+        if tile is not None:
+            self.values["tile"] = int(tile)
+        if fda_order is not None:
+            self.values["fda_order"] = _ORDER[fda_order]
+        self.saved = {}
 
     def __enter__(self):
+        import ctypes
         for name, value in self.values.items():
+            old = ctypes.c_int(0)
+            _lib.check(_L.dcnv4_gfx950_get_launch_option(name.encode(), ctypes.byref(old)))
+            self.saved[name] = old.value
             _lib.check(_L.dcnv4_gfx950_set_launch_option(name.encode(), value))
         return self
 
     def __exit__(self, *exc):
-        for name in self.values:
-            _L.dcnv4_gfx950_set_launch_option(name.encode(), -1 if name == "reach" else 0)
+        for name, value in self.saved.items():
+            _L.dcnv4_gfx950_set_launch_option(name.encode(), value)
+        self.saved = {}
         return False
 
 

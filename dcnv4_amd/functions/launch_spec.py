@@ -11,7 +11,7 @@ B*H*W on every call).
 Measured overrides live in ``gfx950_table.json`` next to this file, written by ``python -m dcnv4_amd.tune``
 (the counterpart of DCNv4_op/scripts/search_dcnv4.py, search_dcnv4_bwd.py and find_best.py).  Its keys are the
 reference's ``"BxHxWxGxC"`` plus the element size and the direction; an entry holds the two hints and, optionally,
-the kernel families to use (``gather`` = tiled / direct, ``scatter`` = tiled / atomic), which
+launch options (``gather`` = tiled / direct, ``tile`` = 8 / 16 / 32, ``reach`` = pixels), which
 :func:`launch_options_for` hands to the library as thread-local launch options around the call.
 """
 import functools
@@ -30,7 +30,8 @@ def _load_table(path=TABLE_PATH):
         return json.load(f).get("entries", {})
 
 
-# key -> {"d_stride": int, "n_thread": int, "gather": str (optional), "scatter": str (optional)}
+# key -> {"d_stride": int, "n_thread": int, and optionally "gather": str, "tile": int, "reach": int}
+OPTION_KEYS = ("gather", "tile", "reach")
 GFX950_TABLE = _load_table()
 
 
@@ -61,7 +62,7 @@ def _spec(group, group_channels, elem_bytes, scatter=False):
 def _lookup(B, H, W, G, C, elem_bytes, direction):
     entry = GFX950_TABLE.get(table_key(B, H, W, G, C, elem_bytes, direction))
     if entry is not None:
-        options = {k: entry[k] for k in ("gather", "scatter") if entry.get(k, "auto") != "auto"}
+        options = {k: entry[k] for k in OPTION_KEYS if entry.get(k, "auto") not in ("auto", None)}
         return (int(entry["d_stride"]), int(entry["n_thread"])), options
     return _spec(G, C, elem_bytes, scatter=direction == "bwd"), {}
 

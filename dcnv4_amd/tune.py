@@ -48,8 +48,8 @@ def candidates(G, D, elem_bytes, direction):
                 out.append((f"direct d{d} n{n}", {"gather": "direct"}, d, n))
     else:
         out.append(("direct gathers", {"gather": "direct"}, 0, 0))
-        out.append(("atomic scatter", {"scatter": "atomic"}, 0, 0))
-        out.append(("direct gathers, atomic scatter", {"gather": "direct", "scatter": "atomic"}, 0, 0))
+        for tile in (16, 8):
+            out.append((f"grad_value tile {tile}", {"tile": tile}, 0, 0))
     return out
 
 

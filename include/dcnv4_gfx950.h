@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define DCNV4_GFX950_ABI_VERSION 3
+#define DCNV4_GFX950_ABI_VERSION 4
 
 #define DCNV4_DTYPE_F32 0
 #define DCNV4_DTYPE_F16 1
@@ -50,18 +50,23 @@ const char *dcnv4_gfx950_last_error(void);
 /*
  * Launch options of the calling thread, for tuners and for dispatch tables made by them; they play the
  * part of the reference's per-shape launch table (DCNv4_op/DCNv4/functions/table.py, filled by
- * DCNv4_op/scripts/search_dcnv4.py, search_dcnv4_bwd.py and find_best.py).  Results never depend on them
- * beyond the rounding of sums.
- *   "gather"   0 library's choice, 1 LDS-tiled gathers where the shape allows, 2 direct gathers
- *              (forward and grad_offset_mask kernels)
- *   "scatter"  0 library's choice, 1 tiled LDS accumulation where the shape allows, 2 global atomics
- *              (grad_value of both operators; decides the workspace size as well)
- *   "reach"    -1 library's choice, else 0..64: input pixels around an output pixel's reference point that
- *              the tiled DCNv4 kernels cover
- * An option that is not set falls back to the environment variable of the same purpose
- * (DCNV4_GFX950_GATHER=direct, DCNV4_GFX950_FDA_SCATTER=atomic, DCNV4_GFX950_REACH=n).
+ * DCNv4_op/scripts/search_dcnv4.py, search_dcnv4_bwd.py and find_best.py).  They choose between kernels that
+ * compute the same result (up to the rounding of sums); workspace sizes never depend on them, and the library
+ * reads no environment variables.
+ *   "gather"     0 library's choice, 1 LDS-tiled gathers where the shape allows, 2 direct gathers
+ *                (DCNv4 forward and grad_offset_mask kernels)
+ *   "scatter"    0 library's choice, 1 binned LDS accumulation where the shape allows, 2 global atomics
+ *                (grad_value of flash deformable attention)
+ *   "reach"      -1 library's choice (5), else 0..64: input pixels around an output pixel's reference point that
+ *                the LDS-tiled DCNv4 gathers stage; sampling points beyond it are fetched from memory
+ *   "tile"       0 library's choice (32), else 8, 16 or 32: largest side of the input tile a workgroup of the
+ *                DCNv4 grad_value kernel owns
+ *   "fda_order"  0 library's choice, 1 whole query rows per workgroup, 2 one head per workgroup
+ *                (flash deformable attention forward and grad_sampling_loc_attn kernels)
+ * dcnv4_gfx950_get_launch_option reads a value back, so that a caller can restore what it found.
  */
 int dcnv4_gfx950_set_launch_option(const char *name, int value);
+int dcnv4_gfx950_get_launch_option(const char *name, int *value);
 
 /*
  * DCNv4 forward.  Replaces dcnv4_forward / dcnv4_cuda_forward
@@ -81,7 +86,7 @@ int dcnv4_gfx950_forward(const void *value, const void *offset_mask, void *outpu
                          int im2col_step, int remove_center, int padded_offset_dim, int softmax,
                          int d_stride, int block_thread, void *stream);
 
-/* Scratch bytes dcnv4_gfx950_backward needs for these sizes (0 for fp32). */
+/* Scratch bytes dcnv4_gfx950_backward needs: 256 (a few words of state shared by its kernels), whatever the sizes. */
 size_t dcnv4_gfx950_backward_workspace_bytes(int dtype, int batch, int height_in, int width_in,
                                              int group, int group_channels);
 

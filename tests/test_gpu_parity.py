@@ -35,6 +35,12 @@ DCN_CASES = {
     "d6_three_lane_cluster": (2, 6, 5, 3, 6, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
     "d48_six_lane_cluster": (1, 8, 8, 2, 48, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
     "d64": (1, 8, 9, 2, 64, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
+    # four lanes of 32 channels per (cell, group) in the tiled grad_value kernel, the last one partly idle
+    "d104_four_lanes_per_slot": (1, 9, 7, 2, 104, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
+    # the widest group the fp32 backward takes: 64 gather lanes, eight lanes of 32 channels per (cell, group)
+    "d256_eight_lanes_per_slot": (1, 5, 6, 1, 256, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
+    # 49 taps: strips of a few pixels
+    "kernel_7x7_g3": (1, 12, 11, 3, 16, (7, 7, 1, 1, 3, 3, 1, 1), 0, 1.0, 1.5),
     "far_offsets_mostly_outside": (1, 5, 5, 4, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 9.0),
     "single_pixel": (1, 1, 1, 1, 16, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 1.0),
     # 32-wide grad_value tiles, one group per workgroup: a one-pixel remainder tile in both directions
@@ -76,16 +82,16 @@ def test_dcnv4_forward_and_backward_match_oracle(oracle, name, dtype):
     assert (gom[..., used:] == 0).all(), "padded tail of grad_offset_mask must be exactly zero"
 
 
-# The library picks between kernel families by shape; these settings force the other branches:
-# the global-memory gather kernels, and (tiny reach) the per-point fallbacks of the LDS-tiled
-# kernels plus the far-corner scatter of the backward.
+# The library picks between kernel families by shape; these launch options force the other branches:
+# the global-memory gather kernels, (tiny reach) the per-point global fetches of the LDS-tiled
+# gathers, and smaller grad_value tiles with several groups per workgroup.
 KERNEL_PATHS = {
-    "direct_gather": {"DCNV4_GFX950_GATHER": "direct"},
-    "reach1": {"DCNV4_GFX950_REACH": "1"},
-    "reach0": {"DCNV4_GFX950_REACH": "0"},
-    "reach9": {"DCNV4_GFX950_REACH": "9"},
-    "tile16": {"DCNV4_GFX950_TILE": "16"},                                   # grad_value on 16x16 tiles, four groups each
-    "tile16_reach1": {"DCNV4_GFX950_TILE": "16", "DCNV4_GFX950_REACH": "1"},
+    "direct_gather": dict(gather="direct"),
+    "reach1": dict(reach=1),
+    "reach0": dict(reach=0),
+    "reach9": dict(reach=9),
+    "tile16": dict(tile=16),                                   # grad_value on 16x16 tiles, four groups each
+    "tile8_reach1": dict(tile=8, reach=1),
 }
 
 
@@ -93,16 +99,16 @@ KERNEL_PATHS = {
 @pytest.mark.parametrize("path", list(KERNEL_PATHS))
 @pytest.mark.parametrize("name", ["cfg1_56x56_c64_g4", "g7_c112_scale_half", "remove_center", "stride2", "dilation2_pad2",
                                   "kernel_5x5", "far_offsets_mostly_outside", "wide_g80"])
-def test_dcnv4_every_kernel_path_matches_oracle(oracle, monkeypatch, name, path, dtype):
-    for key, val in KERNEL_PATHS[path].items():
-        monkeypatch.setenv(key, val)
+def test_dcnv4_every_kernel_path_matches_oracle(oracle, name, path, dtype):
+    from dcnv4_amd import ext
     v, om, go, (geom, G, D, scale, rc) = _dcn_inputs(DCN_CASES[name], dtype, seed=zlib.crc32((name + path).encode()) % 1000)
     print(f"case {name} path {path} dtype {dtype}", flush=True)
     args = _oracle_args(geom, G, D, scale, rc)
     want = oracle.dcnv4_forward(cabi.f64(v), cabi.f64(om), *args, coord_f32=True)
     wgv, wgom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *args, coord_f32=True)
-    out = cabi.dcnv4_forward(v.cuda(), om.cuda(), geom, G, D, scale, rc)
-    gv, gom = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), geom, G, D, scale, rc)
+    with ext.launch_options(**KERNEL_PATHS[path]):
+        out = cabi.dcnv4_forward(v.cuda(), om.cuda(), geom, G, D, scale, rc)
+        gv, gom = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), geom, G, D, scale, rc)
     torch.cuda.synchronize()
     cabi.assert_close(out, want, *FWD_TOL[dtype], what="output")
     cabi.assert_close(gv, wgv, *GRAD_TOL[dtype], what="grad_value")
@@ -218,9 +224,8 @@ FDA_PATH_CASES = {
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
 @pytest.mark.parametrize("scatter", ["tiled", "atomic"])
 @pytest.mark.parametrize("name", ["detr_small_4lvl_k4", "five_levels", "k8_one_level"] + list(FDA_PATH_CASES))
-def test_flash_deform_attn_backward_paths_match_oracle(oracle, monkeypatch, name, scatter, dtype):
-    if scatter == "atomic":
-        monkeypatch.setenv("DCNV4_GFX950_FDA_SCATTER", "atomic")
+def test_flash_deform_attn_backward_paths_match_oracle(oracle, name, scatter, dtype):
+    from dcnv4_amd import ext
     if name == "level_wider_than_a_key" and dtype != torch.float32:
         pytest.skip("location gradients scale with the level width (65530) and overflow the 16-bit types")
     B, shapes, G, D, K, Q, (lo, hi) = {**FDA_CASES, **FDA_PATH_CASES}[name]
@@ -228,7 +233,8 @@ def test_flash_deform_attn_backward_paths_match_oracle(oracle, monkeypatch, name
     v, shp, st, sla, go = make_fda_inputs(B, shapes, G, D, K, Q, seed=zlib.crc32((name + scatter).encode()) % 1000, dtype=dtype,
                                           loc_lo=lo, loc_hi=hi)
     wgv, wgs = oracle.flash_deform_attn_backward(cabi.f64(v), shp.numpy(), st.numpy(), cabi.f64(sla), cabi.f64(go), K, coord_f32=True)
-    gv, gs = cabi.fda_backward(v.cuda(), shp.cuda(), st.cuda(), sla.cuda(), go.cuda(), K)
+    with ext.launch_options(scatter=scatter):
+        gv, gs = cabi.fda_backward(v.cuda(), shp.cuda(), st.cuda(), sla.cuda(), go.cuda(), K)
     torch.cuda.synchronize()
     rtol, atol = GRAD_TOL[dtype]
     if name == "crowded_small_level":       # thousands of terms per cell: the tolerance scales with the sum's magnitude
@@ -380,7 +386,7 @@ def test_layer_norm_residual_rejects_unsupported_widths():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16], ids=["fp32", "fp16"])
-def test_flash_deform_attn_head_major_order_matches_oracle_and_row_order(oracle, dtype, monkeypatch):
+def test_flash_deform_attn_head_major_order_matches_oracle_and_row_order(oracle, dtype):
     """A value image larger than half an L2 slice whose heads each fit one: the library then gives every workgroup one
     head and orders workgroups [image][head][queries].  Same arithmetic per (query, head), so the same bits as the
     row order, and parity with the oracle."""
@@ -391,9 +397,10 @@ def test_flash_deform_attn_head_major_order_matches_oracle_and_row_order(oracle,
     print(f"head-major case {dtype}", flush=True)
     out = cabi.fda_forward(*args, K)
     gv, gs = cabi.fda_backward(*args, go.cuda(), K)
-    monkeypatch.setenv("DCNV4_GFX950_FDA_ORDER", "rows")
-    out_rows = cabi.fda_forward(*args, K)
-    gv_rows, gs_rows = cabi.fda_backward(*args, go.cuda(), K)
+    from dcnv4_amd import ext
+    with ext.launch_options(fda_order="rows"):
+        out_rows = cabi.fda_forward(*args, K)
+        gv_rows, gs_rows = cabi.fda_backward(*args, go.cuda(), K)
     assert torch.equal(out, out_rows) and torch.equal(gs, gs_rows) and torch.equal(gv, gv_rows)
     want = oracle.flash_deform_attn_forward(cabi.f64(v), shp.numpy(), st.numpy(), cabi.f64(sla), K, coord_f32=True)
     wgv, wgs = oracle.flash_deform_attn_backward(cabi.f64(v), shp.numpy(), st.numpy(), cabi.f64(sla), cabi.f64(go), K, coord_f32=True)

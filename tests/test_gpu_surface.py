@@ -130,13 +130,17 @@ def test_flash_deform_attn_module_matches_a_reference_built_from_torch_ops():
     assert _rel_err(got.detach().cpu(), want.detach()) < 2e-4
 
 
-def test_backward_is_bit_reproducible():
+def test_backward_repeats_to_the_rounding_of_fp32_sums():
+    """grad_offset_mask has a fixed summation order: same bits every time.  grad_value sums each cell's terms in fp32
+    in the order the hardware ranked them (like the reference's atomics): repeats agree to fp32 rounding, far inside
+    one unit of the fp16 result."""
     B, H, W, G, D = 4, 28, 28, 8, 16
-    v, om, go = (t.cuda() for t in make_dcnv4_inputs(B, H, W, G, D, offset_range=3.0, seed=8, dtype=torch.float16))
+    v, om, go = (t.cuda() for t in make_dcnv4_inputs(B, H, W, G, D, offset_range=3.0, seed=8, dtype=torch.float32))
     first = cabi.dcnv4_backward(v, om, go, GEOM, G, D, 1.0)
     for _ in range(3):
         again = cabi.dcnv4_backward(v, om, go, GEOM, G, D, 1.0)
-        assert torch.equal(first[0], again[0]) and torch.equal(first[1], again[1])
+        assert torch.equal(first[1], again[1])
+        assert (first[0] - again[0]).abs().max().item() <= 2e-5 and _rel_err(first[0], again[0]) < 1e-6
 
 
 def test_nan_in_grad_output_propagates_like_the_oracle(oracle):
@@ -260,7 +264,7 @@ def test_batches_beyond_the_32_bit_addressing_span_are_chunked_consistently():
     gv, gom = cabi.dcnv4_backward(v, om, g, GEOM, G, D, 1.0)
     pv, pom = cabi.dcnv4_backward(v[9:12].contiguous(), om[9:12].contiguous(), g[9:12].contiguous(), GEOM, G, D, 1.0)
     assert torch.equal(gom[9:12], pom)
-    assert _rel_err(gv[9:12], pv) < 1e-6       # fixed-point scale comes from the global maxima of each call
+    assert _rel_err(gv[9:12], pv) < 1e-6       # fp32 sums in hardware order
 
 
 def test_forward_and_backward_replay_correctly_from_a_hip_graph():
@@ -288,7 +292,10 @@ def test_forward_and_backward_replay_correctly_from_a_hip_graph():
         (v.float() @ torch.ones(64, 8, device="cuda")).sum().item()      # unrelated eager work + sync between replays
         graph.replay()
         torch.cuda.synchronize()
-        assert torch.equal(g_out, eager_out) and torch.equal(g_gv, eager_gv) and torch.equal(g_gom, eager_gom)
+        assert torch.equal(g_out, eager_out) and torch.equal(g_gom, eager_gom)
+        # grad_value: fp32 sums in hardware order, rounded once to fp16: at most one unit apart, and rarely
+        diff = (g_gv.float() - eager_gv.float()).abs()
+        assert (diff <= 2e-3 * eager_gv.float().abs() + 1e-6).all() and (diff > 0).float().mean().item() < 0.01
 
 
 def test_small_flash_intern_image_matches_the_same_network_on_the_torch_core(monkeypatch):
@@ -421,8 +428,8 @@ def test_dcnv4_module_under_autocast_runs_the_half_kernels_and_returns_fp32_para
         assert _rel_err(p.grad.cpu(), ref_grads[k].cpu()) < tol, k
 
 
-@pytest.mark.parametrize("options", [dict(gather="direct"), dict(scatter="atomic"), dict(gather="direct", scatter="atomic"),
-                                     dict(gather="tiled", scatter="tiled", reach=2)])
+@pytest.mark.parametrize("options", [dict(gather="direct"), dict(tile=16), dict(gather="direct", tile=8),
+                                     dict(gather="tiled", reach=2)])
 def test_launch_options_change_the_kernels_not_the_results(options):
     """Thread-local launch options (what a tuned table entry applies around a call) against the library's own choice."""
     import dcnv4_amd
@@ -438,9 +445,10 @@ def test_launch_options_change_the_kernels_not_the_results(options):
     assert _rel_err(out.float().cpu(), want.float().cpu()) < 2e-3
     assert _rel_err(gv.float().cpu(), wgv.float().cpu()) < 1e-2
     assert _rel_err(gom.float().cpu(), wgom.float().cpu()) < 2e-3
-    # the options are back at the library's choice afterwards: same bits as before
+    # the options are back at the library's choice afterwards: same kernels as before (grad_offset_mask has a
+    # fixed summation order, so the same bits)
     again = ext.dcnv4_backward(v, om, *geom, 4, 16, 1.0, 64, go, 0, 0, 0, False)
-    assert torch.equal(again[0], wgv) and torch.equal(again[1], wgom)
+    assert torch.equal(again[1], wgom) and _rel_err(again[0].float().cpu(), wgv.float().cpu()) < 1e-3
 
 
 def test_fused_block_tail_has_autograd_gradients_and_falls_back_under_autocast():
@@ -553,7 +561,7 @@ def test_autograd_function_applies_a_tuned_table_entry(monkeypatch):
     v, om, go = (t.cuda() for t in make_dcnv4_inputs(B, H, W, G, D, seed=14, dtype=torch.float16))
     want = dcnv4_amd.DCNv4Function.apply(v, om, *GEOM, G, D, 1.0, 256, 0)
     monkeypatch.setitem(ls.GFX950_TABLE, ls.table_key(B, H, W, G, D, 2, "fwd"), {"d_stride": 8, "n_thread": 128, "gather": "direct"})
-    monkeypatch.setitem(ls.GFX950_TABLE, ls.table_key(B, H, W, G, D, 2, "bwd"), {"d_stride": 1, "n_thread": 64, "scatter": "atomic"})
+    monkeypatch.setitem(ls.GFX950_TABLE, ls.table_key(B, H, W, G, D, 2, "bwd"), {"d_stride": 1, "n_thread": 64, "tile": 16})
     ls._lookup.cache_clear()
     seen = []
     real = _lib.load().dcnv4_gfx950_set_launch_option
@@ -570,8 +578,8 @@ def test_autograd_function_applies_a_tuned_table_entry(monkeypatch):
         out.backward(go)
     finally:
         ls._lookup.cache_clear()
-    assert (b"gather", 2) in seen and (b"scatter", 2) in seen
-    assert seen[-3:] == [(b"gather", 0), (b"scatter", 0), (b"reach", -1)]          # back at the library's choice
+    assert (b"gather", 2) in seen and (b"tile", 16) in seen
+    assert seen[-1] == (b"tile", 0) and (b"gather", 0) in seen          # back at the library's choice
     assert _rel_err(out.float().cpu(), want.float().cpu()) < 2e-3 and vg.grad is not None and omg.grad is not None
 
 

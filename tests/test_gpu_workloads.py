@@ -248,15 +248,10 @@ def test_flash_deform_attn_value_rows_no_level_covers_get_zero_gradient(oracle):
     big[:, :30] = v[:, :30]
     big[:, 30 + gap: 30 + gap + 12] = v[:, 30:]
     starts = torch.tensor([0, 30 + gap], dtype=torch.int64)
+    from dcnv4_amd import ext
     for scatter in ("tiled", "atomic"):
-        import os
-        os.environ.pop("DCNV4_GFX950_FDA_SCATTER", None)
-        if scatter == "atomic":
-            os.environ["DCNV4_GFX950_FDA_SCATTER"] = "atomic"
-        try:
+        with ext.launch_options(scatter=scatter):
             gv, _ = cabi.fda_backward(big.cuda(), shp.cuda(), starts.cuda(), sla.cuda(), go.cuda(), K)
-        finally:
-            os.environ.pop("DCNV4_GFX950_FDA_SCATTER", None)
         torch.cuda.synchronize()
         gv = gv.cpu()
         assert (gv[:, 30: 30 + gap] == 0).all() and (gv[:, 30 + gap + 12:] == 0).all(), scatter

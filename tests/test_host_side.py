@@ -24,7 +24,7 @@ def test_library_exports_every_symbol_the_header_declares():
     from dcnv4_amd import _lib
     lib = ctypes.CDLL(_lib.LIB_PATH)
     declared = _declared_functions()
-    assert len(declared) == 13, sorted(declared)
+    assert len(declared) == 14, sorted(declared)
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in include/dcnv4_gfx950.h but not exported"
     assert set(declared) == set(_lib.SIGNATURES), "ctypes table and header list different functions"
@@ -50,8 +50,8 @@ def test_abi_version_and_error_string_work_without_a_gpu():
     rc = lib.flash_deform_attn_gfx950_forward(None, None, None, None, None, 1, 1, 16, 1, 16, 6, 4, 16, 64, 0, 0, None)
     assert rc == _lib.ERR_INVALID_ARGUMENT and b"points" in lib.dcnv4_gfx950_last_error()
     assert lib.dcnv4_gfx950_backward_workspace_bytes(1, 64, 56, 56, 4, 16) == 256
-    assert lib.dcnv4_gfx950_backward_workspace_bytes(1, 2, 8, 8, 1, 128) == 2 * 8 * 8 * 128 * 4
-    assert lib.dcnv4_gfx950_backward_workspace_bytes(0, 2, 8, 8, 1, 128) == 0
+    assert lib.dcnv4_gfx950_backward_workspace_bytes(1, 2, 8, 8, 1, 128) == 256
+    assert lib.dcnv4_gfx950_backward_workspace_bytes(0, 2, 8, 8, 1, 384) == 256
 
 
 def test_cpu_tensors_are_refused_like_the_reference():
@@ -207,16 +207,52 @@ def test_launch_options_are_validated_without_a_gpu():
     lib = _lib.load()
     assert lib.dcnv4_gfx950_set_launch_option(b"gather", 2) == 0 and lib.dcnv4_gfx950_set_launch_option(b"gather", 0) == 0
     assert lib.dcnv4_gfx950_set_launch_option(b"reach", 7) == 0 and lib.dcnv4_gfx950_set_launch_option(b"reach", -1) == 0
+    assert lib.dcnv4_gfx950_set_launch_option(b"tile", 16) == 0 and lib.dcnv4_gfx950_set_launch_option(b"tile", 0) == 0
+    assert lib.dcnv4_gfx950_set_launch_option(b"tile", 12) == _lib.ERR_INVALID_ARGUMENT
     assert lib.dcnv4_gfx950_set_launch_option(b"gather", 5) == _lib.ERR_INVALID_ARGUMENT
     assert lib.dcnv4_gfx950_set_launch_option(b"nonsense", 1) == _lib.ERR_INVALID_ARGUMENT
     assert b"nonsense" in lib.dcnv4_gfx950_last_error()
-    # the scatter option decides the workspace: global atomics need an fp32 image for 16-bit tensors
-    tiled = lib.dcnv4_gfx950_backward_workspace_bytes(1, 2, 8, 8, 2, 16)
-    lib.dcnv4_gfx950_set_launch_option(b"scatter", 2)
-    try:
-        assert lib.dcnv4_gfx950_backward_workspace_bytes(1, 2, 8, 8, 2, 16) == 2 * 8 * 8 * 32 * 4 and tiled == 256
-    finally:
-        lib.dcnv4_gfx950_set_launch_option(b"scatter", 0)
+
+
+def test_launch_option_contexts_nest_and_restore_what_they_found():
+    import ctypes
+    from dcnv4_amd import _lib, ext
+    lib = _lib.load()
+
+    def get(name):
+        v = ctypes.c_int(123)
+        assert lib.dcnv4_gfx950_get_launch_option(name, ctypes.byref(v)) == 0
+        return v.value
+
+    assert get(b"reach") == -1 and get(b"gather") == 0
+    with ext.launch_options(reach=3, gather="direct"):
+        assert get(b"reach") == 3 and get(b"gather") == 2
+        with ext.launch_options(reach=9):
+            assert get(b"reach") == 9 and get(b"gather") == 2
+        assert get(b"reach") == 3
+    assert get(b"reach") == -1 and get(b"gather") == 0
+    assert lib.dcnv4_gfx950_get_launch_option(b"nonsense", ctypes.byref(ctypes.c_int())) == _lib.ERR_INVALID_ARGUMENT
+
+
+def test_workspace_sizes_do_not_depend_on_launch_options_or_threads():
+    """The size query and the call must agree whatever happens between them: the sizes are functions of the
+    arguments only."""
+    import threading
+    from dcnv4_amd import _lib, ext
+    lib = _lib.load()
+    dcn = lambda: lib.dcnv4_gfx950_backward_workspace_bytes(1, 2, 8, 8, 2, 16)
+    fda = lambda: lib.flash_deform_attn_gfx950_backward_workspace_bytes(1, 2, 80, 4, 32, 2, 50, 4)
+    base = (dcn(), fda())
+    assert base[0] == 256 and base[1] > 0
+    for options in (dict(scatter="atomic"), dict(gather="direct", tile=8), dict(fda_order="rows", reach=0)):
+        with ext.launch_options(**options):
+            assert (dcn(), fda()) == base
+    seen = []
+    t = threading.Thread(target=lambda: seen.append((dcn(), fda())))
+    with ext.launch_options(scatter="atomic"):
+        t.start()
+        t.join()
+    assert seen == [base]
 
 
 def test_tuner_candidates_are_valid_hints_and_start_with_the_library_choice():
@@ -227,7 +263,7 @@ def test_tuner_candidates_are_valid_hints_and_start_with_the_library_choice():
         for _, options, d_stride, n_thread in fwd[1:]:
             assert options == {"gather": "direct"} and D % d_stride == 0 and d_stride * es <= 16 and n_thread in (128, 256, 512)
         bwd = tune.candidates(G, D, es, "bwd")
-        assert bwd[0] == ("library", {}, 0, 0) and {"scatter": "atomic"} in [c[1] for c in bwd]
+        assert bwd[0] == ("library", {}, 0, 0) and {"tile": 16} in [c[1] for c in bwd]
     assert set(tune.SHAPES) == {"t", "b", "dense"} and all(len(v) == 4 for v in tune.SHAPES.values())
 
 
