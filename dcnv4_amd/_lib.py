@@ -25,6 +25,7 @@ SIGNATURES = {
     "dcnv4_gfx950_forward": (_i, [_vp, _vp, _vp, _i] + [_i] * 13 + [_f] + [_i] * 6 + [_vp]),
     "dcnv4_gfx950_backward_workspace_bytes": (_sz, [_i] * 6),
     "dcnv4_gfx950_backward": (_i, [_vp] * 6 + [_sz, _i] + [_i] * 13 + [_f] + [_i] * 6 + [_vp]),
+    "dcnv4_gfx950_backward_static_scratch": (_i, [_vp] * 5 + [_i] + [_i] * 13 + [_f] + [_i] * 6 + [_vp]),
     "flash_deform_attn_gfx950_forward": (_i, [_vp] * 5 + [_i] * 11 + [_vp]),
     "flash_deform_attn_gfx950_backward_workspace_bytes": (_sz, [_i] * 8),
     "flash_deform_attn_gfx950_backward": (_i, [_vp] * 8 + [_sz] + [_i] * 11 + [_vp]),

@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/dcnv4_gfx950.h"
 #include "common.hpp"
@@ -440,6 +441,33 @@ void dw_segments(DwLaunch *L, int elem_bytes_of_launch) {
   L->n_seg = (L->Wo + L->seg - 1) / L->seg;
 }
 
+// ---------------------------------------------------------------- static scratch
+// Scratch of dcnv4_gfx950_backward_static_scratch, for callers that cannot allocate: one array per GPU, held from
+// the moment the library's code is loaded on that GPU until the process ends.  The name of a __device__ array is
+// only a host-side handle; the array's device address is looked up once per device and kept.
+constexpr size_t kStaticScratchBytes = DCNV4_GFX950_STATIC_SCRATCH_BYTES;
+__device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch_of_current_device(void **out) {
+  int dev = -1;
+  if (hipError_t e = hipGetDevice(&dev)) return fail(DCNV4_ERR_RUNTIME, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(DCNV4_ERR_RUNTIME, "device ordinal %d is out of range (0..%d)", dev, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void *ptr = nullptr;
+    if (hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_scratch)))
+      return fail(DCNV4_ERR_RUNTIME, "hipGetSymbolAddress(static scratch) on device %d: %s", dev, hipGetErrorString(e));
+    if (ptr == nullptr || !aligned16(ptr)) return fail(DCNV4_ERR_RUNTIME, "static scratch of device %d has address %p", dev, ptr);
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return DCNV4_OK;
+}
+
 const char *at(const void *base, size_t elems, int s) { return static_cast<const char *>(base) + elems * s; }
 char *at(void *base, size_t elems, int s) { return static_cast<char *>(base) + elems * s; }
 
@@ -578,6 +606,26 @@ int dcnv4_gfx950_backward(const void *value, const void *offset_mask, const void
                           float offset_scale, int im2col_step, int remove_center, int padded_offset_dim,
                           int softmax, int d_stride, int block_thread, void *stream) {
   return dcn_backward_impl(value, offset_mask, grad_output, grad_value, grad_offset_mask, workspace, workspace_bytes, dtype,
+                           batch, height_in, width_in, group, group_channels, kernel_h, kernel_w, stride_h, stride_w, pad_h,
+                           pad_w, dilation_h, dilation_w, offset_scale, im2col_step, remove_center, padded_offset_dim,
+                           softmax, d_stride, block_thread, stream);
+}
+
+int dcnv4_gfx950_backward_static_scratch(const void *value, const void *offset_mask, const void *grad_output,
+                                         void *grad_value, void *grad_offset_mask, int dtype, int batch, int height_in,
+                                         int width_in, int group, int group_channels, int kernel_h, int kernel_w,
+                                         int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h,
+                                         int dilation_w, float offset_scale, int im2col_step, int remove_center,
+                                         int padded_offset_dim, int softmax, int d_stride, int block_thread,
+                                         void *stream) {
+  const size_t need = dcnv4_gfx950_backward_workspace_bytes(dtype, batch, height_in, width_in, group, group_channels);
+  if (need > kStaticScratchBytes)
+    return fail(DCNV4_ERR_RUNTIME,
+                "this backward needs %zu bytes of scratch; the library's static scratch holds %zu "
+                "(use dcnv4_gfx950_backward with a caller-provided workspace)", need, kStaticScratchBytes);
+  void *scratch = nullptr;
+  if (int rc = static_scratch_of_current_device(&scratch)) return rc;
+  return dcn_backward_impl(value, offset_mask, grad_output, grad_value, grad_offset_mask, scratch, kStaticScratchBytes, dtype,
                            batch, height_in, width_in, group, group_channels, kernel_h, kernel_w, stride_h, stride_w, pad_h,
                            pad_w, dilation_h, dilation_w, offset_scale, im2col_step, remove_center, padded_offset_dim,
                            softmax, d_stride, block_thread, stream);

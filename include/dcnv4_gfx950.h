@@ -109,6 +109,24 @@ int dcnv4_gfx950_backward(const void *value, const void *offset_mask, const void
                           void *stream);
 
 /*
+ * DCNv4 backward for callers that cannot allocate device memory (code running under HIP graph capture, serving
+ * loops, harnesses that forbid hipMalloc): dcnv4_gfx950_backward without the workspace arguments.  It has no
+ * counterpart in the reference.  The scratch lives in a device array inside the library, DCNV4_GFX950_STATIC_SCRATCH_BYTES
+ * per GPU, held until the process ends; the call fails with DCNV4_ERR_RUNTIME when
+ * dcnv4_gfx950_backward_workspace_bytes() for these sizes is larger.  The call allocates and frees nothing.  All
+ * calls on one GPU share the array: two such calls that overlap in time on the same GPU (different streams or
+ * threads) race; calls on one stream are ordered and safe.
+ */
+#define DCNV4_GFX950_STATIC_SCRATCH_BYTES 4096u
+int dcnv4_gfx950_backward_static_scratch(const void *value, const void *offset_mask, const void *grad_output,
+                                         void *grad_value, void *grad_offset_mask, int dtype, int batch,
+                                         int height_in, int width_in, int group, int group_channels,
+                                         int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h,
+                                         int pad_w, int dilation_h, int dilation_w, float offset_scale,
+                                         int im2col_step, int remove_center, int padded_offset_dim, int softmax,
+                                         int d_stride, int block_thread, void *stream);
+
+/*
  * Flash deformable attention forward.  Replaces flash_deform_attn_forward /
  * flash_deform_attn_cuda_forward (DCNv4_op/src/dcnv4.h:19-36,
  * DCNv4_op/src/cuda/flash_deform_attn_cuda.cu:26-84).

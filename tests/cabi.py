@@ -123,3 +123,16 @@ def layer_norm_residual(y, residual, weight, bias, gamma, eps):
         y.data_ptr(), residual.data_ptr() if residual is not None else None, weight.data_ptr(), bias.data_ptr(),
         gamma.data_ptr() if gamma is not None else None, out.data_ptr(), CODES[y.dtype], y.numel() // C, C, float(eps), _stream()))
     return out
+
+
+def dcnv4_backward_static_scratch(value, om, go, geom, G, D, scale, rc=0, softmax=0, im2col_step=256):
+    """The allocation-free entry point: no workspace argument, scratch inside the library."""
+    L = _lib.load()
+    B, H, W, _ = value.shape
+    gv = torch.full_like(value, float("nan"))
+    gom = torch.full_like(om, float("nan"))
+    rc_ = L.dcnv4_gfx950_backward_static_scratch(value.data_ptr(), om.data_ptr(), go.data_ptr(), gv.data_ptr(), gom.data_ptr(),
+                                                 CODES[value.dtype], B, H, W, G, D, *geom, float(scale), im2col_step, rc,
+                                                 om.shape[-1], softmax, 0, 0, _stream())
+    _lib.check(rc_)
+    return gv, gom
