@@ -742,7 +742,6 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
     // every term is grad_out * (probability * bilinear weight <= 1); at most Q * K of them meet in one cell
     // (a term must also stay below 2^51, the conversion's range)
     base.fix_bits = std::min(50, 62 - ceil_log2((int)std::min<long long>((long long)num_query * num_points, 1 << 30)));
-    if (pr.s == 2) base.fix_bits = std::min(base.fix_bits, 30);     // 32-bit conversion path for 16-bit tensors
     hipLaunchKernelGGL(init_state_kernel, dim3(1), dim3(64), 0, st, base.state);
     if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);
     for (int pass = 0; pass < 3; ++pass) {

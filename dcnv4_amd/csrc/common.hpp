@@ -118,9 +118,19 @@ template <typename Tag, int N> struct Pack {
 // source order (dcnv4_im2col_cuda.cuh:203-224, flash_deform_im2col_cuda.cuh:188-189), never
 // fused: a coordinate that differs by one ulp moves every bilinear weight of the tap, which
 // is visible at the fp32 forward tolerance.
-__device__ __forceinline__ float mul_rn(float a, float b) { return __fmul_rn(a, b); }
-__device__ __forceinline__ float add_rn(float a, float b) { return __fadd_rn(a, b); }
-__device__ __forceinline__ float sub_rn(float a, float b) { return __fsub_rn(a, b); }
+// (the pragma keeps the compiler from contracting a product with a later sum into one fma)
+__device__ __forceinline__ float mul_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a * b;
+}
+__device__ __forceinline__ float add_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a + b;
+}
+__device__ __forceinline__ float sub_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a - b;
+}
 
 // ---------------------------------------------------------------- bilinear tap
 // Corner order: (y0,x0) (y0,x0+1) (y0+1,x0) (y0+1,x0+1), as common.h:48-58.

@@ -27,6 +27,8 @@
 //       B      every lane walks its own slot's entries: sum += weight * grad_out row.
 // Integer atomics only order the entries inside a slot; sums depend on that order at the level
 // of fp32 rounding, like the reference's atomics do.
+#include <algorithm>
+
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -42,19 +44,23 @@ template <> struct ParkType<F16> { typedef _Float16 type; };
 
 __device__ __forceinline__ int fdiv_small(int n, float inv) { return (int)(((float)n + 0.5f) * inv); }   // exact for n < 2^20
 
-__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, int lane) {
-#pragma unroll
-  for (int o = 1; o < kWave; o <<= 1) {
-    const uint32_t up = (uint32_t)__shfl_up((int)v, o, kWave);
-    if (lane >= o) v += up;
-  }
+// Inclusive prefix sum over the 64 lanes of a wave with DPP moves: within rows of 16 lanes by shifts, then the last
+// lane of a row is broadcast into the rows after it.  Lanes without a source add 0.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_add(uint32_t v) {
+  return v + (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
+  v = dpp_add<0x111, 0xf>(v);      // row_shr:1
+  v = dpp_add<0x112, 0xf>(v);      // row_shr:2
+  v = dpp_add<0x114, 0xf>(v);      // row_shr:4
+  v = dpp_add<0x118, 0xf>(v);      // row_shr:8
+  v = dpp_add<0x142, 0xa>(v);      // row_bcast:15 into rows 1 and 3
+  v = dpp_add<0x143, 0xc>(v);      // row_bcast:31 into rows 2 and 3
   return v;
 }
-
 __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += (uint32_t)__shfl_xor((int)v, o, kWave);
-  return v;
+  return (uint32_t)__builtin_amdgcn_readlane((int)wave_inclusive_scan(v), kWave - 1);
 }
 
 // CW: channels a lane accumulates (8, 16 or 32): the group width rounded up, or 32 with several lanes per slot.
@@ -100,10 +106,11 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   const int cols_cap = max(1, min(wo_hi_all - wo_lo_all, p.strip_pix));
 
   // this lane's slot: (cell, group of the chunk), and its part of the group's channels
+  const float inv_ng = 1.f / (float)p.ng_chunk;
   const int my_slot = tid >> lps_log2, my_part = tid & ((1 << lps_log2) - 1);
-  const int my_cell = my_slot / p.ng_chunk, my_gl = my_slot - my_cell * p.ng_chunk;
+  const int my_cell = fdiv_small(my_slot, inv_ng), my_gl = my_slot - my_cell * p.ng_chunk;
   const int my_ly = my_cell >> p.tile_w_log2, my_lx = my_cell & (p.tile_w - 1);
-  const bool slot_live = my_ly < th && my_lx < tw && my_gl < ng && my_ly < p.tile_h;
+  const bool slot_live = my_ly < th && my_lx < tw && my_gl < ng;
   float acc[CW];
 #pragma unroll
   for (int c = 0; c < CW; ++c) acc[c] = 0.f;
@@ -111,12 +118,15 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   s_count[tid] = 0u;
   __syncthreads();
 
+  const float x_sub = mul_rn((float)half_w, p.offset_scale), y_sub = mul_rn((float)half_h, p.offset_scale);
+  const float Hf = (float)p.H, Wf = (float)p.W;
+  const elem_t *om_img = reinterpret_cast<const elem_t *>(p.offset_mask) + (size_t)b * p.Q * p.P_pad;
+  const elem_t *go_img = reinterpret_cast<const elem_t *>(p.grad_out) + (size_t)b * p.Q * C;
+  auto load_f = [](const elem_t *ptr) { float f[1]; Pack<Tag, 1>::decode(*ptr, f); return f[0]; };
+  auto to_f = [](elem_t raw) { float f[1]; Pack<Tag, 1>::decode(raw, f); return f[0]; };
+
   for (int wo_lo = wo_lo_all; wo_lo < wo_hi_all && n_rows > 0; wo_lo += cols_cap) {
     const int nwx = min(cols_cap, wo_hi_all - wo_lo);
-    const float x_sub = mul_rn((float)half_w, p.offset_scale), y_sub = mul_rn((float)half_h, p.offset_scale);
-    const elem_t *om_img = reinterpret_cast<const elem_t *>(p.offset_mask) + (size_t)b * p.Q * p.P_pad;
-    const elem_t *go_img = reinterpret_cast<const elem_t *>(p.grad_out) + (size_t)b * p.Q * C;
-    auto load_f = [](const elem_t *ptr) { float f[1]; Pack<Tag, 1>::decode(*ptr, f); return f[0]; };
 
     // strips of interleaved rows: strip s takes rows ho_lo + s, ho_lo + s + n_strips, ...
     const int rows_cap = max(1, p.strip_pix / nwx);
@@ -148,9 +158,100 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
     const int vpp = vec_park ? ng * D / kVec : ng * Dp;                 // vectors (elements) per parked pixel
     const float inv_vpp = 1.f / (float)vpp;
 
+    // a lane's offsets and modulation scalars of a strip, requested one strip ahead (before the previous strip's
+    // phase B) so that their latency hides there
+    elem_t pf_x[ROUNDS], pf_y[ROUNDS], pf_m[ROUNDS];
+    auto prefetch = [&](int s) {
+      const int rows_s = (n_rows - s + n_strips - 1) / n_strips;
+#pragma unroll
+      for (int v = 0; v < ROUNDS; ++v) {
+        pf_x[v] = pf_y[v] = pf_m[v] = elem_t(0);
+        const uint32_t it = item[v];
+        const int r = (int)(it & 0x3ffu), col = (int)((it >> 10) & 0x3ffu), gl = (int)((it >> 20) & 0x3fu), t = (int)(it >> 26);
+        if (it == ~0u || r >= rows_s) continue;
+        const int ho = ho_lo + s + r * n_strips, wo = wo_lo + col;
+        const elem_t *om = om_img + ((uint32_t)(ho * p.Wo + wo) * (uint32_t)p.P_pad + (uint32_t)((g0 + gl) * 3 * Kp));
+        pf_x[v] = om[2 * t]; pf_y[v] = om[2 * t + 1]; pf_m[v] = om[2 * Kp + t];
+      }
+    };
+    prefetch(0);
+
+    // Barriers of a strip: after phase A (counts complete), after scan + park (offsets and grad_out in place), after
+    // place (entries in place).  None after phase B: the next strip's phase A only touches the counters, which phase B
+    // does not read, and everything phase B reads is rewritten only after the next strip's first barrier.
     for (int s = 0; s < n_strips; ++s) {
       const int rows_s = (n_rows - s + n_strips - 1) / n_strips;
       const int npx = rows_s * nwx;
+
+      // ---- phase A: one lane per (group, pixel, tap): corners inside the tile draw a rank in their slot.  A record
+      // (what the lane keeps until the entries are placed): modulation and the two fractions, the slot of the first
+      // corner with the corners that count, and the four ranks.
+      float rec_m[ROUNDS], rec_ly[ROUNDS], rec_lx[ROUNDS];
+      uint32_t rec_slot[ROUNDS], rec_rank[ROUNDS][2];       // first slot (signed, 24 bits) | corners << 24; ranks, 16 bits each
+#pragma unroll
+      for (int v = 0; v < ROUNDS; ++v) {
+        rec_m[v] = rec_ly[v] = rec_lx[v] = 0.f;
+        rec_slot[v] = rec_rank[v][0] = rec_rank[v][1] = 0u;
+        if (v * kValThreads >= n_items) continue;               // uniform
+        const uint32_t it = item[v];
+        const int r = (int)(it & 0x3ffu), col = (int)((it >> 10) & 0x3ffu), gl = (int)((it >> 20) & 0x3fu), t = (int)(it >> 26);
+        if (it == ~0u || r >= rows_s) continue;
+        int ti, tj;
+        if constexpr (KP > 0) {
+          tap_ij_3x3(KP, t, ti, tj);
+        } else {      // x index outer, y index inner, centre skipped when remove_center
+          int tt = t;
+          if (p.remove_center && tt >= (p.kw / 2) * p.kh + p.kh / 2) ++tt;
+          ti = tt / p.kh; tj = tt - ti * p.kh;
+        }
+        const int ho = ho_lo + s + r * n_strips, wo = wo_lo + col;
+        const float off_x = to_f(pf_x[v]), off_y = to_f(pf_y[v]);
+        const float x_base = sub_rn((float)(cx0 + wo * p.sw), x_sub), y_base = sub_rn((float)(cy0 + ho * p.sh), y_sub);
+        const float x = add_rn(x_base, mul_rn(add_rn((float)(ti * p.dw), off_x), p.offset_scale));
+        const float y = add_rn(y_base, mul_rn(add_rn((float)(tj * p.dh), off_y), p.offset_scale));
+        // the reference's range test (dcnv4_col2im_cuda.cuh:317); NaN and huge coordinates fail it
+        if (!((y > -1.f) && (x > -1.f) && (y < Hf) && (x < Wf))) continue;
+        const float fy = floorf(y), fx = floorf(x);
+        // corner 0 relative to the tile; a corner inside the tile is inside the image (the tile is clipped to it)
+        const int ly = (int)fy - ty0, lx = (int)fx - tx0;
+        const bool r0 = (unsigned)ly < (unsigned)th, r1 = (unsigned)(ly + 1) < (unsigned)th;
+        const bool c0 = (unsigned)lx < (unsigned)tw, c1 = (unsigned)(lx + 1) < (unsigned)tw;
+        const uint32_t valid = (uint32_t)(r0 && c0) | ((uint32_t)(r0 && c1) << 1) | ((uint32_t)(r1 && c0) << 2) | ((uint32_t)(r1 && c1) << 3);
+        if (valid == 0) continue;
+        float m = to_f(pf_m[v]);
+        if (p.softmax) {          // rare: normalise over this group's taps
+          const elem_t *om = om_img + ((uint32_t)(ho * p.Wo + wo) * (uint32_t)p.P_pad + (uint32_t)((g0 + gl) * 3 * Kp));
+          float mx = load_f(om + 2 * Kp), sum = 0.f;
+          for (int k = 1; k < Kp; ++k) mx = fmaxf(mx, load_f(om + 2 * Kp + k));
+          for (int k = 0; k < Kp; ++k) sum += __expf(load_f(om + 2 * Kp + k) - mx);
+          m = __expf(m - mx) / sum;
+        }
+        rec_m[v] = m; rec_ly[v] = y - fy; rec_lx[v] = x - fx;
+        const int slot0 = ((ly << p.tile_w_log2) + lx) * p.ng_chunk + gl;      // may be negative: corner block starts outside
+        rec_slot[v] = ((uint32_t)slot0 & 0xffffffu) | (valid << 24);
+        uint32_t ranks[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn) {
+          if (!(valid & (1u << cn))) continue;
+          const int slot = slot0 + (((cn >> 1) << p.tile_w_log2) + (cn & 1)) * p.ng_chunk;
+          ranks[cn] = __hip_atomic_fetch_add(&s_count[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+        rec_rank[v][0] = ranks[0] | (ranks[1] << 16);
+        rec_rank[v][1] = ranks[2] | (ranks[3] << 16);
+        __builtin_amdgcn_sched_barrier(0);      // one round at a time: interleaved, the rounds' temporaries spill
+      }
+      __syncthreads();
+
+      // ---- scan: exclusive prefix sum of the slot counts (a wave adds up the counts of the waves before it itself)
+      {
+        const uint32_t c = s_count[tid];
+        const uint32_t incl = wave_inclusive_scan(c);
+        uint32_t before = 0;
+        for (int w = 0; w < wave; ++w) before += s_count[w * kWave + lane];
+        before = wave_sum(before);
+        s_offs[tid] = before + incl - c;
+        if (tid == kValThreads - 1) s_offs[kValThreads] = before + incl;
+      }
 
       // ---- park the strip's grad_out (this chunk's channels)
       for (int idx = tid; idx < npx * vpp; idx += kValThreads) {
@@ -175,74 +276,6 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
           reinterpret_cast<park_t *>(dst)[u] = (park_t)f;
         }
       }
-
-      // ---- phase A: one lane per (group, pixel, tap): corners inside the tile draw a rank in their slot.  A record
-      // (what the lane keeps until the entries are placed): modulation and the two fractions, the slot of the first
-      // corner with the corners that count, and the four ranks.
-      float rec_m[ROUNDS], rec_ly[ROUNDS], rec_lx[ROUNDS];
-      uint32_t rec_slot[ROUNDS], rec_rank[ROUNDS][2];       // first slot (signed, 24 bits) | corners << 24; ranks, 16 bits each
-#pragma unroll
-      for (int v = 0; v < ROUNDS; ++v) {
-        rec_m[v] = rec_ly[v] = rec_lx[v] = 0.f;
-        rec_slot[v] = rec_rank[v][0] = rec_rank[v][1] = 0u;
-        if (v * kValThreads >= n_items) continue;               // uniform
-        const uint32_t it = item[v];
-        const int r = (int)(it & 0x3ffu), col = (int)((it >> 10) & 0x3ffu), gl = (int)((it >> 20) & 0x3fu), t = (int)(it >> 26);
-        if (it == ~0u || r >= rows_s) continue;
-        int ti, tj;
-        if constexpr (KP > 0) {
-          tap_ij_3x3(KP, t, ti, tj);
-        } else {      // x index outer, y index inner, centre skipped when remove_center
-          int tt = t;
-          if (p.remove_center && tt >= (p.kw / 2) * p.kh + p.kh / 2) ++tt;
-          ti = tt / p.kh; tj = tt - ti * p.kh;
-        }
-        const int ho = ho_lo + s + r * n_strips, wo = wo_lo + col;
-        const elem_t *om = om_img + ((uint32_t)(ho * p.Wo + wo) * (uint32_t)p.P_pad + (uint32_t)((g0 + gl) * 3 * Kp));
-        const float off_x = load_f(om + 2 * t), off_y = load_f(om + 2 * t + 1);
-        const float x_base = sub_rn((float)(cx0 + wo * p.sw), x_sub), y_base = sub_rn((float)(cy0 + ho * p.sh), y_sub);
-        const float x = add_rn(x_base, mul_rn(add_rn((float)(ti * p.dw), off_x), p.offset_scale));
-        const float y = add_rn(y_base, mul_rn(add_rn((float)(tj * p.dh), off_y), p.offset_scale));
-        const Tap tp = make_tap(y, x, p.H, p.W, 0u, 0u);
-        const int ly = tp.y0 - ty0, lx = tp.x0 - tx0;
-        const bool r0 = ly >= 0 && ly < th, r1 = ly + 1 >= 0 && ly + 1 < th;
-        const bool c0 = lx >= 0 && lx < tw, c1 = lx + 1 >= 0 && lx + 1 < tw;
-        const uint32_t valid = tp.valid & ((uint32_t)(r0 && c0) | ((uint32_t)(r0 && c1) << 1) |
-                                           ((uint32_t)(r1 && c0) << 2) | ((uint32_t)(r1 && c1) << 3));
-        if (valid == 0) continue;
-        float m = load_f(om + 2 * Kp + t);
-        if (p.softmax) {          // rare: normalise over this group's taps
-          float mx = load_f(om + 2 * Kp), sum = 0.f;
-          for (int k = 1; k < Kp; ++k) mx = fmaxf(mx, load_f(om + 2 * Kp + k));
-          for (int k = 0; k < Kp; ++k) sum += __expf(load_f(om + 2 * Kp + k) - mx);
-          m = __expf(m - mx) / sum;
-        }
-        rec_m[v] = m; rec_ly[v] = tp.ly; rec_lx[v] = tp.lx;
-        const int slot0 = ((ly << p.tile_w_log2) + lx) * p.ng_chunk + gl;      // may be negative: corner block starts outside
-        rec_slot[v] = ((uint32_t)slot0 & 0xffffffu) | (valid << 24);
-        uint32_t ranks[4] = {0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int cn = 0; cn < 4; ++cn) {
-          if (!(valid & (1u << cn))) continue;
-          const int slot = slot0 + (((cn >> 1) << p.tile_w_log2) + (cn & 1)) * p.ng_chunk;
-          ranks[cn] = __hip_atomic_fetch_add(&s_count[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        }
-        rec_rank[v][0] = ranks[0] | (ranks[1] << 16);
-        rec_rank[v][1] = ranks[2] | (ranks[3] << 16);
-        __builtin_amdgcn_sched_barrier(0);      // one round at a time: interleaved, the rounds' temporaries spill
-      }
-      __syncthreads();
-
-      // ---- scan: exclusive prefix sum of the slot counts (a wave adds up the counts of the waves before it itself)
-      {
-        const uint32_t c = s_count[tid];
-        const uint32_t incl = wave_inclusive_scan(c, lane);
-        uint32_t before = 0;
-        for (int w = 0; w < wave; ++w) before += s_count[w * kWave + lane];
-        before = wave_sum(before);
-        s_offs[tid] = before + incl - c;
-        if (tid == kValThreads - 1) s_offs[kValThreads] = before + incl;
-      }
       __syncthreads();
 
       // ---- place: the entries, sorted by slot
@@ -257,7 +290,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
         const int px = (int)(it & 0x3ffu) * nwx + (int)((it >> 10) & 0x3ffu), gl = (int)((it >> 20) & 0x3fu);
         const uint32_t go_addr = (uint32_t)(px * go_stride + gl * Dp * kParkBytes);
         const float m = rec_m[v], ly = rec_ly[v], lx = rec_lx[v], hy = 1.f - ly, hx = 1.f - lx;
-        const float wv[4] = {m * (hy * hx), m * (hy * lx), m * (ly * hx), m * (ly * lx)};     // as make_tap forms them
+        const float wv[4] = {m * (hy * hx), m * (hy * lx), m * (ly * hx), m * (ly * lx)};     // common.h:48-58, 153-184
         const uint32_t ranks[4] = {rec_rank[v][0] & 0xffffu, rec_rank[v][0] >> 16, rec_rank[v][1] & 0xffffu, rec_rank[v][1] >> 16};
 #pragma unroll
         for (int cn = 0; cn < 4; ++cn) {
@@ -266,50 +299,67 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
           s_entry[s_offs[slot] + ranks[cn]] = u32x2{__builtin_bit_cast(uint32_t, wv[cn]), go_addr};
         }
       }
+      if (s + 1 < n_strips) prefetch(s + 1);
       __syncthreads();
 
-      // ---- phase B: every lane sums its slot's entries
+      // ---- phase B: every lane sums its slot's entries; the next entry is read while the current one is applied
       if (slot_live) {
-        const uint32_t beg = s_offs[my_slot], end = s_offs[my_slot + 1];
+        uint32_t e = s_offs[my_slot];
+        const uint32_t end = s_offs[my_slot + 1];
         const char *go_lane = s_go + my_part * kLaneBytes;
-        for (uint32_t e = beg; e < end; ++e) {
-          const u32x2 ent = s_entry[e];
+        u32x2 ent = s_entry[e];                                  // (one entry past the last is inside the allocation)
+        while (e < end) {
+          const u32x2 next = s_entry[++e];
           const float w = __builtin_bit_cast(float, ent.x);
-          const park_t *g = reinterpret_cast<const park_t *>(go_lane + ent.y);
+          const char *g = go_lane + ent.y;
           park_t gv[CW];
 #pragma unroll
           for (int q = 0; q < kLaneBytes / 16; ++q)
-            *reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(gv) + 16 * q) = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(g) + 16 * q);
+            *reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(gv) + 16 * q) = *reinterpret_cast<const u32x4 *>(g + 16 * q);
 #pragma unroll
           for (int c = 0; c < CW; ++c) acc[c] = fmaf(w, (float)gv[c], acc[c]);
+          ent = next;
         }
       }
-      __syncthreads();      // the parked rows, the entries and the offsets are replaced next
     }
   }
+  __syncthreads();      // the last phase B is over: LDS is free
 
-  // the tile is complete: registers -> tensor dtype, plain stores
-  if (slot_live) {
-    const int ch0 = my_part * CW;                              // first channel of this lane within its group
+  // The tile is complete: registers -> tensor dtype -> memory.  Whole 16-byte pieces go through LDS so that the lanes
+  // of a store instruction cover consecutive pieces of a (cell, group) instead of one piece of 64 different ones.
+  constexpr int kVecOut = 16 / Tag::kBytes;
+  if (D % kVecOut == 0) {
+    constexpr int kPieces = CW / kVecOut;                       // 16-byte pieces a lane holds
+    u32x4 *s_out = reinterpret_cast<u32x4 *>(lds32);
+#pragma unroll
+    for (int q = 0; q < kPieces; ++q) {
+      float f[kVecOut];
+#pragma unroll
+      for (int i = 0; i < kVecOut; ++i) f[i] = acc[q * kVecOut + i];
+      s_out[tid * kPieces + q] = Pack<Tag, kVecOut>::encode(f);
+    }
+    __syncthreads();
+    elem_t *gv_img = reinterpret_cast<elem_t *>(p.grad_value) + (size_t)b * p.H * p.W * C;
+#pragma unroll
+    for (int k = 0; k < kPieces; ++k) {
+      const int idx = k * kValThreads + tid;
+      const int src = idx / kPieces, q = idx - src * kPieces;   // the lane that held this piece, and which of its pieces
+      const int slot = src >> lps_log2, part = src & ((1 << lps_log2) - 1);
+      const int cell = fdiv_small(slot, inv_ng), gl = slot - cell * p.ng_chunk;
+      const int cy = cell >> p.tile_w_log2, cx = cell & (p.tile_w - 1);
+      const int ch = part * CW + q * kVecOut;                   // first channel of the piece within its group
+      if (cy < th && cx < tw && gl < ng && ch < D)
+        *reinterpret_cast<u32x4 *>(gv_img + ((size_t)((ty0 + cy) * p.W + tx0 + cx) * C + (g0 + gl) * D + ch)) = s_out[idx];
+    }
+  } else if (slot_live) {
+    const int ch0 = my_part * CW;
     elem_t *dst = reinterpret_cast<elem_t *>(p.grad_value) +
                   ((((size_t)b * p.H + ty0 + my_ly) * p.W + tx0 + my_lx) * C + (g0 + my_gl) * D + ch0);
-    constexpr int kVec = 16 / Tag::kBytes;
-    if (D % kVec == 0) {
 #pragma unroll
-      for (int q = 0; q < CW / kVec; ++q) {
-        if (ch0 + q * kVec >= D) break;
-        float f[kVec];
-#pragma unroll
-        for (int i = 0; i < kVec; ++i) f[i] = acc[q * kVec + i];
-        *reinterpret_cast<typename Pack<Tag, kVec>::raw_t *>(dst + q * kVec) = Pack<Tag, kVec>::encode(f);
-      }
-    } else {
-#pragma unroll
-      for (int c = 0; c < CW; ++c) {
-        if (ch0 + c < D) {
-          const float f[1] = {acc[c]};
-          dst[c] = Pack<Tag, 1>::encode(f);
-        }
+    for (int c = 0; c < CW; ++c) {
+      if (ch0 + c < D) {
+        const float f[1] = {acc[c]};
+        dst[c] = Pack<Tag, 1>::encode(f);
       }
     }
   }
@@ -343,7 +393,10 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
 
 size_t dcnv4_grad_value_lds_bytes(const DcnLaunch &p) {
   const size_t items = (size_t)p.strip_pix * p.Kp * p.ng_chunk;
-  return (2 * kValThreads + 4) * sizeof(uint32_t) + (size_t)p.strip_pix * p.gv_go_stride + items * 4 * sizeof(u32x2);
+  // counters and offsets, parked grad_out, entries (+ the one the read-ahead of phase B touches); at the end the
+  // finished tile is staged over all of it: at most 4 bytes per channel and lane
+  const size_t strip = (2 * kValThreads + 4) * sizeof(uint32_t) + (size_t)p.strip_pix * p.gv_go_stride + (items * 4 + 2) * sizeof(u32x2);
+  return std::max(strip, (size_t)kValThreads * p.gv_cw * 4);
 }
 
 hipError_t launch_dcnv4_grad_value(int dtype, const DcnLaunch &p, hipStream_t stream) {

@@ -230,6 +230,23 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
   const int n_tiles = s_first[p.L];
   const int BG = p.n_img * p.G;
 
+  // value rows that no level covers (spatial_size beyond the levels, gaps between them) get zeros, like the
+  // reference's zeros_like(value) (flash_deform_attn_cuda.cu:118)
+  {
+    typedef typename RawWord<Tag::kBytes>::type elem0_t;
+    const long long rows = (long long)p.n_img * p.N;
+    const int row_elems = p.G * p.D;
+    for (long long r = (long long)blockIdx.x * kApplyThreads + tid; r < rows; r += (long long)gridDim.x * kApplyThreads) {
+      const int n = (int)(r % p.N);
+      bool covered = false;
+      for (int l = 0; l < p.L; ++l) covered |= n >= s_plan[l].start && n < s_plan[l].start + s_plan[l].H * s_plan[l].W;
+      if (!covered) {
+        elem0_t *row = reinterpret_cast<elem0_t *>(p.grad_value) + (size_t)r * row_elems;
+        for (int i = 0; i < row_elems; ++i) row[i] = elem0_t(0);
+      }
+    }
+  }
+
   const uint32_t gmax = p.state->go_max_bits;
   const bool usable = gmax < 0x7f800000u && gmax != 0u && p.state->reserved == 0u;
   const int e_go = (int)(gmax >> 23) - 126;                  // 2^e_go > max |grad_out|
@@ -363,21 +380,13 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
 #pragma unroll
           for (int cn = 0; cn < 4; ++cn) {
             unsigned long long *dst = acc + __umul24(cells[cn], (uint32_t)DP) + c;
-            if constexpr (Tag::kBytes == 4) {
-              const double wd = (double)wv[cn];
+            // the same resolution for every tensor dtype: small gradients next to large ones (loss scaling) keep
+            // their bits, as they do when the reference sums in fp32
+            const double wd = (double)wv[cn];
 #pragma unroll
-              for (int j = 0; j < CPL; ++j)
-                __hip_atomic_fetch_add(dst + slot_off[j], fixed_product((double)gn[j], wd), __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_WORKGROUP);
-            } else {
-              // 16-bit tensors carry 8-11 significant bits: terms below 2^31 (fix_bits <= 30), truncated
-#pragma unroll
-              for (int j = 0; j < CPL; ++j) {
-                const int t = (int)(gn[j] * wv[cn]);
-                __hip_atomic_fetch_add(dst + slot_off[j], ((unsigned long long)(uint32_t)(t >> 31) << 32) | (uint32_t)t,
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-              }
-            }
+            for (int j = 0; j < CPL; ++j)
+              __hip_atomic_fetch_add(dst + slot_off[j], fixed_product((double)gn[j], wd), __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_WORKGROUP);
           }
         }
         if (nb_next > 0) park(nxt, nb_next, buf ^ 1);
@@ -441,7 +450,8 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
       const unsigned long long a = acc[cell * DP + ch / CPL + kRowLanes * (ch % CPL)];
       const double v = ldexp((double)(int)(a >> 32) * 4294967296.0 + (double)(uint32_t)a, e_out);
       const float f[1] = {(float)v};
-      gv[(((size_t)b * p.N + lp.start + (size_t)(ty0 + cy) * lp.W + tx0 + cx) * p.G + g) * D + ch] = Pack<Tag, 1>::encode(f);
+      const long long n = (long long)lp.start + (long long)(ty0 + cy) * lp.W + tx0 + cx;      // level tables are not validated
+      if (n >= 0 && n < p.N) gv[(((size_t)b * p.N + (size_t)n) * p.G + g) * D + ch] = Pack<Tag, 1>::encode(f);
     }
     __syncthreads();
   }

@@ -597,3 +597,65 @@ def test_block_tail_at_the_model_stage_one_size_normalises_every_row():
     gamma = torch.full((112,), 0.5, device="cuda").half()
     both = ext.layer_norm_residual_forward(y, res, ones, zeros, gamma, 1e-6).float()
     assert (both - (res.float() + 0.5 * out)).abs().max().item() < 4e-3
+
+
+def test_flash_deform_attn_adjoint_identity_at_full_benchmark_size_in_fp16():
+    """The attention benchmark configuration in fp16: <g, f(v)> = <grad_value, v> (the operator is linear in value)."""
+    torch.manual_seed(6)
+    shapes = [(128, 128), (64, 64), (32, 32), (16, 16)]
+    B, G, D, L, K = 4, 8, 32, 4, 4
+    N = sum(h * w for h, w in shapes)
+    dev = "cuda"
+    shp = torch.tensor(shapes, device=dev)
+    sizes = [h * w for h, w in shapes]
+    st = torch.tensor([sum(sizes[:i]) for i in range(L)], device=dev)
+    v = torch.randn(B, N, G, D, device=dev).half()
+    sla = torch.cat([torch.rand(B, N, G, L * K * 2, device=dev), torch.randn(B, N, G, L * K, device=dev)], -1).half()
+    g = torch.randn(B, N, G * D, device=dev).half()
+    out = cabi.fda_forward(v, shp, st, sla, K)
+    gv, gs = cabi.fda_backward(v, shp, st, sla, g, K)
+    lhs = (g.double() * out.double()).sum()
+    rhs = (gv.double() * v.double()).sum()
+    scale = (g.double().abs() * out.double().abs()).sum()
+    assert abs(float(lhs - rhs)) / float(scale) < 1e-3          # outputs and gradients rounded to fp16
+    assert float(gs[..., 2 * L * K:].double().sum(-1).abs().max()) < 2e-2
+
+
+def test_flash_intern_image_b_in_fp16_matches_the_same_weights_on_the_torch_core(monkeypatch):
+    """The whole FlashInternImage-B (33 DCNv4 layers, groups 7 / 14 / 28 / 56) in fp16 at batch 8 against the same,
+    fp16-rounded weights evaluated in fp32 on the CPU with the operators swapped for torch formulations.  Offsets and
+    layer scales are made non-trivial first: at their initial values (zero offsets, 1e-5) the operator would hardly
+    show in the logits."""
+    import copy
+    from dcnv4_amd.models import flash_intern_image
+    from dcnv4_amd.modules import dcnv4 as dcnv4_module
+
+    torch.manual_seed(3)
+    model = flash_intern_image("b").eval()
+    with torch.no_grad():
+        for m in model.modules():
+            if isinstance(m, dcnv4_module.DCNv4):
+                m.offset_mask.weight.normal_(0, 0.02)
+                m.offset_mask.bias.normal_(0, 0.7)
+        for name, prm in model.named_parameters():
+            if name.endswith("gamma1") or name.endswith("gamma2"):
+                prm.fill_(0.2)
+    x = torch.randn(8, 3, 224, 224)
+    half = copy.deepcopy(model).half().cuda()
+    with torch.no_grad():
+        got = half(x.half().cuda()).float().cpu()
+    ref = copy.deepcopy(model)
+    ref.load_state_dict({k: v.float().cpu() for k, v in half.state_dict().items()})      # the fp16-rounded weights
+
+    class CoreOnCpu:
+        @staticmethod
+        def apply(inp, om, kh, kw_, sh, sw, ph, pw, dh, dw, group, group_channels, offset_scale, im2col_step, remove_center):
+            return torch_core.dcnv4_core_torch(inp, om, kh, kw_, sh, sw, ph, pw, dh, dw, group, group_channels,
+                                               offset_scale, remove_center)
+
+    monkeypatch.setattr(dcnv4_module, "DCNv4Function", CoreOnCpu)
+    monkeypatch.setattr(dcnv4_module, "DepthwiseConvNHWCFunction", DepthwiseOnCpu)
+    with torch.no_grad():
+        want = ref(x.half().float())
+    assert got.shape == (8, 1000) and torch.isfinite(got).all()
+    assert _rel_err(got, want) < 3e-2
