@@ -660,14 +660,14 @@ int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_s
   return DCNV4_OK;
 }
 
-// Scratch of the tiled attention backward, in this order: GradState, keys, probabilities, tile table, sorted
-// point lists.  The last two are sized for the images of one launch and reused by the next.
+// Scratch of the tiled attention backward, in this order: GradState, keys, point records, grad_out regrouped by head,
+// tile table, sorted point lists.  The last two are sized for the images of one launch and reused by the next.
 struct FdaScratch {
-  size_t keys, probs, table, regions, total;     // byte offsets, total bytes
+  size_t keys, recs, go_rows, table, regions, total;     // byte offsets, total bytes
   int n_chunks, tile_stride, per;
 };
 
-FdaScratch fda_scratch(int batch, int N, int G, int D, int L, int Q, int K) {
+FdaScratch fda_scratch(int s, int batch, int N, int G, int D, int L, int Q, int K) {
   FdaScratch sc;
   const uint64_t per_img = (uint64_t)N * G * D * 4;
   uint64_t per = std::max<uint64_t>(1, kMaxSpanBytes / per_img);
@@ -679,8 +679,9 @@ FdaScratch fda_scratch(int batch, int N, int G, int D, int L, int Q, int K) {
   sc.tile_stride = (int)std::min<size_t>(kFdaMaxTilesPerLevel, (size_t)N / 8 + 64);
   const size_t segs = (size_t)sc.per * G * L * sc.n_chunks;
   sc.keys = kStateBytes;
-  sc.probs = sc.keys + round16((size_t)batch * points * sizeof(uint16_t));
-  sc.table = sc.probs + round16((size_t)batch * points * sizeof(float));
+  sc.recs = sc.keys + round16((size_t)batch * points * sizeof(uint16_t));
+  sc.go_rows = sc.recs + round16((size_t)batch * points * 16);
+  sc.table = sc.go_rows + round16((size_t)batch * G * Q * D * s);
   sc.regions = sc.table + round16(segs * sc.tile_stride * sizeof(uint32_t));
   sc.total = sc.regions + round16(segs * 4 * kFdaChunkPoints * sizeof(uint32_t));
   return sc;
@@ -693,7 +694,7 @@ size_t flash_deform_attn_gfx950_backward_workspace_bytes(int dtype, int batch, i
   size_t need = 0;
   if (elem_bytes(dtype) == 2) need = round16((size_t)batch * spatial_size * num_heads * head_channels * sizeof(float));
   if (fda_tiled_shape(head_channels, num_levels, num_query, num_points))
-    need = std::max(need, fda_scratch(batch, spatial_size, num_heads, head_channels, num_levels, num_query, num_points).total);
+    need = std::max(need, fda_scratch(elem_bytes(dtype), batch, spatial_size, num_heads, head_channels, num_levels, num_query, num_points).total);
   return need;
 }
 
@@ -727,21 +728,19 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
   const int per = images_per_launch(pr, true);      // equals FdaScratch::per
 
   if (tiled) {
-    // pass 0: grad_sampling_loc_attn, keys and max |grad_out|; pass 1: tiled grad_value; pass 2: fallback
+    // pass 0: grad_sampling_loc_attn, keys, point records, regrouped grad_out; pass 1: tiled grad_value; pass 2: fallback
     FdaLaunch base = pr.launch;
     base.state = static_cast<GradState *>(workspace);
-    const FdaScratch sc = fda_scratch(batch, spatial_size, num_heads, head_channels, num_levels, num_query, num_points);
+    const FdaScratch sc = fda_scratch(pr.s, batch, spatial_size, num_heads, head_channels, num_levels, num_query, num_points);
     const size_t img_keys = (size_t)num_heads * num_levels * fda_key_stride(num_query, num_points);
     char *ws = static_cast<char *>(workspace);
     uint16_t *keys = reinterpret_cast<uint16_t *>(ws + sc.keys);
-    float *probs = reinterpret_cast<float *>(ws + sc.probs);
+    f32x4_t *recs = reinterpret_cast<f32x4_t *>(ws + sc.recs);
+    char *go_rows = ws + sc.go_rows;
     base.table = reinterpret_cast<uint32_t *>(ws + sc.table);
     base.regions = reinterpret_cast<uint32_t *>(ws + sc.regions);
     base.n_chunks = sc.n_chunks;
     base.tile_stride = sc.tile_stride;
-    // every term is grad_out * (probability * bilinear weight <= 1); at most Q * K of them meet in one cell
-    // (a term must also stay below 2^51, the conversion's range)
-    base.fix_bits = std::min(50, 62 - ceil_log2((int)std::min<long long>((long long)num_query * num_points, 1 << 30)));
     hipLaunchKernelGGL(init_state_kernel, dim3(1), dim3(64), 0, st, base.state);
     if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);
     for (int pass = 0; pass < 3; ++pass) {
@@ -754,7 +753,8 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
         F.grad_value = at(grad_value, b0 * pr.img_elems, pr.s);
         F.grad_sla = at(grad_sampling_loc_attn, b0 * pr.img_row_elems, pr.s);
         F.keys = keys + b0 * img_keys;
-        F.probs = probs + b0 * img_keys;
+        F.recs = recs + b0 * img_keys;
+        F.go_rows = go_rows + (size_t)b0 * pr.img_out_elems * pr.s;
         F.shapes = spatial_shapes;
         F.level_start = level_start_index;
         F.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);

@@ -66,7 +66,7 @@ __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
 // CW: channels a lane accumulates (8, 16 or 32): the group width rounded up, or 32 with several lanes per slot.
 template <typename Tag, int KP, int CW, int ROUNDS>
 __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const DcnLaunch p) {
-  extern __shared__ uint32_t lds32[];
+  extern __shared__ __align__(16) uint32_t lds32[];
   typedef typename ParkType<Tag>::type park_t;
   typedef typename RawWord<Tag::kBytes>::type elem_t;
   constexpr int kParkBytes = sizeof(park_t);
@@ -310,7 +310,8 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
         u32x2 ent = s_entry[e];                                  // (one entry past the last is inside the allocation)
         while (e < end) {
           const u32x2 next = s_entry[++e];
-          const float w = __builtin_bit_cast(float, ent.x);
+          const uint32_t w_bits = ent.x;
+          const float w = __builtin_bit_cast(float, w_bits);
           const char *g = go_lane + ent.y;
           park_t gv[CW];
 #pragma unroll

@@ -42,13 +42,11 @@ namespace {
 
 constexpr int kBinThreads = 1024;
 constexpr int kBinWordsPerLane = kFdaChunkPoints / 2 / kBinThreads;      // dwords of two keys per lane: 4
-constexpr int kApplyThreads = 512;
-constexpr int kRowLanes = 8;                 // lanes that apply one listed point
-constexpr int kBatch = 128;                  // listed points applied between two barriers
-constexpr int kListCap = 1024;               // listed points held in LDS at a time
+constexpr int kBatch = 256;                  // listed points per batch: one per lane of the first four waves
+constexpr int kListCap = 1024;               // listed point ids held in LDS at a time
 constexpr int kTabCap = 256;                 // chunk table entries held in LDS at a time
-constexpr int kCellBitsF = 7;                // tiles have at most 64 cells; cell 64.. = trash
-constexpr int kTileCells = 64;
+constexpr int kTileCells = 64;               // tiles have at most 8 x 8 cells
+constexpr int kSubLists = 1;                 // sub-lists (groups of lanes) every cell has at least; small tiles get more
 
 struct LevelPlan {
   int H, W, start;
@@ -200,19 +198,44 @@ __global__ void __launch_bounds__(kBinThreads) fda_bin_points_kernel(const FdaLa
 }
 
 // ------------------------------------------------------------------------------- accumulation
-template <typename Tag, int CPL>
-__global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const FdaLaunch p) {
-  extern __shared__ unsigned long long lds64[];
+// Inclusive prefix sum over a wave with DPP moves (rows of 16 lanes by shifts, then row broadcasts).
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_add(uint32_t v) {
+  return v + (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
+  v = dpp_add<0x111, 0xf>(v);      // row_shr:1
+  v = dpp_add<0x112, 0xf>(v);      // row_shr:2
+  v = dpp_add<0x114, 0xf>(v);      // row_shr:4
+  v = dpp_add<0x118, 0xf>(v);      // row_shr:8
+  v = dpp_add<0x142, 0xa>(v);      // row_bcast:15 into rows 1 and 3
+  v = dpp_add<0x143, 0xc>(v);      // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
+// CW: channels a lane accumulates (at most 16 bytes of the tensor dtype); LPC lanes (4 or 8) share a cell, so a cell
+// holds DP = LPC * CW channels (the head width rounded up to 8, 16 or 32).  A workgroup has one lane per (cell, part):
+// 64 * LPC lanes.  grad_out rows are parked in LDS in the tensor dtype.
+template <typename Tag, int CW, int LPC, int SUBS>
+__global__ void __launch_bounds__(kTileCells * LPC * SUBS) fda_grad_value_kernel(const FdaLaunch p) {
+  extern __shared__ __align__(16) uint32_t lds32[];      // 16-byte aligned behind the static arrays: LDS stalls on 8- and 16-byte accesses that are not
   typedef typename RawWord<Tag::kBytes>::type elem_t;
-  constexpr int DP = CPL * kRowLanes;                         // accumulator channels per cell (D rounded up)
+  constexpr int kSlots = kTileCells * SUBS;                   // every cell has at least SUBS sub-lists
+  constexpr int kApplyThreads = kSlots * LPC;
+  static_assert(kBatch <= kApplyThreads && (kBatch * LPC) % kApplyThreads == 0, "a lane per point, whole rows per lane");
+  constexpr int kCellLanes = LPC;
+  constexpr int kCellLanesLog2 = LPC == 8 ? 3 : 2;
+  constexpr int DP = CW * kCellLanes;
+  constexpr int kParkBytes = Tag::kBytes;
+  constexpr int kGoStride = (((DP * kParkBytes + 15) / 16) | 1) * 16;     // an odd number of 16-byte units per parked row
   const int D = p.D, LK = p.L * p.K, QK = p.Q * p.K;
-  unsigned long long *acc = lds64;                            // [(kTileCells + 1) * DP], last cell = trash
-  constexpr int n_acc = (kTileCells + 1) * DP;
-  f32x4 *rec_w = reinterpret_cast<f32x4 *>(lds64 + n_acc);    // [2][kBatch]: one batch is applied while the next is prepared
-  uint32_t *rec_meta = reinterpret_cast<uint32_t *>(rec_w + 2 * kBatch);   // [2][kBatch] four 7-bit cells
-  uint32_t *s_list = rec_meta + 2 * kBatch;                   // [kListCap]
+  uint32_t *s_count = lds32;                                  // [kTileCells] entries per cell in this batch
+  uint32_t *s_offs = s_count + kTileCells;                    // [kTileCells + 4] first entry of every cell, then the total
+  uint32_t *s_list = s_offs + kTileCells + 4;                 // [kListCap] listed point ids
   uint32_t *s_tab = s_list + kListCap;                        // [kTabCap] (offset | count << 16) of the item's tile per chunk
-  uint32_t *s_pre = s_tab + kTabCap;                          // [kTabCap + 1] exclusive prefix of the counts
+  uint32_t *s_pre = s_tab + kTabCap;                          // [kTabCap + 4] exclusive prefix of the counts
+  u32x2 *s_entry = reinterpret_cast<u32x2 *>(s_pre + kTabCap + 4);      // [4 * kBatch + 2] (weight, parked row), sorted by cell
+  char *s_go = reinterpret_cast<char *>(s_entry + 4 * kBatch + 2);      // [kBatch + 1] parked grad_out rows of the batch, then a row of zeros
   __shared__ LevelPlan s_plan[kMaxLevels];
   __shared__ int s_first[kMaxLevels + 1];                     // rank of each level's first tile in the walk
 
@@ -226,6 +249,8 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
     }
     s_first[p.L] = rank;                                      // total
   }
+  if (tid < kTileCells) s_count[tid] = 0u;
+  if (tid < kGoStride / 4) reinterpret_cast<uint32_t *>(s_go + kBatch * kGoStride)[tid] = 0u;      // the row of zeros
   __syncthreads();
   const int n_tiles = s_first[p.L];
   const int BG = p.n_img * p.G;
@@ -233,7 +258,6 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
   // value rows that no level covers (spatial_size beyond the levels, gaps between them) get zeros, like the
   // reference's zeros_like(value) (flash_deform_attn_cuda.cu:118)
   {
-    typedef typename RawWord<Tag::kBytes>::type elem0_t;
     const long long rows = (long long)p.n_img * p.N;
     const int row_elems = p.G * p.D;
     for (long long r = (long long)blockIdx.x * kApplyThreads + tid; r < rows; r += (long long)gridDim.x * kApplyThreads) {
@@ -241,20 +265,35 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
       bool covered = false;
       for (int l = 0; l < p.L; ++l) covered |= n >= s_plan[l].start && n < s_plan[l].start + s_plan[l].H * s_plan[l].W;
       if (!covered) {
-        elem0_t *row = reinterpret_cast<elem0_t *>(p.grad_value) + (size_t)r * row_elems;
-        for (int i = 0; i < row_elems; ++i) row[i] = elem0_t(0);
+        elem_t *row = reinterpret_cast<elem_t *>(p.grad_value) + (size_t)r * row_elems;
+        for (int i = 0; i < row_elems; ++i) row[i] = elem_t(0);
       }
     }
   }
 
-  const uint32_t gmax = p.state->go_max_bits;
-  const bool usable = gmax < 0x7f800000u && gmax != 0u && p.state->reserved == 0u;
-  const int e_go = (int)(gmax >> 23) - 126;                  // 2^e_go > max |grad_out|
-  const int e_out = e_go - p.fix_bits;
+  const bool usable = p.state->reserved == 0u;               // else the atomic fallback kernel adds everything
   const size_t QKp = fda_key_stride(p.Q, p.K);
+  const int my_slot = tid >> kCellLanesLog2, my_part = tid & (kCellLanes - 1);      // slot: (cell, sub-list), 64 of them
 
-  for (int item = blockIdx.x; item < n_tiles * BG; item += gridDim.x) {
-    const int rank = item / BG, bg = item - rank * BG;
+  // Item order.  The hardware deals consecutive workgroup ids to the 8 XCDs in turn.  When the (image, head) pairs
+  // divide evenly among them, an XCD works through its pairs one after the other, and through a pair level by level
+  // (coarsest first): the pair's regrouped grad_out rows and the level's point records and lists - a few MB - then
+  // stay in that XCD's L2 while its points are gathered.  Otherwise tiles are dealt over everything, in the same
+  // level order.
+  const bool by_pair = BG % kXcds == 0 && (int)gridDim.x % kXcds == 0;
+  const int n_items = n_tiles * BG;
+  const int xcd = blockIdx.x % kXcds, wg_in_xcd = blockIdx.x / kXcds, wgs_per_xcd = gridDim.x / kXcds;
+  const int items_per_xcd = n_items / kXcds;
+  for (int it = by_pair ? wg_in_xcd : (int)blockIdx.x; it < (by_pair ? items_per_xcd : n_items); it += by_pair ? wgs_per_xcd : (int)gridDim.x) {
+    int rank, bg;
+    if (by_pair) {
+      const int j = it / n_tiles;                             // the XCD's j-th pair
+      rank = it - j * n_tiles;
+      bg = j * kXcds + xcd;
+    } else {
+      rank = it / BG;
+      bg = it - rank * BG;
+    }
     const int b = bg / p.G, g = bg - b * p.G;
     int l = 0;
     for (int i = 0; i < p.L; ++i)       // first ranks fall with the level index: the first level whose rank fits
@@ -264,136 +303,142 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
     const int ty = t_in / lp.ntx, tx = t_in - ty * lp.ntx;
     const int ty0 = ty * lp.th, tx0 = tx * lp.tw;
     const int th = min(lp.th, lp.H - ty0), tw = min(lp.tw, lp.W - tx0);
-    const int n_cells = th * tw;                             // <= 64; cell n_cells.. = trash
+    const int n_cells = th * tw;                             // <= 64
+    // A tile of few cells gives every cell several lanes: cells rounded up to a power of two, 64 / that many sub-lists
+    // per cell; lane (cell, sub) takes the cell's entries sub, sub + n_sub, ...; the partial sums meet at the end.
+    int cells_log2 = 0;
+    while ((1 << cells_log2) < n_cells) ++cells_log2;
+    const int n_sub = kSlots >> cells_log2;
+    const int my_cell = my_slot & ((1 << cells_log2) - 1), my_sub = my_slot >> cells_log2;
     const int seg = bg * p.L + l;
+    const float Hf = (float)lp.H, Wf = (float)lp.W;
 
-    for (int i = tid; i < n_acc; i += kApplyThreads) acc[i] = 0ull;
-
-    const float *probs = p.probs + (size_t)seg * QKp;
-    const size_t sla_bg = ((size_t)b * p.Q * p.G + g) * 3 * LK;       // + q * G * 3LK
-    const size_t go_bg = ((size_t)b * p.Q * p.G + g) * D;             // + q * G * D
+    float acc[CW];
+#pragma unroll
+    for (int c = 0; c < CW; ++c) acc[c] = 0.f;
 
     // Everything a batch needs is requested through range-checked buffer loads of raw words: no branches
     // around the loads, so they all fly together, and nothing is converted before it is needed.
-    typedef typename RawWord<2 * Tag::kBytes>::type xy_t;      // (x, y) of a point are adjacent
-    const __amdgpu_buffer_rsrc_t sla_rs = make_rsrc(reinterpret_cast<const elem_t *>(p.sla) + sla_bg,
-                                                    (uint32_t)((size_t)p.Q * p.G * 3 * LK * Tag::kBytes));
-    const __amdgpu_buffer_rsrc_t go_rs = make_rsrc(reinterpret_cast<const elem_t *>(p.grad_out) + go_bg,
-                                                   (uint32_t)((size_t)p.Q * p.G * D * Tag::kBytes));
-    const __amdgpu_buffer_rsrc_t pr_rs = make_rsrc(probs, (uint32_t)QK * 4u);
-    // A row of 8 lanes owns a listed point; lane c of the row owns the CPL consecutive channels from c * CPL, loads
-    // them itself and keeps them in registers until the point is applied.
-    typedef typename RawWord<CPL * Tag::kBytes>::type goN_t;
-    constexpr int kRowsPerLane = kBatch * kRowLanes / kApplyThreads;      // rows a lane serves per batch: 2
-    constexpr int kRowStep = kApplyThreads / kRowLanes;
-    const int row_in_block = tid / kRowLanes, c = tid & (kRowLanes - 1);
+    const __amdgpu_buffer_rsrc_t rec_rs = make_rsrc(p.recs + (size_t)seg * QKp, (uint32_t)QK * 16u);
+    const __amdgpu_buffer_rsrc_t go_rs = make_rsrc(reinterpret_cast<const elem_t *>(p.go_rows) + (size_t)bg * p.Q * D,
+                                                   (uint32_t)((size_t)p.Q * D * Tag::kBytes));
+    // kCellLanes lanes fetch a listed point's grad_out row, CW channels each; a lane serves kRowsPerLane rows of a batch.
+    typedef typename RawWord<CW * Tag::kBytes>::type goN_t;
+    constexpr int kRowsPerLane = kBatch * kCellLanes / kApplyThreads;
+    constexpr int kRowStep = kApplyThreads / kCellLanes;
     struct Ahead {
-      xy_t xy;                         // lanes < batch size: their point
-      uint32_t pr;
+      u32x4 rec;                       // this lane's point of the batch: x, y, probability
       goN_t go[kRowsPerLane];
     };
     auto fetch = [&](uint32_t b0, int nb) {
       Ahead a;
       {
-        const uint32_t pt = s_list[b0 + min(tid, max(nb - 1, 0))];
-        const uint32_t q = pt / (uint32_t)p.K;
-        const int t = l * p.K + (int)(pt - q * p.K);
-        const bool live = tid < nb;
-        a.xy = buffer_load<2 * Tag::kBytes>(sla_rs, live ? (q * (uint32_t)(p.G * 3 * LK) + 2u * t) * Tag::kBytes : kDropOffset);
-        a.pr = buffer_load<4>(pr_rs, live ? pt * 4u : kDropOffset);
+        const uint32_t pt = s_list[min((int)b0 + min(tid, max(nb - 1, 0)), kListCap - 1)];
+        a.rec = buffer_load<16>(rec_rs, tid < nb ? pt * 16u : kDropOffset);
       }
 #pragma unroll
       for (int u = 0; u < kRowsPerLane; ++u) {
-        const int h = row_in_block + u * kRowStep;
-        const bool live = h < nb && c * CPL < D;
-        const uint32_t q = s_list[b0 + min(h, max(nb - 1, 0))] / (uint32_t)p.K;
-        a.go[u] = buffer_load<CPL * Tag::kBytes>(go_rs, live ? (q * (uint32_t)(p.G * D) + (uint32_t)(c * CPL)) * Tag::kBytes : kDropOffset);
+        const int h = my_slot + u * kRowStep;
+        const bool live = h < nb && my_part * CW < D;
+        const uint32_t q = s_list[min((int)b0 + min(h, max(nb - 1, 0)), kListCap - 1)] / (uint32_t)p.K;
+        a.go[u] = buffer_load<CW * Tag::kBytes>(go_rs, live ? (q * (uint32_t)D + (uint32_t)(my_part * CW)) * Tag::kBytes : kDropOffset);
       }
       return a;
     };
-    // one lane per point: corner weights and accumulator cells, into record buffer `buf`
-    auto park = [&](const Ahead &a, int nb, int buf) {
-      if (tid < nb) {
-        float xy[2];
-        Pack<Tag, 2>::decode(a.xy, xy);
-        const float x = sub_rn(mul_rn(xy[0], (float)lp.W), 0.5f);       // flash_deform_im2col_cuda.cuh:188-189
-        const float y = sub_rn(mul_rn(xy[1], (float)lp.H), 0.5f);
-        const Tap tp = make_tap(y, x, lp.H, lp.W, 0u, 0u);
-        const float ps = ldexpf(__builtin_bit_cast(float, a.pr), p.fix_bits);
-        const int ly = tp.y0 - ty0, lx = tp.x0 - tx0;
-        uint32_t cells[4];
-        float w[4];
-#pragma unroll
-        for (int cn = 0; cn < 4; ++cn) {
-          const int cy = ly + (cn >> 1), cx = lx + (cn & 1);
-          const bool ok = (tp.valid & (1u << cn)) && cy >= 0 && cy < th && cx >= 0 && cx < tw;
-          cells[cn] = ok ? (uint32_t)(cy * tw + cx) : (uint32_t)n_cells;
-          w[cn] = ok ? ps * tp.w[cn] : 0.f;
-        }
-        rec_w[buf * kBatch + tid] = f32x4{w[0], w[1], w[2], w[3]};
-        rec_meta[buf * kBatch + tid] = cells[0] | (cells[1] << kCellBitsF) | (cells[2] << (2 * kCellBitsF)) | (cells[3] << (3 * kCellBitsF));
-      }
-    };
-    // Accumulator word of (lane c, slot j) is c + 8 j: the lanes of a row touch consecutive words.  The LDS serves a
-    // wave's 64-bit atomics 16 lanes per pass over its 32 banks, two rows of eight lanes: row r visits its slots
-    // starting from slot r mod CPL, so neighbouring rows are on slots of different parity and the two rows of a pass
-    // fill the banks exactly once whatever their cells are.  The lane's channel values are rotated to that order
-    // once per point.
-    const int rot = row_in_block & (CPL - 1);
-    int slot_off[CPL];
-#pragma unroll
-    for (int j = 0; j < CPL; ++j) slot_off[j] = kRowLanes * ((j + rot) & (CPL - 1));
-    // applies the first n entries of s_list; called by every lane, ends past a barrier
+
+    // Applies the first n entries of s_list in batches of kBatch points, one lane per point:
+    //   A      the lane rebuilds its point's position; each corner inside the tile draws a rank in its cell
+    //          (integer LDS atomic) - barrier
+    //   scan   exclusive prefix sum of the 64 cell counts (one wave); all lanes park the batch's grad_out rows - barrier
+    //   place  (weight, parked row) entries go to cell start + rank; the next batch's loads are requested - barrier
+    //   B      four lanes per cell walk the cell's entries: sum += weight * grad_out row, fp32, in registers.
+    // No barrier after B: the next batch's phase A only touches the counters, and everything B reads is rewritten
+    // after that batch's first barrier.
     auto apply_list = [&](uint32_t n) {
       if (n == 0) return;
       int nb = (int)min((uint32_t)kBatch, n);
       Ahead cur = fetch(0, nb);
-      park(cur, nb, 0);
-      __syncthreads();
-      int buf = 0;
       for (uint32_t b0 = 0; b0 < n; b0 += kBatch) {
-        const int nb_next = b0 + kBatch < n ? (int)min((uint32_t)kBatch, n - b0 - kBatch) : 0;
-        Ahead nxt = cur;
-        if (nb_next > 0) nxt = fetch(b0 + kBatch, nb_next);      // flies while this batch is applied
+        // ---- phase A
+        float rec_w[4] = {0.f, 0.f, 0.f, 0.f};
+        uint32_t rec_cr[4] = {~0u, ~0u, ~0u, ~0u};            // cell << 16 | rank
+        if (tid < nb) {
+          // the position the first backward kernel formed (flash_deform_im2col_cuda.cuh:188-189), and the probability
+          // (a vector element is copied to a scalar first: a bit cast of the element expression itself reads element 0)
+          const uint32_t rx = cur.rec.x, ry = cur.rec.y, rz = cur.rec.z;
+          const float x = __builtin_bit_cast(float, rx), y = __builtin_bit_cast(float, ry);
+          if ((y > -1.f) && (x > -1.f) && (y < Hf) && (x < Wf)) {
+            const float fy = floorf(y), fx = floorf(x);
+            const float ly = y - fy, lx = x - fx, hy = 1.f - ly, hx = 1.f - lx;
+            const float pr = __builtin_bit_cast(float, rz);
+            const float w4[4] = {hy * hx, hy * lx, ly * hx, ly * lx};
+            // corner 0 relative to the tile; a corner inside the tile is inside the level (tiles are clipped to it)
+            const int cy0 = (int)fy - ty0, cx0 = (int)fx - tx0;
 #pragma unroll
-        for (int u = 0; u < kRowsPerLane; ++u) {
-          const int h = row_in_block + u * kRowStep;
-          if (h >= nb) break;
-          const f32x4 w = rec_w[buf * kBatch + h];
-          const uint32_t meta = rec_meta[buf * kBatch + h];
-          const uint32_t cells[4] = {meta & 127u, (meta >> kCellBitsF) & 127u, (meta >> (2 * kCellBitsF)) & 127u,
-                                     (meta >> (3 * kCellBitsF)) & 127u};
-          const float wv[4] = {w.x, w.y, w.z, w.w};
-          float g[CPL], gn[CPL];
-          Pack<Tag, CPL>::decode(cur.go[u], g);
-#pragma unroll
-          for (int j = 0; j < CPL; ++j) g[j] = ldexpf(g[j], -e_go);      // normalised to [-1, 1]
-          if constexpr (CPL == 4) {          // gn[j] = g[(j + rot) & 3]
-            const bool r1 = rot & 1, r2 = rot & 2;
-            const float a0 = r1 ? g[1] : g[0], a1 = r1 ? g[2] : g[1], a2 = r1 ? g[3] : g[2], a3 = r1 ? g[0] : g[3];
-            gn[0] = r2 ? a2 : a0; gn[1] = r2 ? a3 : a1; gn[2] = r2 ? a0 : a2; gn[3] = r2 ? a1 : a3;
-          } else if constexpr (CPL == 2) {
-            gn[0] = rot ? g[1] : g[0]; gn[1] = rot ? g[0] : g[1];
-          } else {
-            gn[0] = g[0];
-          }
-#pragma unroll
-          for (int cn = 0; cn < 4; ++cn) {
-            unsigned long long *dst = acc + __umul24(cells[cn], (uint32_t)DP) + c;
-            // the same resolution for every tensor dtype: small gradients next to large ones (loss scaling) keep
-            // their bits, as they do when the reference sums in fp32
-            const double wd = (double)wv[cn];
-#pragma unroll
-            for (int j = 0; j < CPL; ++j)
-              __hip_atomic_fetch_add(dst + slot_off[j], fixed_product((double)gn[j], wd), __ATOMIC_RELAXED,
-                                     __HIP_MEMORY_SCOPE_WORKGROUP);
+            for (int cn = 0; cn < 4; ++cn) {
+              const int cy = cy0 + (cn >> 1), cx = cx0 + (cn & 1);
+              if ((unsigned)cy < (unsigned)th && (unsigned)cx < (unsigned)tw) {
+                const uint32_t cell = (uint32_t)(cy * tw + cx);
+                rec_w[cn] = pr * w4[cn];
+                rec_cr[cn] = (cell << 16) | __hip_atomic_fetch_add(&s_count[cell], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+              }
+            }
           }
         }
-        if (nb_next > 0) park(nxt, nb_next, buf ^ 1);
         __syncthreads();
-        cur = nxt;
+
+        // ---- scan (first wave) and park (everyone)
+        if (tid < kWave) {
+          const uint32_t c = s_count[tid];
+          const uint32_t incl = wave_inclusive_scan(c);
+          s_offs[tid] = incl - c;
+          if (tid == kWave - 1) s_offs[kWave] = incl;
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsPerLane; ++u) {
+          const int h = my_slot + u * kRowStep;
+          if (h >= nb) break;
+          *reinterpret_cast<goN_t *>(s_go + h * kGoStride + my_part * (CW * kParkBytes)) = cur.go[u];
+        }
+        __syncthreads();
+
+        // ---- place
+        if (tid < kTileCells) s_count[tid] = 0u;              // for the next batch; the scan has read them
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn) {
+          const uint32_t cr = rec_cr[cn];
+          if (cr == ~0u) continue;
+          s_entry[s_offs[cr >> 16] + (cr & 0xffffu)] = u32x2{__builtin_bit_cast(uint32_t, rec_w[cn]), (uint32_t)(tid * kGoStride)};
+        }
+        const int nb_next = b0 + kBatch < n ? (int)min((uint32_t)kBatch, n - b0 - kBatch) : 0;
+        cur = fetch(b0 + kBatch, nb_next);      // flies while this batch is applied (after the last batch: nothing is read)
+        __syncthreads();
+
+        // ---- phase B: a lane walks every n_sub-th entry of its cell, two at a time and without branches inside
+        // (past the end of the list: weight 0 times the row of zeros), so that all LDS reads of a step are in
+        // flight together
+        if (my_cell < n_cells) {
+          const uint32_t beg = s_offs[my_cell], end = s_offs[my_cell + 1];
+          const char *go_lane = s_go + my_part * (CW * kParkBytes);
+          const uint32_t step = (uint32_t)n_sub;
+          for (uint32_t e = beg + (uint32_t)my_sub; e < end; e += 2u * step) {
+            const bool two = e + step < end;
+            const u32x2 ent0 = s_entry[e];
+            u32x2 ent1 = s_entry[two ? e + step : e];
+            ent1.x = two ? ent1.x : 0u;
+            ent1.y = two ? ent1.y : (uint32_t)(kBatch * kGoStride);
+            const goN_t row0 = *reinterpret_cast<const goN_t *>(go_lane + ent0.y);
+            const goN_t row1 = *reinterpret_cast<const goN_t *>(go_lane + ent1.y);
+            const uint32_t w0_bits = ent0.x, w1_bits = ent1.x;
+            const float w0 = __builtin_bit_cast(float, w0_bits), w1 = __builtin_bit_cast(float, w1_bits);
+            float g0[CW], g1[CW];
+            Pack<Tag, CW>::decode(row0, g0);
+            Pack<Tag, CW>::decode(row1, g1);
+#pragma unroll
+            for (int c = 0; c < CW; ++c) acc[c] = fmaf(w1, g1[c], fmaf(w0, g0[c], acc[c]));
+          }
+        }
         nb = nb_next;
-        buf ^= 1;
       }
     };
 
@@ -410,13 +455,9 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
           for (int base = 0; base < nc; base += kWave) {
             const int c = base + tid;
             const uint32_t v = c < nc ? s_tab[c] >> 16 : 0u;
-            uint32_t incl = v;
-            for (int o = 1; o < kWave; o <<= 1) {
-              const uint32_t up = (uint32_t)__shfl_up((int)incl, o, kWave);
-              if (tid >= o) incl += up;
-            }
+            const uint32_t incl = wave_inclusive_scan(v);
             if (c < nc) s_pre[c] = run + incl - v;
-            run += (uint32_t)__shfl((int)incl, kWave - 1, kWave);
+            run += (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
           }
           if (tid == 0) s_pre[nc] = run;
         }
@@ -425,6 +466,7 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
         // copy the slices into s_list, kListCap entries at a time; lane -> entry -> chunk by bisection
         for (uint32_t e0 = 0; e0 < total; e0 += kListCap) {
           const uint32_t ne = min((uint32_t)kListCap, total - e0);
+          __syncthreads();                                     // the previous list has been fetched from
           for (uint32_t i = tid; i < ne; i += kApplyThreads) {
             const uint32_t e = e0 + i;
             int lo = 0, hi = nc;                       // largest c with s_pre[c] <= e
@@ -440,22 +482,45 @@ __global__ void __launch_bounds__(kApplyThreads) fda_grad_value_kernel(const Fda
         }
       }
     }
-    __syncthreads();
 
-    // ---- the tile is complete (zeros when the statistics are unusable: the fallback kernel then adds everything)
-    elem_t *gv = reinterpret_cast<elem_t *>(p.grad_value);
-    for (int i = tid; i < n_cells * D; i += kApplyThreads) {
-      const int cell = i / D, ch = i - cell * D;
-      const int cy = cell / tw, cx = cell - cy * tw;
-      const unsigned long long a = acc[cell * DP + ch / CPL + kRowLanes * (ch % CPL)];
-      const double v = ldexp((double)(int)(a >> 32) * 4294967296.0 + (double)(uint32_t)a, e_out);
-      const float f[1] = {(float)v};
-      const long long n = (long long)lp.start + (long long)(ty0 + cy) * lp.W + tx0 + cx;      // level tables are not validated
-      if (n >= 0 && n < p.N) gv[(((size_t)b * p.N + (size_t)n) * p.G + g) * D + ch] = Pack<Tag, 1>::encode(f);
+    // ---- the tile is complete: the sub-lists' partial sums meet in LDS, then registers -> memory (zeros when the
+    // binning gave up: the fallback kernel then adds everything).  The lanes of a cell write DP contiguous channels.
+    if (n_sub > 1) {
+      __syncthreads();                                       // the last phase B is over: lists, entries and rows are free
+      float *s_part = reinterpret_cast<float *>(s_list);     // [kSlots][kCellLanes][CW]
+#pragma unroll
+      for (int c = 0; c < CW; ++c) s_part[(tid * CW) + c] = acc[c];
+      __syncthreads();
+      if (my_sub == 0) {
+        for (int j = 1; j < n_sub; ++j) {
+          const float *o = s_part + ((((j << cells_log2) + my_cell) << kCellLanesLog2) + my_part) * CW;
+#pragma unroll
+          for (int c = 0; c < CW; ++c) acc[c] += o[c];
+        }
+      }
+      __syncthreads();                                       // read before the row of zeros is restored
+      if (tid < kGoStride / 4) reinterpret_cast<uint32_t *>(s_go + kBatch * kGoStride)[tid] = 0u;
     }
-    __syncthreads();
+    if (my_cell < n_cells && my_sub == 0) {
+      const int cy = my_cell / tw, cx = my_cell - cy * tw;
+      const long long n = (long long)lp.start + (long long)(ty0 + cy) * lp.W + tx0 + cx;      // level tables are not validated
+      if (n >= 0 && n < p.N) {
+        elem_t *dst = reinterpret_cast<elem_t *>(p.grad_value) + (((size_t)b * p.N + (size_t)n) * p.G + g) * D + my_part * CW;
+        if ((D % CW) == 0 && (CW * Tag::kBytes) % 4 == 0) {
+          if (my_part * CW < D) *reinterpret_cast<goN_t *>(dst) = Pack<Tag, CW>::encode(acc);
+        } else {
+#pragma unroll
+          for (int c = 0; c < CW; ++c)
+            if (my_part * CW + c < D) { const float f[1] = {acc[c]}; dst[c] = Pack<Tag, 1>::encode(f); }
+        }
+      }
+    }
   }
 }
+
+// lanes per cell: four, or eight when four lanes of 16 bytes do not cover the (padded) head width
+int fda_cell_lanes(int D, int elem_bytes) { return fda_padded_channels(D) * elem_bytes > 64 ? 8 : 4; }
+int fda_sub_lists_for(int) { return kSubLists; }
 
 template <typename Tag>
 hipError_t launch_t(const FdaLaunch &p, hipStream_t stream) {
@@ -468,28 +533,46 @@ hipError_t launch_t(const FdaLaunch &p, hipStream_t stream) {
     int v = 0;
     if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
   }
-  const size_t lds = fda_grad_value_lds_bytes(p);
-  const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(4, (kMaxLdsPerWorkgroup - 4096) / (lds + 1024)));
-  const dim3 grid((unsigned)(cus * per_cu)), block(kApplyThreads);
+  const size_t lds = fda_grad_value_lds_bytes(p, Tag::kBytes);
+  const int lpc = fda_cell_lanes(p.D, Tag::kBytes), cw = fda_padded_channels(p.D) / lpc;
+  const int subs = fda_sub_lists_for(lpc);
+  const int threads = kTileCells * lpc * subs;
+  // persistent workgroups: as many per CU as LDS and wave slots (32 per CU) allow
+  // persistent workgroups: as many as are resident at once (registers, LDS and wave slots decide)
+  const dim3 block((unsigned)threads);
   auto go = [&](auto kernel) -> hipError_t {
     if (hipError_t e = ensure_dynamic_lds_limit(reinterpret_cast<const void *>(kernel), kMaxLdsPerWorkgroup - 2048)) return e;
-    hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, lds) != hipSuccess || per_cu < 1) per_cu = 1;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(cus * per_cu)), block, lds, stream, p);
     return hipGetLastError();
   };
-  switch (fda_padded_channels(p.D) / kRowLanes) {
-    case 1: return go(fda_grad_value_kernel<Tag, 1>);
-    case 2: return go(fda_grad_value_kernel<Tag, 2>);
-    case 4: return go(fda_grad_value_kernel<Tag, 4>);
+  if (lpc == 8) {
+    if constexpr (Tag::kBytes == 4) {
+      if (cw == 4) return go(fda_grad_value_kernel<Tag, 4, 8, kSubLists>);      // fp32 heads of 17 .. 32 channels
+    }
+    return hipErrorInvalidValue;
+  }
+  switch (cw) {
+    case 2: return go(fda_grad_value_kernel<Tag, 2, 4, kSubLists>);
+    case 4: return go(fda_grad_value_kernel<Tag, 4, 4, kSubLists>);
+    case 8:
+      if constexpr (Tag::kBytes == 2) return go(fda_grad_value_kernel<Tag, 8, 4, kSubLists>);
+      break;
   }
   return hipErrorInvalidValue;      // wider heads take the atomic path (the entry point checks)
 }
 
 }  // namespace
 
-size_t fda_grad_value_lds_bytes(const FdaLaunch &p) {
-  const size_t dp = (size_t)fda_padded_channels(p.D);
-  return ((size_t)kTileCells + 1) * dp * sizeof(unsigned long long) + 2 * kBatch * (sizeof(f32x4) + sizeof(uint32_t)) +
-         ((size_t)kListCap + 2 * kTabCap + 4) * sizeof(uint32_t);
+size_t fda_grad_value_lds_bytes(const FdaLaunch &p, int elem_bytes) {
+  const size_t go_stride = ((((size_t)fda_padded_channels(p.D) * elem_bytes + 15) / 16) | 1) * 16;
+  const size_t head = ((size_t)2 * kTileCells + 4) * sizeof(uint32_t);
+  const size_t batch = head + ((size_t)kListCap + 2 * kTabCap + 4) * sizeof(uint32_t) + ((size_t)4 * kBatch + 2) * sizeof(u32x2) +
+                       (size_t)(kBatch + 1) * go_stride;
+  // the sub-lists' partial sums meet in LDS behind the counters: a float per lane and channel it holds
+  const size_t meet = head + (size_t)kTileCells * kSubLists * fda_padded_channels(p.D) * sizeof(float);
+  return std::max(batch, meet);
 }
 
 hipError_t launch_fda_grad_value(int dtype, const FdaLaunch &p, hipStream_t stream) {

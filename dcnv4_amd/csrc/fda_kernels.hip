@@ -117,17 +117,16 @@ __global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLau
 // One kernel body, three roles (FdaBackwardMode):
 //   kFdaFull       grad_sampling_loc_attn, and grad_value scattered with fp32 buffer atomics into a
 //                  cleared fp32 image (any head width)
-//   kFdaNoScatter  grad_sampling_loc_attn, plus what the tiled grad_value kernel needs: one key per
-//                  sampling point and the maximum of |grad_out|
-//   kFdaFallback   exits at once unless max |grad_out| is not finite or the binning kernel flagged a level
-//                  it cannot hold; then it scatters with atomics in the tensor dtype into grad_value,
-//                  which the tiled kernel has left zeroed
+//   kFdaNoScatter  grad_sampling_loc_attn, plus what the tiled grad_value kernel needs: per sampling point a key
+//                  and a (position, softmax probability) record, and grad_out regrouped by head
+//   kFdaFallback   exits at once unless the binning kernel flagged a level it cannot hold; then it scatters
+//                  with atomics in the tensor dtype into grad_value, which the tiled kernel has left zeroed
 template <typename Tag, int CPT, int KT, int MODE>
 __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLaunch p) {
   extern __shared__ float lds[];
   typedef Pack<Tag, CPT> pack;
   if constexpr (MODE == kFdaFallback) {
-    if (p.state->go_max_bits < 0x7f800000u && p.state->reserved == 0u) return;
+    if (p.state->reserved == 0u) return;
   }
   const int LK = p.L * p.K, row_len = 3 * LK;
   const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
@@ -168,7 +167,6 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
   const int items = (nrow * heads_here) << tpgp_log2;
   const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
   const int K = KT > 0 ? KT : p.K;
-  uint32_t go_max = 0;
 
   for (int it = threadIdx.x; it < items; it += blockDim.x) {
     const int chunk = it & (width - 1);
@@ -192,11 +190,13 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
       }
     }
     float dot_rg = 0.f;
-    if constexpr (MODE == kFdaNoScatter) {
-#pragma unroll
-      for (int c = 0; c < CPT; ++c) go_max = max(go_max, __builtin_bit_cast(uint32_t, fabsf(go[c])));
-    }
     const int b_local = (row0 + lr) / p.Q, q = (row0 + lr) - b_local * p.Q;
+    if constexpr (MODE == kFdaNoScatter) {      // grad_out regrouped by head: the grad_value kernel gathers rows of one head at a time
+      if (active) {
+        char *dst = (char *)p.go_rows + ((((size_t)b_local * p.G + g) * p.Q + q) * p.D + chunk * CPT) * Tag::kBytes;
+        *reinterpret_cast<typename pack::raw_t *>(dst) = pack::encode(go);
+      }
+    }
 
     for (int l = 0; l < p.L; ++l) {
       const Level lv = load_level(p, l);
@@ -220,7 +220,7 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
                                                                                   : ((uint32_t)(tp.y0 + 1) << 8) | (uint32_t)(tp.x0 + 1);
             const size_t slot = (((size_t)b_local * p.G + g) * p.L + l) * fda_key_stride(p.Q, K) + (size_t)q * K + k;
             p.keys[slot] = (uint16_t)key;
-            p.probs[slot] = pr;
+            p.recs[slot] = f32x4_t{x, y, pr, 0.f};
           }
         }
         if constexpr (MODE == kFdaFallback) {
@@ -277,19 +277,6 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
     }
   }
   if constexpr (MODE == kFdaFallback) return;
-  if constexpr (MODE == kFdaNoScatter) {
-    // fold the statistic in LDS first: same-address global atomics retire slowly
-    __shared__ uint32_t s_stat;
-    if (threadIdx.x == 0) s_stat = 0u;
-    __syncthreads();
-    go_max = wave_max_u32(go_max);
-    if ((threadIdx.x & (kWave - 1)) == 0) atomicMax(&s_stat, go_max);
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      uint32_t *dst = &p.state->go_max_bits;
-      if (s_stat > __hip_atomic_load(dst, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(dst, s_stat);
-    }
-  }
   __syncthreads();
   if (p.head_major) {
     elem_t *dst = reinterpret_cast<elem_t *>(p.grad_sla) + ((size_t)row0 * p.G + g_fixed) * row_len;

@@ -20,8 +20,8 @@ constexpr size_t kMaxLdsPerWorkgroup = 160 * 1024;  // gfx950
 
 // Device-side scratch word block shared by the kernels of one backward call (16 bytes).
 struct GradState {
-  uint32_t go_max_bits;    // attention backward: max |grad_out| as IEEE bits (ordered like unsigned ints for x >= 0; NaN sorts last)
-  uint32_t unused;
+  uint32_t unused0;
+  uint32_t unused1;
   uint32_t reach_needed;   // DCNv4: largest Chebyshev distance (pixels) of an in-image corner of non-zero weight from its output pixel's reference point
   uint32_t reserved;       // attention backward: set when a level has more tiles than the binning kernel can count
 };
@@ -90,6 +90,8 @@ struct DcnLaunch {
 constexpr int dcnv4_grad_value_rounds(int cw) { return cw <= 16 ? 4 : 2; }
 
 // Flash deformable attention (reference: DCNv4_op/src/cuda/flash_deform_im2col_cuda.cuh:211-272)
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
 struct FdaLaunch {
   const void *value;        // [n_img, N, G, D]
   const void *sla;          // [n_row, G, 3*L*K]       n_row = images * Q
@@ -107,15 +109,15 @@ struct FdaLaunch {
   LaneMap lanes;
   // tiled grad_value path
   void *grad_value;         // [n_img, N, G, D] in the tensor dtype
-  GradState *state;         // go_max_bits only
+  GradState *state;         // `reserved` only
   uint16_t *keys;           // [n_img, G, L, QKp] one key per sampling point (QKp = Q*K rounded up to even)
-  float *probs;             // same layout: softmax probability of the point
+  f32x4_t *recs;            // same layout: (x, y, softmax probability, 0) of the point, x and y in cells of its level
+  void *go_rows;            // [n_img, G, Q, D] grad_out regrouped by head, tensor dtype: a head's rows lie densely
   uint32_t *table;          // [n_img * G * L * n_chunks][tile_stride] (offset | count << 16) of every tile in every chunk's sorted list
   uint32_t *regions;        // [n_img * G * L * n_chunks][4 * kFdaChunkPoints] point ids of a chunk, sorted by tile
   int n_chunks;             // chunks of kFdaChunkPoints points per (image, head, level)
   int tile_stride;          // table row length: an upper bound of the tiles of one level
   int n_img;
-  int fix_bits;             // fractional bits of the fixed-point accumulators
 };
 
 // Key of a sampling point: (y0 + 1) << 8 | (x0 + 1) for the integer position (y0, x0) of its first
@@ -130,8 +132,8 @@ __host__ __device__ inline size_t fda_key_stride(int Q, int K) { return ((size_t
 
 enum FdaBackwardMode {
   kFdaFull = 0,        // grad_sampling_loc_attn + fp32 atomic scatter of grad_value (any head width)
-  kFdaNoScatter = 1,   // grad_sampling_loc_attn + keys + max |grad_out|, no scatter
-  kFdaFallback = 2,    // scatter with atomics in the tensor dtype, only when max |grad_out| is not finite
+  kFdaNoScatter = 1,   // grad_sampling_loc_attn + keys + probabilities, no scatter
+  kFdaFallback = 2,    // scatter with atomics in the tensor dtype, only when the binning kernel gave up on a level
 };
 
 // Accumulator channels per cell of the tiled flash-attention grad_value kernel (head width rounded up to
@@ -187,7 +189,7 @@ size_t dcnv4_tiled_gather_lds_bytes(const DcnLaunch &p, int elem_bytes);
 hipError_t launch_fda_forward(int dtype, const FdaLaunch &p, hipStream_t stream);
 hipError_t launch_fda_backward(int dtype, const FdaLaunch &p, int mode, hipStream_t stream);
 hipError_t launch_fda_grad_value(int dtype, const FdaLaunch &p, hipStream_t stream);
-size_t fda_grad_value_lds_bytes(const FdaLaunch &p);
+size_t fda_grad_value_lds_bytes(const FdaLaunch &p, int elem_bytes);
 
 size_t dcnv4_forward_lds_bytes(const DcnLaunch &p);
 size_t dcnv4_backward_lds_bytes(const DcnLaunch &p);

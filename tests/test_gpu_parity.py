@@ -243,15 +243,20 @@ def test_flash_deform_attn_backward_paths_match_oracle(oracle, name, scatter, dt
     cabi.assert_close(gs, wgs, *GRAD_TOL[dtype], what="grad_sampling_loc_attn")
 
 
-def test_flash_deform_attn_backward_is_bit_reproducible_and_handles_non_finite_grad_out(oracle):
+def test_flash_deform_attn_backward_repeats_and_handles_non_finite_grad_out(oracle):
     B, shapes, G, D, K, Q, (lo, hi) = FDA_CASES["detr_small_4lvl_k4"]
     v, shp, st, sla, go = make_fda_inputs(B, shapes, G, D, K, Q, seed=4, dtype=torch.float16, loc_lo=lo, loc_hi=hi)
     args = (v.cuda(), shp.cuda(), st.cuda(), sla.cuda())
     first = cabi.fda_backward(*args, go.cuda(), K)
     for _ in range(3):
+        # grad_sampling_loc_attn has a fixed summation order; grad_value sums in fp32 in the order the hardware ranked the
+        # terms and rounds once: repeats differ by at most one unit of fp16, rarely
         again = cabi.fda_backward(*args, go.cuda(), K)
-        assert torch.equal(first[0], again[0]) and torch.equal(first[1], again[1])
-    # NaN / Inf in grad_out: the fixed-point path steps aside, the result still matches the oracle's pattern
+        assert torch.equal(first[1], again[1])
+        diff = (first[0].float() - again[0].float()).abs()
+        assert (diff <= 2e-3 * first[0].float().abs() + 1e-6).all() and (diff > 0).float().mean().item() < 0.01
+    # NaN / Inf in grad_out propagate exactly like in the oracle (sums are floating point throughout), and every
+    # finite element keeps the gradient tolerance
     go32 = go.float()
     go32[0, 3, 5] = float("nan")
     go32[1, 7, 40] = float("inf")
@@ -259,10 +264,9 @@ def test_flash_deform_attn_backward_is_bit_reproducible_and_handles_non_finite_g
     gv, _ = cabi.fda_backward(*args, go32.half().cuda(), K)
     gv = cabi.f64(gv)
     assert np.array_equal(np.isnan(gv), np.isnan(wgv))
+    assert np.array_equal(np.isposinf(gv), np.isposinf(wgv)) and np.array_equal(np.isneginf(gv), np.isneginf(wgv))
     ok = np.isfinite(wgv)
-    # this path adds with fp16 atomics in whatever order the hardware takes them: sums of some tens of terms, each
-    # rounded to fp16 (40 runs of this case showed up to 2.2e-2 of absolute + relative error)
-    np.testing.assert_allclose(gv[ok], wgv[ok], rtol=4e-2, atol=4e-2)
+    np.testing.assert_allclose(gv[ok], wgv[ok], rtol=1e-2, atol=1e-2)
 
 
 def test_c_abi_rejects_bad_arguments():
@@ -401,7 +405,8 @@ def test_flash_deform_attn_head_major_order_matches_oracle_and_row_order(oracle,
     with ext.launch_options(fda_order="rows"):
         out_rows = cabi.fda_forward(*args, K)
         gv_rows, gs_rows = cabi.fda_backward(*args, go.cuda(), K)
-    assert torch.equal(out, out_rows) and torch.equal(gs, gs_rows) and torch.equal(gv, gv_rows)
+    assert torch.equal(out, out_rows) and torch.equal(gs, gs_rows)
+    assert (gv.float() - gv_rows.float()).abs().max().item() <= 2e-3 * gv.float().abs().max().item()      # fp32 sums in hardware order
     want = oracle.flash_deform_attn_forward(cabi.f64(v), shp.numpy(), st.numpy(), cabi.f64(sla), K, coord_f32=True)
     wgv, wgs = oracle.flash_deform_attn_backward(cabi.f64(v), shp.numpy(), st.numpy(), cabi.f64(sla), cabi.f64(go), K, coord_f32=True)
     cabi.assert_close(out, want, *FWD_TOL[dtype], what="output")
