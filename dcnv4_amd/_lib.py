@@ -10,7 +10,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libdcnv4_gfx950.so")
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 OK, ERR_INVALID_ARGUMENT, ERR_RUNTIME = 0, 1, 2
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 
@@ -33,6 +33,12 @@ SIGNATURES = {
     "dcnv4_gfx950_depthwise_conv_backward_workspace_bytes": (_sz, [_i] * 7),
     "dcnv4_gfx950_depthwise_conv_backward": (_i, [_vp] * 7 + [_sz] + [_i] * 7 + [_vp]),
     "dcnv4_gfx950_layer_norm_residual_forward": (_i, [_vp] * 6 + [_i, ctypes.c_longlong, _i, _f, _vp]),
+    "flash_deform_attn_gfx950_forward_split": (_i, [_vp] * 6 + [_i] * 12 + [_vp]),
+    "flash_deform_attn_gfx950_backward_split": (_i, [_vp] * 10 + [_sz] + [_i] * 12 + [_vp]),
+    "dcnv4_gfx950_layer_norm_residual_backward_workspace_bytes": (_sz, [_i, ctypes.c_longlong, _i]),
+    "dcnv4_gfx950_layer_norm_residual_backward": (_i, [_vp] * 10 + [_sz, _i, ctypes.c_longlong, _i, _f, _vp]),
+    "dcnv4_gfx950_center_feature_blend_forward": (_i, [_vp] * 5 + [_i, ctypes.c_longlong, _i, _i, _vp]),
+    "dcnv4_gfx950_center_feature_blend_backward": (_i, [_vp] * 8 + [_i, ctypes.c_longlong, _i, _i, _vp]),
 }
 
 _lib = None

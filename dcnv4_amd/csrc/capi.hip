@@ -631,23 +631,49 @@ int dcnv4_gfx950_backward_static_scratch(const void *value, const void *offset_m
                            softmax, d_stride, block_thread, stream);
 }
 
-int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_shapes,
-                                     const int64_t *level_start_index, const void *sampling_loc_attn,
-                                     void *output, int dtype, int batch, int spatial_size, int num_heads,
-                                     int head_channels, int num_levels, int num_query, int num_points,
-                                     int im2col_step, int d_stride, int block_thread, void *stream) {
+// Rows of a (query, head): either one packed tensor (sla) or locations + logits (loc, logits; the locations in fp32
+// or in the tensor dtype).
+struct FdaRows {
+  const void *sla, *loc, *logits;
+  void *grad_sla, *grad_loc, *grad_logits;
+  int loc_bytes;      // 0: packed rows
+};
+
+static void fda_set_rows(FdaLaunch *F, const FdaRows &r, const FdaProblem &pr, int b0, int LK) {
+  const size_t pairs = (size_t)b0 * F->Q * F->G;
+  F->sla = r.sla ? at(r.sla, b0 * pr.img_row_elems, pr.s) : nullptr;
+  F->grad_sla = r.grad_sla ? at(r.grad_sla, b0 * pr.img_row_elems, pr.s) : nullptr;
+  F->loc = r.loc ? at(r.loc, pairs * 2 * LK, r.loc_bytes) : nullptr;
+  F->grad_loc = r.grad_loc ? at(r.grad_loc, pairs * 2 * LK, r.loc_bytes) : nullptr;
+  F->logits = r.logits ? at(r.logits, pairs * LK, pr.s) : nullptr;
+  F->grad_logits = r.grad_logits ? at(r.grad_logits, pairs * LK, pr.s) : nullptr;
+  F->loc_f32 = r.loc_bytes == 4 ? 1 : 0;
+}
+
+static int fda_check_split(int dtype, int location_dtype, int *loc_bytes) {
+  if (elem_bytes(dtype) == 0) return fail(DCNV4_ERR_RUNTIME, "unsupported dtype code %d (fp32, fp16, bf16 only)", dtype);
+  if (location_dtype != DCNV4_DTYPE_F32 && location_dtype != dtype)
+    return fail(DCNV4_ERR_RUNTIME, "sampling locations must be fp32 or of the value's dtype (codes %d, %d)", location_dtype, dtype);
+  *loc_bytes = elem_bytes(location_dtype);
+  return DCNV4_OK;
+}
+
+static int fda_forward_impl(const void *value, const int64_t *spatial_shapes, const int64_t *level_start_index,
+                            const FdaRows &rows, void *output, int dtype, int batch, int spatial_size, int num_heads,
+                            int head_channels, int num_levels, int num_query, int num_points, int im2col_step,
+                            int d_stride, int block_thread, void *stream) {
   FdaProblem pr;
   if (int rc = fda_prepare(&pr, false, false, dtype, batch, spatial_size, num_heads, head_channels, num_levels, num_query,
                            num_points, im2col_step, d_stride, block_thread))
     return rc;
-  if (int rc = check_ptrs({value, sampling_loc_attn, output})) return rc;
+  if (int rc = rows.loc_bytes == 0 ? check_ptrs({value, rows.sla, output}) : check_ptrs({value, rows.loc, rows.logits, output})) return rc;
   if (spatial_shapes == nullptr || level_start_index == nullptr) return fail(DCNV4_ERR_RUNTIME, "null level tensors");
   const int per = images_per_launch(pr, false);
   for (int b0 = 0; b0 < batch; b0 += per) {
     const int nb = std::min(per, batch - b0);
     FdaLaunch F = pr.launch;
     F.value = at(value, b0 * pr.img_elems, pr.s);
-    F.sla = at(sampling_loc_attn, b0 * pr.img_row_elems, pr.s);
+    fda_set_rows(&F, rows, pr, b0, num_levels * num_points);
     F.out = at(output, b0 * pr.img_out_elems, pr.s);
     F.shapes = spatial_shapes;
     F.level_start = level_start_index;
@@ -658,6 +684,29 @@ int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_s
       return hip_fail("flash_deform_attn forward launch", e);
   }
   return DCNV4_OK;
+}
+
+int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_shapes,
+                                     const int64_t *level_start_index, const void *sampling_loc_attn,
+                                     void *output, int dtype, int batch, int spatial_size, int num_heads,
+                                     int head_channels, int num_levels, int num_query, int num_points,
+                                     int im2col_step, int d_stride, int block_thread, void *stream) {
+  const FdaRows rows{sampling_loc_attn, nullptr, nullptr, nullptr, nullptr, nullptr, 0};
+  return fda_forward_impl(value, spatial_shapes, level_start_index, rows, output, dtype, batch, spatial_size, num_heads,
+                          head_channels, num_levels, num_query, num_points, im2col_step, d_stride, block_thread, stream);
+}
+
+int flash_deform_attn_gfx950_forward_split(const void *value, const int64_t *spatial_shapes,
+                                           const int64_t *level_start_index, const void *sampling_locations,
+                                           const void *attention_logits, void *output, int dtype, int location_dtype,
+                                           int batch, int spatial_size, int num_heads, int head_channels,
+                                           int num_levels, int num_query, int num_points, int im2col_step,
+                                           int d_stride, int block_thread, void *stream) {
+  int loc_bytes = 0;
+  if (int rc = fda_check_split(dtype, location_dtype, &loc_bytes)) return rc;
+  const FdaRows rows{nullptr, sampling_locations, attention_logits, nullptr, nullptr, nullptr, loc_bytes};
+  return fda_forward_impl(value, spatial_shapes, level_start_index, rows, output, dtype, batch, spatial_size, num_heads,
+                          head_channels, num_levels, num_query, num_points, im2col_step, d_stride, block_thread, stream);
 }
 
 // Scratch of the tiled attention backward, in this order: GradState, keys, point records, grad_out regrouped by head,
@@ -698,13 +747,11 @@ size_t flash_deform_attn_gfx950_backward_workspace_bytes(int dtype, int batch, i
   return need;
 }
 
-int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_shapes,
-                                      const int64_t *level_start_index, const void *sampling_loc_attn,
-                                      const void *grad_output, void *grad_value, void *grad_sampling_loc_attn,
-                                      void *workspace, size_t workspace_bytes, int dtype, int batch,
-                                      int spatial_size, int num_heads, int head_channels, int num_levels,
-                                      int num_query, int num_points, int im2col_step, int d_stride,
-                                      int block_thread, void *stream) {
+static int fda_backward_impl(const void *value, const int64_t *spatial_shapes, const int64_t *level_start_index,
+                             const FdaRows &rows, const void *grad_output, void *grad_value, void *workspace,
+                             size_t workspace_bytes, int dtype, int batch, int spatial_size, int num_heads,
+                             int head_channels, int num_levels, int num_query, int num_points, int im2col_step,
+                             int d_stride, int block_thread, void *stream) {
   FdaProblem pr;
   // the tiled grad_value kernel addresses one image's sampling_loc_attn and grad_out with 32-bit byte offsets
   const unsigned long long row_bytes = (unsigned long long)std::max(num_heads, 1) *
@@ -715,7 +762,9 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
   if (int rc = fda_prepare(&pr, true, !tiled, dtype, batch, spatial_size, num_heads, head_channels, num_levels, num_query,
                            num_points, im2col_step, d_stride, block_thread))
     return rc;
-  if (int rc = check_ptrs({value, sampling_loc_attn, grad_output, grad_value, grad_sampling_loc_attn})) return rc;
+  if (int rc = rows.loc_bytes == 0 ? check_ptrs({value, rows.sla, grad_output, grad_value, rows.grad_sla})
+                        : check_ptrs({value, rows.loc, rows.logits, grad_output, grad_value, rows.grad_loc, rows.grad_logits}))
+    return rc;
   if (spatial_shapes == nullptr || level_start_index == nullptr) return fail(DCNV4_ERR_RUNTIME, "null level tensors");
   const size_t need = flash_deform_attn_gfx950_backward_workspace_bytes(dtype, batch, spatial_size, num_heads, head_channels,
                                                                         num_levels, num_query, num_points);
@@ -748,10 +797,9 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
         const int nb = std::min(per, batch - b0);
         FdaLaunch F = base;
         F.value = at(value, b0 * pr.img_elems, pr.s);
-        F.sla = at(sampling_loc_attn, b0 * pr.img_row_elems, pr.s);
+        fda_set_rows(&F, rows, pr, b0, num_levels * num_points);
         F.grad_out = at(grad_output, b0 * pr.img_out_elems, pr.s);
         F.grad_value = at(grad_value, b0 * pr.img_elems, pr.s);
-        F.grad_sla = at(grad_sampling_loc_attn, b0 * pr.img_row_elems, pr.s);
         F.keys = keys + b0 * img_keys;
         F.recs = recs + b0 * img_keys;
         F.go_rows = go_rows + (size_t)b0 * pr.img_out_elems * pr.s;
@@ -778,10 +826,9 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
     const int nb = std::min(per, batch - b0);
     FdaLaunch F = pr.launch;
     F.value = at(value, b0 * pr.img_elems, pr.s);
-    F.sla = at(sampling_loc_attn, b0 * pr.img_row_elems, pr.s);
+    fda_set_rows(&F, rows, pr, b0, num_levels * num_points);
     F.grad_out = at(grad_output, b0 * pr.img_out_elems, pr.s);
     F.grad_value_acc = acc + b0 * pr.img_elems;
-    F.grad_sla = at(grad_sampling_loc_attn, b0 * pr.img_row_elems, pr.s);
     F.shapes = spatial_shapes;
     F.level_start = level_start_index;
     F.value_bytes = (uint32_t)(nb * pr.img_elems * pr.s);
@@ -791,6 +838,35 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
   if (widen)
     if (hipError_t e = narrow_async(dtype, acc, grad_value, total, st)) return hip_fail("cast launch", e);
   return DCNV4_OK;
+}
+
+int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_shapes,
+                                      const int64_t *level_start_index, const void *sampling_loc_attn,
+                                      const void *grad_output, void *grad_value, void *grad_sampling_loc_attn,
+                                      void *workspace, size_t workspace_bytes, int dtype, int batch,
+                                      int spatial_size, int num_heads, int head_channels, int num_levels,
+                                      int num_query, int num_points, int im2col_step, int d_stride,
+                                      int block_thread, void *stream) {
+  const FdaRows rows{sampling_loc_attn, nullptr, nullptr, grad_sampling_loc_attn, nullptr, nullptr, 0};
+  return fda_backward_impl(value, spatial_shapes, level_start_index, rows, grad_output, grad_value, workspace, workspace_bytes,
+                           dtype, batch, spatial_size, num_heads, head_channels, num_levels, num_query, num_points,
+                           im2col_step, d_stride, block_thread, stream);
+}
+
+int flash_deform_attn_gfx950_backward_split(const void *value, const int64_t *spatial_shapes,
+                                            const int64_t *level_start_index, const void *sampling_locations,
+                                            const void *attention_logits, const void *grad_output, void *grad_value,
+                                            void *grad_sampling_locations, void *grad_attention_logits,
+                                            void *workspace, size_t workspace_bytes, int dtype, int location_dtype,
+                                            int batch, int spatial_size, int num_heads, int head_channels,
+                                            int num_levels, int num_query, int num_points, int im2col_step,
+                                            int d_stride, int block_thread, void *stream) {
+  int loc_bytes = 0;
+  if (int rc = fda_check_split(dtype, location_dtype, &loc_bytes)) return rc;
+  const FdaRows rows{nullptr, sampling_locations, attention_logits, nullptr, grad_sampling_locations, grad_attention_logits, loc_bytes};
+  return fda_backward_impl(value, spatial_shapes, level_start_index, rows, grad_output, grad_value, workspace, workspace_bytes,
+                           dtype, batch, spatial_size, num_heads, head_channels, num_levels, num_query, num_points,
+                           im2col_step, d_stride, block_thread, stream);
 }
 
 int dcnv4_gfx950_depthwise_conv_forward(const void *input, const void *weight, const void *bias, void *output,
@@ -874,9 +950,8 @@ int dcnv4_gfx950_depthwise_conv_backward(const void *input, const void *weight, 
   return DCNV4_OK;
 }
 
-int dcnv4_gfx950_layer_norm_residual_forward(const void *input, const void *residual, const void *weight,
-                                             const void *bias, const void *gamma, void *output, int dtype,
-                                             long long rows, int channels, float eps, void *stream) {
+// Row geometry shared by the layer-norm forward and backward: a team of lanes per row, 16-byte vectors per lane.
+static int ln_prepare(LnLaunch *L, int dtype, long long rows, int channels, float eps) {
   const int s = elem_bytes(dtype);
   if (s == 0) return fail(DCNV4_ERR_RUNTIME, "unsupported dtype code %d (fp32, fp16, bf16 only)", dtype);
   if (rows <= 0 || channels <= 0) return fail(DCNV4_ERR_RUNTIME, "empty or negative extent (rows %lld, channels %d)", rows, channels);
@@ -884,18 +959,107 @@ int dcnv4_gfx950_layer_norm_residual_forward(const void *input, const void *resi
   if (channels % V != 0) return fail(DCNV4_ERR_INVALID_ARGUMENT, "channels (%d) must be a multiple of %d for this dtype", channels, V);
   const int nvec = channels / V;
   if (nvec > 64 * 8) return fail(DCNV4_ERR_INVALID_ARGUMENT, "rows of %d channels are too long (at most %d)", channels, 64 * 8 * V);
+  *L = LnLaunch{};
+  L->rows = rows; L->C = channels; L->eps = eps;
+  L->team = 1;
+  while (L->team < 64 && L->team < nvec) L->team *= 2;
+  L->vpl = 1;
+  while (L->team * L->vpl < nvec) L->vpl *= 2;
+  // backward: about 2048 workgroups at most, each a slab of whole passes; partial sums stay below 32 MB
+  const long long rows_per_pass = 256 / L->team;
+  long long parts = std::min<long long>((rows + rows_per_pass - 1) / rows_per_pass, 2048);
+  while (parts > 1 && (size_t)parts * 3 * channels * sizeof(float) > (size_t(32) << 20)) parts /= 2;
+  L->slab = ((rows + parts - 1) / parts + rows_per_pass - 1) / rows_per_pass * rows_per_pass;
+  L->n_part = (int)((rows + L->slab - 1) / L->slab);
+  return DCNV4_OK;
+}
+
+int dcnv4_gfx950_layer_norm_residual_forward(const void *input, const void *residual, const void *weight,
+                                             const void *bias, const void *gamma, void *output, int dtype,
+                                             long long rows, int channels, float eps, void *stream) {
+  LnLaunch L;
+  if (int rc = ln_prepare(&L, dtype, rows, channels, eps)) return rc;
   if (int rc = check_ptrs({input, weight, bias, output})) return rc;
   if ((residual != nullptr && !aligned16(residual)) || (gamma != nullptr && !aligned16(gamma)))
     return fail(DCNV4_ERR_RUNTIME, "tensor pointer is not 16-byte aligned");
-  LnLaunch L{};
   L.y = input; L.residual = residual; L.weight = weight; L.bias = bias; L.gamma = gamma; L.out = output;
-  L.rows = rows; L.C = channels; L.eps = eps;
-  L.team = 1;
-  while (L.team < 64 && L.team < nvec) L.team *= 2;
-  L.vpl = 1;
-  while (L.team * L.vpl < nvec) L.vpl *= 2;
   if (hipError_t e = launch_layer_norm_residual(dtype, L, static_cast<hipStream_t>(stream)))
     return hip_fail("layer norm launch", e);
+  return DCNV4_OK;
+}
+
+size_t dcnv4_gfx950_layer_norm_residual_backward_workspace_bytes(int dtype, long long rows, int channels) {
+  LnLaunch L;
+  if (ln_prepare(&L, dtype, rows, channels, 0.f)) return 0;
+  return round16((size_t)L.n_part * 3 * channels * sizeof(float));
+}
+
+int dcnv4_gfx950_layer_norm_residual_backward(const void *grad_output, const void *input, const void *weight,
+                                              const void *bias, const void *gamma, void *grad_input,
+                                              void *grad_weight, void *grad_bias, void *grad_gamma, void *workspace,
+                                              size_t workspace_bytes, int dtype, long long rows, int channels,
+                                              float eps, void *stream) {
+  LnLaunch L;
+  if (int rc = ln_prepare(&L, dtype, rows, channels, eps)) return rc;
+  if (int rc = check_ptrs({grad_output, input, weight, grad_input})) return rc;
+  if (gamma != nullptr && bias == nullptr) return fail(DCNV4_ERR_RUNTIME, "the gradient of gamma needs the bias of the normalisation");
+  for (const void *q : {bias, gamma, (const void *)grad_weight, (const void *)grad_bias, (const void *)grad_gamma})
+    if (q != nullptr && !aligned16(q)) return fail(DCNV4_ERR_RUNTIME, "tensor pointer %p is not 16-byte aligned", q);
+  if (grad_gamma != nullptr && gamma == nullptr) return fail(DCNV4_ERR_RUNTIME, "grad_gamma asked for without gamma");
+  const size_t need = round16((size_t)L.n_part * 3 * channels * sizeof(float));
+  if (workspace == nullptr || !aligned16(workspace) || workspace_bytes < need)
+    return fail(DCNV4_ERR_RUNTIME, "workspace of %zu bytes needed, got %zu at %p", need, workspace_bytes, workspace);
+  L.grad_out = grad_output; L.y = input; L.weight = weight; L.bias = bias; L.gamma = gamma;
+  L.grad_y = grad_input; L.grad_weight = grad_weight; L.grad_bias = grad_bias; L.grad_gamma = grad_gamma;
+  L.partial = static_cast<float *>(workspace);
+  if (hipError_t e = launch_layer_norm_residual_backward(dtype, L, static_cast<hipStream_t>(stream)))
+    return hip_fail("layer norm backward launch", e);
+  return DCNV4_OK;
+}
+
+static int cf_prepare(CfLaunch *L, int dtype, long long rows, int channels, int groups) {
+  const int s = elem_bytes(dtype);
+  if (s == 0) return fail(DCNV4_ERR_RUNTIME, "unsupported dtype code %d (fp32, fp16, bf16 only)", dtype);
+  if (rows <= 0 || channels <= 0 || groups <= 0)
+    return fail(DCNV4_ERR_RUNTIME, "empty or negative extent (rows %lld, channels %d, groups %d)", rows, channels, groups);
+  const int V = 16 / s;
+  if (channels % groups != 0) return fail(DCNV4_ERR_INVALID_ARGUMENT, "%d channels cannot be split into %d equal groups", channels, groups);
+  const int D = channels / groups;
+  if (D % V != 0) return fail(DCNV4_ERR_INVALID_ARGUMENT, "group width (%d) must be a multiple of %d for this dtype", D, V);
+  const int nvec = channels / V;
+  if (nvec > 64 * 8) return fail(DCNV4_ERR_INVALID_ARGUMENT, "rows of %d channels are too long (at most %d)", channels, 64 * 8 * V);
+  *L = CfLaunch{};
+  L->rows = rows; L->C = channels; L->G = groups; L->D = D;
+  L->team = 1;
+  while (L->team < 64 && L->team < nvec) L->team *= 2;
+  L->vpl = 1;
+  while (L->team * L->vpl < nvec) L->vpl *= 2;
+  return DCNV4_OK;
+}
+
+int dcnv4_gfx950_center_feature_blend_forward(const void *sampled, const void *projected, const void *weight,
+                                              const void *bias, void *output, int dtype, long long rows,
+                                              int channels, int groups, void *stream) {
+  CfLaunch L;
+  if (int rc = cf_prepare(&L, dtype, rows, channels, groups)) return rc;
+  if (int rc = check_ptrs({sampled, projected, weight, bias, output})) return rc;
+  L.y = sampled; L.x = projected; L.weight = weight; L.bias = bias; L.out = output;
+  if (hipError_t e = launch_center_feature_blend(dtype, L, false, static_cast<hipStream_t>(stream)))
+    return hip_fail("centre-feature blend launch", e);
+  return DCNV4_OK;
+}
+
+int dcnv4_gfx950_center_feature_blend_backward(const void *grad_output, const void *sampled, const void *projected,
+                                               const void *weight, const void *bias, void *grad_sampled,
+                                               void *grad_projected, float *grad_gate_logits, int dtype,
+                                               long long rows, int channels, int groups, void *stream) {
+  CfLaunch L;
+  if (int rc = cf_prepare(&L, dtype, rows, channels, groups)) return rc;
+  if (int rc = check_ptrs({grad_output, sampled, projected, weight, bias, grad_sampled, grad_projected, grad_gate_logits})) return rc;
+  L.grad_out = grad_output; L.y = sampled; L.x = projected; L.weight = weight; L.bias = bias;
+  L.grad_y = grad_sampled; L.grad_x = grad_projected; L.grad_logits = grad_gate_logits;
+  if (hipError_t e = launch_center_feature_blend(dtype, L, true, static_cast<hipStream_t>(stream)))
+    return hip_fail("centre-feature blend backward launch", e);
   return DCNV4_OK;
 }
 

@@ -87,10 +87,9 @@ __global__ void __launch_bounds__(kBinThreads) fda_bin_points_kernel(const FdaLa
   __shared__ uint32_t s_hist[kFdaMaxTilesPerLevel];       // counts, then running cursors
   __shared__ uint32_t s_wave_sum[kBinThreads / kWave];
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-  const int QK = p.Q * p.K, LK = p.L * p.K;
+  const int QK = p.Q * p.K;
   const int chunk = blockIdx.x % p.n_chunks, seg = blockIdx.x / p.n_chunks;       // seg = (image * G + head) * L + level
-  const int l = seg % p.L, bg = seg / p.L;
-  const int b = bg / p.G, g = bg - b * p.G;
+  const int l = seg % p.L;
   const LevelPlan lp = level_plan(p, l);
   const int n_tiles = lp.nty * lp.ntx;
   if (n_tiles > p.tile_stride || n_tiles > kFdaMaxTilesPerLevel) {
@@ -104,7 +103,6 @@ __global__ void __launch_bounds__(kBinThreads) fda_bin_points_kernel(const FdaLa
   const uint32_t *keys = reinterpret_cast<const uint32_t *>(p.keys + (size_t)seg * QKp);
   const int n_words = (int)(QKp / 2);
   const float inv_th = 1.f / (float)lp.th, inv_tw = 1.f / (float)lp.tw;
-  const size_t sla_bg = ((size_t)b * p.Q * p.G + g) * 3 * LK;
 
   auto touch_of = [&](uint32_t k16, uint32_t pt) {
     Touch t;
@@ -112,12 +110,8 @@ __global__ void __launch_bounds__(kBinThreads) fda_bin_points_kernel(const FdaLa
     if (pt >= (uint32_t)QK || k16 == kFdaKeyOutside) return t;
     int y1 = (int)(k16 >> 8), x1 = (int)(k16 & 0xffu);             // y0 + 1, x0 + 1
     if (k16 == kFdaKeySaturated) {                                // position beyond the key's fields: recompute it
-      const uint32_t q = pt / (uint32_t)p.K;
-      const int tt = l * p.K + (int)(pt - q * p.K);
-      const size_t row = sla_bg + (size_t)q * p.G * 3 * LK;
-      const float x = sub_rn(mul_rn(elem_at<Tag>(p.sla, row + 2 * tt), (float)lp.W), 0.5f);
-      const float y = sub_rn(mul_rn(elem_at<Tag>(p.sla, row + 2 * tt + 1), (float)lp.H), 0.5f);
-      const Tap tp = make_tap(y, x, lp.H, lp.W, 0u, 0u);
+      const f32x4_t rec = p.recs[(size_t)seg * QKp + pt];          // the position the first backward kernel formed
+      const Tap tp = make_tap(rec.y, rec.x, lp.H, lp.W, 0u, 0u);
       if (tp.valid == 0) return t;
       y1 = tp.y0 + 1; x1 = tp.x0 + 1;
     }
@@ -228,7 +222,7 @@ __global__ void __launch_bounds__(kTileCells * LPC * SUBS) fda_grad_value_kernel
   constexpr int DP = CW * kCellLanes;
   constexpr int kParkBytes = Tag::kBytes;
   constexpr int kGoStride = (((DP * kParkBytes + 15) / 16) | 1) * 16;     // an odd number of 16-byte units per parked row
-  const int D = p.D, LK = p.L * p.K, QK = p.Q * p.K;
+  const int D = p.D, QK = p.Q * p.K;
   uint32_t *s_count = lds32;                                  // [kTileCells] entries per cell in this batch
   uint32_t *s_offs = s_count + kTileCells;                    // [kTileCells + 4] first entry of every cell, then the total
   uint32_t *s_list = s_offs + kTileCells + 4;                 // [kListCap] listed point ids

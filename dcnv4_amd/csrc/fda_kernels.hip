@@ -27,6 +27,93 @@ __device__ __forceinline__ Level load_level(const FdaLaunch &p, int l) {
   return lv;
 }
 
+// n / d for 0 <= n < 2^20 with inv = 1 / d
+__device__ __forceinline__ int fdiv20(int n, float inv) { return (int)(((float)n + 0.5f) * inv); }
+
+template <typename Tag>
+__device__ __forceinline__ float elem_f32(const void *base, size_t i) {
+  float f[1];
+  Pack<Tag, 1>::decode(reinterpret_cast<const typename RawWord<Tag::kBytes>::type *>(base)[i], f);
+  return f[0];
+}
+
+// Rows of the workgroup's (query, head) pairs into LDS as fp32, [pair][3 * L * K]: 2 L K locations, then L K logits.
+// Pair j is query row0 + j / heads_here, head g0 + j % heads_here.  Packed input: one tensor in the tensor dtype.
+// Split input (p.loc set): locations and logits are separate tensors, and every location passes through fp16 on its
+// way in, which is what the reference's module does before it packs them
+// (DCNv4_op/DCNv4/modules/flash_deform_attn.py:132-133: `.half()`, then `cat` with the logits).
+template <typename Tag>
+__device__ __forceinline__ void fda_stage_rows(float *lds, const FdaLaunch &p, int row0, int nrow, int g0, int heads_here) {
+  const int LK = p.L * p.K, row_len = 3 * LK, pairs = nrow * heads_here;
+  const float inv_h = 1.f / (float)heads_here;
+  if (p.loc == nullptr) {
+    if (heads_here == p.G) {
+      const bool vec16 = ((size_t)p.G * row_len * Tag::kBytes) % 16 == 0;
+      stage_rows_to_lds<Tag>(lds, (const char *)p.sla + (size_t)row0 * p.G * row_len * Tag::kBytes, pairs * row_len, vec16);
+    } else {
+      const float inv_len = 1.f / (float)row_len;
+      for (int i = threadIdx.x; i < pairs * row_len; i += blockDim.x) {
+        const int j = fdiv20(i, inv_len), e = i - j * row_len;
+        const int r = fdiv20(j, inv_h), gh = j - r * heads_here;
+        lds[i] = elem_f32<Tag>(p.sla, ((size_t)(row0 + r) * p.G + g0 + gh) * row_len + e);
+      }
+    }
+    return;
+  }
+  const float inv_2lk = 1.f / (float)(2 * LK), inv_lk = 1.f / (float)LK;
+  for (int i = threadIdx.x; i < pairs * 2 * LK; i += blockDim.x) {
+    const int j = fdiv20(i, inv_2lk), e = i - j * 2 * LK;
+    const int r = fdiv20(j, inv_h), gh = j - r * heads_here;
+    const size_t src = ((size_t)(row0 + r) * p.G + g0 + gh) * (2 * LK) + e;
+    const float v = p.loc_f32 ? reinterpret_cast<const float *>(p.loc)[src] : elem_f32<Tag>(p.loc, src);
+    lds[j * row_len + e] = (float)(_Float16)v;
+  }
+  for (int i = threadIdx.x; i < pairs * LK; i += blockDim.x) {
+    const int j = fdiv20(i, inv_lk), e = i - j * LK;
+    const int r = fdiv20(j, inv_h), gh = j - r * heads_here;
+    lds[j * row_len + 2 * LK + e] = elem_f32<Tag>(p.logits, ((size_t)(row0 + r) * p.G + g0 + gh) * LK + e);
+  }
+}
+
+// The gradient rows back to memory, same layouts; the gradient of a location passes through the fp16 rounding
+// unchanged (the derivative of a cast) and is written in the locations' dtype.
+template <typename Tag>
+__device__ __forceinline__ void fda_unstage_grads(const float *lds, const FdaLaunch &p, int row0, int nrow, int g0, int heads_here) {
+  typedef typename RawWord<Tag::kBytes>::type elem_t;
+  const int LK = p.L * p.K, row_len = 3 * LK, pairs = nrow * heads_here;
+  const float inv_h = 1.f / (float)heads_here;
+  if (p.loc == nullptr) {
+    if (heads_here == p.G) {
+      const bool vec16 = ((size_t)p.G * row_len * Tag::kBytes) % 16 == 0;
+      unstage_rows_from_lds<Tag>((char *)p.grad_sla + (size_t)row0 * p.G * row_len * Tag::kBytes, lds, pairs * row_len, vec16);
+    } else {
+      const float inv_len = 1.f / (float)row_len;
+      for (int i = threadIdx.x; i < pairs * row_len; i += blockDim.x) {
+        const int j = fdiv20(i, inv_len), e = i - j * row_len;
+        const int r = fdiv20(j, inv_h), gh = j - r * heads_here;
+        const float f[1] = {lds[i]};
+        reinterpret_cast<elem_t *>(p.grad_sla)[((size_t)(row0 + r) * p.G + g0 + gh) * row_len + e] = Pack<Tag, 1>::encode(f);
+      }
+    }
+    return;
+  }
+  const float inv_2lk = 1.f / (float)(2 * LK), inv_lk = 1.f / (float)LK;
+  for (int i = threadIdx.x; i < pairs * 2 * LK; i += blockDim.x) {
+    const int j = fdiv20(i, inv_2lk), e = i - j * 2 * LK;
+    const int r = fdiv20(j, inv_h), gh = j - r * heads_here;
+    const size_t dst = ((size_t)(row0 + r) * p.G + g0 + gh) * (2 * LK) + e;
+    const float f[1] = {lds[j * row_len + e]};
+    if (p.loc_f32) reinterpret_cast<float *>(p.grad_loc)[dst] = f[0];
+    else reinterpret_cast<elem_t *>(p.grad_loc)[dst] = Pack<Tag, 1>::encode(f);
+  }
+  for (int i = threadIdx.x; i < pairs * LK; i += blockDim.x) {
+    const int j = fdiv20(i, inv_lk), e = i - j * LK;
+    const int r = fdiv20(j, inv_h), gh = j - r * heads_here;
+    const float f[1] = {lds[j * row_len + 2 * LK + e]};
+    reinterpret_cast<elem_t *>(p.grad_logits)[((size_t)(row0 + r) * p.G + g0 + gh) * LK + e] = Pack<Tag, 1>::encode(f);
+  }
+}
+
 // ------------------------------------------------------------------------------- forward
 template <typename Tag, int CPT, int KT>
 __global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLaunch p) {
@@ -47,21 +134,11 @@ __global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLau
     const int q0 = rb * p.nq_block;
     nrow = min(p.nq_block, p.Q - q0);
     row0 = b * p.Q + q0;
-    typedef typename RawWord<Tag::kBytes>::type elem_t;
-    const elem_t *src = reinterpret_cast<const elem_t *>(p.sla) + ((size_t)row0 * p.G + g_fixed) * row_len;
-    for (int i = threadIdx.x; i < nrow * row_len; i += blockDim.x) {
-      const int r = i / row_len, e = i - r * row_len;
-      float f[1];
-      Pack<Tag, 1>::decode(src[(size_t)r * p.G * row_len + e], f);
-      lds[i] = f[0];
-    }
   } else {
     row0 = (int)blk * p.nq_block;
     nrow = min(p.nq_block, p.n_row - row0);
-    const int span = nrow * p.G * row_len;
-    const bool vec16 = ((size_t)p.G * row_len * Tag::kBytes) % 16 == 0;
-    stage_rows_to_lds<Tag>(lds, (const char *)p.sla + (size_t)row0 * p.G * row_len * Tag::kBytes, span, vec16);
   }
+  fda_stage_rows<Tag>(lds, p, row0, nrow, g_fixed, heads_here);
   __syncthreads();
 
   const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
@@ -131,8 +208,6 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
   const int LK = p.L * p.K, row_len = 3 * LK;
   const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
   int row0, nrow, heads_here = p.G, g_fixed = 0;
-  typedef typename RawWord<Tag::kBytes>::type elem_t;
-  const bool vec16 = ((size_t)p.G * row_len * Tag::kBytes) % 16 == 0;
   if (p.head_major) {       // one head per workgroup, workgroups ordered [image][head][block of queries] (see the forward kernel)
     const int blocks_per_image = (p.Q + p.nq_block - 1) / p.nq_block;
     const int rb = (int)(blk % (uint32_t)blocks_per_image), bg = (int)(blk / (uint32_t)blocks_per_image);
@@ -146,19 +221,8 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
     row0 = (int)blk * p.nq_block;
     nrow = min(p.nq_block, p.n_row - row0);
   }
-  const int span = nrow * heads_here * row_len;
   float *s_in = lds, *s_grad = lds + p.nq_block * heads_here * row_len;
-  if (p.head_major) {
-    const elem_t *src = reinterpret_cast<const elem_t *>(p.sla) + ((size_t)row0 * p.G + g_fixed) * row_len;
-    for (int i = threadIdx.x; i < span; i += blockDim.x) {
-      const int r = i / row_len, e = i - r * row_len;
-      float f[1];
-      Pack<Tag, 1>::decode(src[(size_t)r * p.G * row_len + e], f);
-      s_in[i] = f[0];
-    }
-  } else {
-    stage_rows_to_lds<Tag>(s_in, (const char *)p.sla + (size_t)row0 * p.G * row_len * Tag::kBytes, span, vec16);
-  }
+  fda_stage_rows<Tag>(s_in, p, row0, nrow, g_fixed, heads_here);
   __syncthreads();      // every slot of s_grad is written below: no clearing needed
 
   const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
@@ -278,16 +342,7 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
   }
   if constexpr (MODE == kFdaFallback) return;
   __syncthreads();
-  if (p.head_major) {
-    elem_t *dst = reinterpret_cast<elem_t *>(p.grad_sla) + ((size_t)row0 * p.G + g_fixed) * row_len;
-    for (int i = threadIdx.x; i < span; i += blockDim.x) {
-      const int r = i / row_len, e = i - r * row_len;
-      const float f[1] = {s_grad[i]};
-      dst[(size_t)r * p.G * row_len + e] = Pack<Tag, 1>::encode(f);
-    }
-  } else {
-    unstage_rows_from_lds<Tag>((char *)p.grad_sla + (size_t)row0 * p.G * row_len * Tag::kBytes, s_grad, span, vec16);
-  }
+  fda_unstage_grads<Tag>(s_grad, p, row0, nrow, g_fixed, heads_here);
 }
 
 template <typename Tag, int CPT, int MODE>      // MODE -1: forward

@@ -94,7 +94,13 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 struct FdaLaunch {
   const void *value;        // [n_img, N, G, D]
-  const void *sla;          // [n_row, G, 3*L*K]       n_row = images * Q
+  const void *sla;          // [n_row, G, 3*L*K]       n_row = images * Q (null when the rows come split)
+  // split rows: locations and logits as two tensors, the locations rounded through fp16 on their way in
+  const void *loc;          // [n_row, G, L*K*2], fp32 (loc_f32) or the tensor dtype; null when the rows come packed
+  const void *logits;       // [n_row, G, L*K], tensor dtype
+  void *grad_loc;           // like loc
+  void *grad_logits;        // like logits
+  int loc_f32;
   const void *grad_out;     // [n_row, G*D]
   void *out;                // [n_row, G*D]
   float *grad_value_acc;    // [n_img, N, G, D] fp32, zeroed
@@ -169,8 +175,27 @@ struct LnLaunch {
   float eps;
   int team;      // lanes per row: a power of two, <= 64
   int vpl;       // 16-byte vectors per lane: 1, 2, 4 or 8 (team * vpl * 16 bytes cover a row)
+  // backward
+  const void *grad_out;
+  void *grad_y, *grad_weight, *grad_bias, *grad_gamma;     // the three parameter gradients may be null
+  float *partial;   // [n_part][3][C] column sums of one workgroup each: grad_weight, grad_bias, grad_gamma
+  long long slab;   // consecutive rows per workgroup (a multiple of the rows one pass of the workgroup takes)
+  int n_part;       // workgroups of the backward
 };
+// Centre-feature blend: out = y * (1 - gate) + x * gate, gate[g] = sigmoid(<W[g,:], y> + b[g]) per (row, group).
+struct CfLaunch {
+  const void *y, *x, *weight, *bias;      // y, x [rows, C]; weight [G, C]; bias [G]
+  void *out;                              // forward
+  const void *grad_out;                   // backward
+  void *grad_y, *grad_x;
+  float *grad_logits;                     // [rows, G] fp32
+  long long rows;
+  int C, G, D;                            // D = C / G channels per group, a whole number of 16-byte vectors
+  int team, vpl;                          // as in LnLaunch
+};
+hipError_t launch_center_feature_blend(int dtype, const CfLaunch &p, bool backward, hipStream_t stream);
 hipError_t launch_layer_norm_residual(int dtype, const LnLaunch &p, hipStream_t stream);
+hipError_t launch_layer_norm_residual_backward(int dtype, const LnLaunch &p, hipStream_t stream);
 
 // Each returns hipSuccess or the launch error.  dtype: 0 fp32, 1 fp16, 2 bf16.
 hipError_t launch_depthwise_forward(int dtype, const DwLaunch &p, hipStream_t stream);

@@ -97,6 +97,167 @@ hipError_t launch_t(const LnLaunch &p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+
+// ------------------------------------------------------------------------------- backward
+// Gradients of out = residual + gamma * (xhat * weight + bias), xhat = (y - mean) * rstd, for grad_out g:
+//   grad_y      = rstd * (a - mean(a) - xhat * mean(a * xhat)),  a = g * gamma * weight      (row-wise)
+//   grad_weight = sum over rows of g * gamma * xhat
+//   grad_bias   = sum over rows of g * gamma
+//   grad_gamma  = sum over rows of g * (xhat * weight + bias)
+// (grad_residual is g itself.)  Same lane layout as the forward: a team owns a row and recomputes its
+// statistics from y in registers, so nothing is saved by the forward.  A workgroup walks a slab of
+// consecutive rows and keeps the three column sums of its lanes' channels in registers; at the end the teams
+// of the workgroup are added through LDS in a fixed order and the workgroup writes one row of partial sums;
+// a second kernel adds the partial rows in order.  No atomics: the result does not depend on scheduling.
+template <typename Tag, int VPL>
+__global__ void __launch_bounds__(kLnThreads) layer_norm_residual_backward_kernel(const LnLaunch p) {
+  extern __shared__ float s_cols[];                     // [teams][C]
+  constexpr int V = 16 / Tag::kBytes;
+  typedef Pack<Tag, V> pack;
+  typedef typename pack::raw_t raw_t;
+  const int team = p.team, nvec = p.C / V;
+  const int teams_per_block = kLnThreads / team;
+  const int lane_in_team = threadIdx.x & (team - 1), team_id = threadIdx.x / team;
+  const float inv_c = 1.f / (float)p.C;
+
+  float w[VPL][V], gam[VPL][V], b[VPL][V];
+  float dw[VPL][V], db[VPL][V], dg[VPL][V];
+  bool col_live[VPL];
+#pragma unroll
+  for (int u = 0; u < VPL; ++u) {
+    const int i = lane_in_team + u * team;
+    col_live[u] = i < nvec;
+#pragma unroll
+    for (int c = 0; c < V; ++c) { w[u][c] = 0.f; gam[u][c] = 1.f; b[u][c] = 0.f; dw[u][c] = db[u][c] = dg[u][c] = 0.f; }
+    if (col_live[u]) {
+      pack::decode(reinterpret_cast<const raw_t *>(p.weight)[i], w[u]);
+      if (p.gamma != nullptr) {
+        pack::decode(reinterpret_cast<const raw_t *>(p.gamma)[i], gam[u]);
+        pack::decode(reinterpret_cast<const raw_t *>(p.bias)[i], b[u]);
+      }
+    }
+  }
+
+  const long long row_begin = (long long)blockIdx.x * p.slab;
+  const long long row_end = row_begin + p.slab < p.rows ? row_begin + p.slab : p.rows;
+  for (long long row0 = row_begin; row0 < row_end; row0 += teams_per_block) {
+    const long long row = row0 + team_id;
+    const bool row_live = row < row_end;
+    const raw_t *y = reinterpret_cast<const raw_t *>(p.y) + row * nvec;
+    const raw_t *go = reinterpret_cast<const raw_t *>(p.grad_out) + row * nvec;
+    float v[VPL][V], g[VPL][V];
+    float sum = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      const int i = lane_in_team + u * team;
+      if (row_live && col_live[u]) {
+        pack::decode(y[i], v[u]);
+        pack::decode(go[i], g[u]);
+      } else {
+#pragma unroll
+        for (int c = 0; c < V; ++c) v[u][c] = g[u][c] = 0.f;
+      }
+#pragma unroll
+      for (int c = 0; c < V; ++c) sum += v[u][c];
+    }
+    for (int o = team >> 1; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
+    const float mean = sum * inv_c;
+    float sq = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u)
+      if (col_live[u])
+#pragma unroll
+        for (int c = 0; c < V; ++c) sq = fmaf(v[u][c] - mean, v[u][c] - mean, sq);
+    for (int o = team >> 1; o > 0; o >>= 1) sq += __shfl_xor(sq, o, kWave);
+    const float rstd = rsqrtf(sq * inv_c + p.eps);
+
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        const float xh = (row_live && col_live[u]) ? (v[u][c] - mean) * rstd : 0.f;
+        const float gg = g[u][c] * gam[u][c];               // g * gamma
+        const float a = gg * w[u][c];
+        s1 += a;
+        s2 = fmaf(a, xh, s2);
+        dw[u][c] = fmaf(gg, xh, dw[u][c]);
+        db[u][c] += gg;
+        dg[u][c] = fmaf(g[u][c], fmaf(xh, w[u][c], b[u][c]), dg[u][c]);
+        v[u][c] = xh;
+        g[u][c] = a;
+      }
+    }
+    for (int o = team >> 1; o > 0; o >>= 1) {
+      s1 += __shfl_xor(s1, o, kWave);
+      s2 += __shfl_xor(s2, o, kWave);
+    }
+    const float m1 = s1 * inv_c, m2 = s2 * inv_c;
+    if (row_live) {
+      raw_t *gy = reinterpret_cast<raw_t *>(p.grad_y) + row * nvec;
+#pragma unroll
+      for (int u = 0; u < VPL; ++u) {
+        if (!col_live[u]) continue;
+        float r[V];
+#pragma unroll
+        for (int c = 0; c < V; ++c) r[c] = rstd * (g[u][c] - m1 - v[u][c] * m2);
+        gy[lane_in_team + u * team] = pack::encode(r);
+      }
+    }
+  }
+
+  // teams of the workgroup, one quantity at a time, added in team order
+  float *part = p.partial + (size_t)blockIdx.x * 3 * p.C;
+#pragma unroll
+  for (int q = 0; q < 3; ++q) {
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      if (!col_live[u]) continue;
+      float *dst = s_cols + (size_t)team_id * p.C + (size_t)(lane_in_team + u * team) * V;
+#pragma unroll
+      for (int c = 0; c < V; ++c) dst[c] = q == 0 ? dw[u][c] : (q == 1 ? db[u][c] : dg[u][c]);
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < p.C; c += kLnThreads) {
+      float acc = 0.f;
+      for (int t = 0; t < teams_per_block; ++t) acc += s_cols[(size_t)t * p.C + c];
+      part[(size_t)q * p.C + c] = acc;
+    }
+  }
+}
+
+// partial [n_part][3][C] -> grad_weight, grad_bias, grad_gamma, added in the order of the workgroups
+template <typename Tag>
+__global__ void __launch_bounds__(kLnThreads) layer_norm_param_grad_kernel(const LnLaunch p) {
+  const int idx = blockIdx.x * kLnThreads + threadIdx.x;
+  if (idx >= 3 * p.C) return;
+  const int q = idx / p.C, c = idx - q * p.C;
+  void *dst = q == 0 ? p.grad_weight : (q == 1 ? p.grad_bias : p.grad_gamma);
+  if (dst == nullptr) return;
+  float acc = 0.f;
+  for (int w = 0; w < p.n_part; ++w) acc += p.partial[(size_t)w * 3 * p.C + idx];
+  const float f[1] = {acc};
+  reinterpret_cast<typename RawWord<Tag::kBytes>::type *>(dst)[c] = Pack<Tag, 1>::encode(f);
+}
+
+template <typename Tag>
+hipError_t launch_bwd_t(const LnLaunch &p, hipStream_t stream) {
+  const int teams_per_block = kLnThreads / p.team;
+  const dim3 grid((unsigned)p.n_part), block(kLnThreads);
+  const size_t lds = (size_t)teams_per_block * p.C * sizeof(float);
+  switch (p.vpl) {
+    case 1: hipLaunchKernelGGL((layer_norm_residual_backward_kernel<Tag, 1>), grid, block, lds, stream, p); break;
+    case 2: hipLaunchKernelGGL((layer_norm_residual_backward_kernel<Tag, 2>), grid, block, lds, stream, p); break;
+    case 4: hipLaunchKernelGGL((layer_norm_residual_backward_kernel<Tag, 4>), grid, block, lds, stream, p); break;
+    case 8: hipLaunchKernelGGL((layer_norm_residual_backward_kernel<Tag, 8>), grid, block, lds, stream, p); break;
+    default: return hipErrorInvalidValue;
+  }
+  if (hipError_t e = hipGetLastError()) return e;
+  hipLaunchKernelGGL((layer_norm_param_grad_kernel<Tag>), dim3((unsigned)((3 * p.C + kLnThreads - 1) / kLnThreads)), block, 0, stream, p);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 hipError_t launch_layer_norm_residual(int dtype, const LnLaunch &p, hipStream_t stream) {
@@ -104,6 +265,15 @@ hipError_t launch_layer_norm_residual(int dtype, const LnLaunch &p, hipStream_t 
     case F32::kCode: return launch_t<F32>(p, stream);
     case F16::kCode: return launch_t<F16>(p, stream);
     case BF16::kCode: return launch_t<BF16>(p, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_layer_norm_residual_backward(int dtype, const LnLaunch &p, hipStream_t stream) {
+  switch (dtype) {
+    case F32::kCode: return launch_bwd_t<F32>(p, stream);
+    case F16::kCode: return launch_bwd_t<F16>(p, stream);
+    case BF16::kCode: return launch_bwd_t<BF16>(p, stream);
   }
   return hipErrorInvalidValue;
 }

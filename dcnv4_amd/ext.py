@@ -271,3 +271,146 @@ def layer_norm_residual_forward(input, residual, weight, bias, gamma, eps):
                 gamma.data_ptr() if gamma is not None else None, output.data_ptr(), code, input.numel() // channels,
                 channels, float(eps), _stream()))
     return output
+
+
+def layer_norm_residual_backward(grad_output, input, weight, bias, gamma, eps, need_param_grads=True):
+    """Gradients of :func:`layer_norm_residual_forward` with respect to ``input``, ``weight``, ``bias`` and ``gamma``
+    (the gradient of the residual is ``grad_output`` itself): ``[grad_input, grad_weight, grad_bias, grad_gamma]``,
+    None for what is absent or not asked for."""
+    _check(grad_output, "grad_output", input.dtype)
+    _check(input, "input")
+    _check(weight, "weight", input.dtype)
+    if bias is not None:
+        _check(bias, "bias", input.dtype)
+    if gamma is not None:
+        _check(gamma, "gamma", input.dtype)
+        if bias is None:
+            raise RuntimeError("the gradient of gamma needs the bias of the normalisation")
+    if grad_output.shape != input.shape:
+        raise RuntimeError("grad_output must have the shape of the input")
+    code = _dtype_code(input, "input")
+    channels = input.shape[-1]
+    rows = input.numel() // max(channels, 1)
+    with torch.cuda.device(input.device):
+        grad_input = torch.empty_like(input)
+        new = lambda: torch.empty(channels, dtype=input.dtype, device=input.device)
+        grad_weight = new() if need_param_grads else None
+        grad_bias = new() if need_param_grads else None
+        grad_gamma = new() if (need_param_grads and gamma is not None) else None
+        if input.numel():
+            ws_bytes = _L.dcnv4_gfx950_layer_norm_residual_backward_workspace_bytes(code, rows, channels)
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=input.device)
+            ptr = lambda t: t.data_ptr() if t is not None else None
+            _lib.check(_L.dcnv4_gfx950_layer_norm_residual_backward(
+                grad_output.data_ptr(), input.data_ptr(), weight.data_ptr(), ptr(bias), ptr(gamma), grad_input.data_ptr(),
+                ptr(grad_weight), ptr(grad_bias), ptr(grad_gamma), ws.data_ptr(), ws_bytes, code, rows, channels,
+                float(eps), _stream()))
+    return [grad_input, grad_weight, grad_bias, grad_gamma]
+
+
+def _blend_common(sampled, projected, weight, bias):
+    _check(sampled, "sampled")
+    _check(projected, "projected", sampled.dtype)
+    _check(weight, "weight", sampled.dtype)
+    _check(bias, "bias", sampled.dtype)
+    channels = sampled.shape[-1]
+    groups = bias.numel()
+    if projected.shape != sampled.shape or tuple(weight.shape) != (groups, channels):
+        raise RuntimeError(f"projected must have the shape of sampled and weight be ({groups}, {channels})")
+    return _dtype_code(sampled, "sampled"), sampled.numel() // max(channels, 1), channels, groups
+
+
+def center_feature_blend_forward(sampled, projected, weight, bias):
+    """``sampled * (1 - gate) + projected * gate`` with ``gate = sigmoid(sampled @ weight.T + bias)`` per (pixel,
+    group), every channel using its group's gate (DCNv4_op/DCNv4/modules/dcnv4.py:142-147) in one kernel."""
+    code, rows, channels, groups = _blend_common(sampled, projected, weight, bias)
+    with torch.cuda.device(sampled.device):
+        output = torch.empty_like(sampled)
+        if sampled.numel():
+            _lib.check(_L.dcnv4_gfx950_center_feature_blend_forward(
+                sampled.data_ptr(), projected.data_ptr(), weight.data_ptr(), bias.data_ptr(), output.data_ptr(), code,
+                rows, channels, groups, _stream()))
+    return output
+
+
+def center_feature_blend_backward(grad_output, sampled, projected, weight, bias):
+    """``[grad_sampled, grad_projected, grad_gate_logits]``; the last is fp32 (rows, groups): ``grad_weight`` is
+    ``grad_gate_logits.T @ sampled`` and ``grad_bias`` its column sums."""
+    code, rows, channels, groups = _blend_common(sampled, projected, weight, bias)
+    _check(grad_output, "grad_output", sampled.dtype)
+    if grad_output.shape != sampled.shape:
+        raise RuntimeError("grad_output must have the shape of sampled")
+    with torch.cuda.device(sampled.device):
+        grad_sampled, grad_projected = torch.empty_like(sampled), torch.empty_like(sampled)
+        grad_logits = torch.empty((rows, groups), dtype=torch.float32, device=sampled.device)
+        if sampled.numel():
+            _lib.check(_L.dcnv4_gfx950_center_feature_blend_backward(
+                grad_output.data_ptr(), sampled.data_ptr(), projected.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                grad_sampled.data_ptr(), grad_projected.data_ptr(), grad_logits.data_ptr(), code, rows, channels,
+                groups, _stream()))
+    return [grad_sampled, grad_projected, grad_logits]
+
+
+def _fda_split_common(value, spatial_shapes, level_start_index, locations, logits, K):
+    _check(value, "value")
+    _check(spatial_shapes, "spatial_shapes", torch.int64)
+    _check(level_start_index, "level_start_index", torch.int64)
+    _check(locations, "sampling_locations")
+    _check(logits, "attention_logits", value.dtype)
+    if locations.dtype not in (torch.float32, value.dtype):
+        raise RuntimeError(f"sampling_locations must be float32 or {value.dtype}, got {locations.dtype}")
+    if value.dim() != 4:
+        raise RuntimeError("value must be (N, S, M, D)")
+    batch, spatial_size, num_heads, channels = value.shape
+    num_levels = spatial_shapes.shape[0]
+    num_query = logits.shape[1]
+    if level_start_index.numel() != num_levels:
+        raise RuntimeError("level_start_index must have one entry per level")
+    if tuple(logits.shape) != (batch, num_query, num_heads, num_levels * K) or \
+            locations.numel() != batch * num_query * num_heads * num_levels * K * 2:
+        raise RuntimeError(f"sampling_locations {tuple(locations.shape)} / attention_logits {tuple(logits.shape)} do not "
+                           f"match {(batch, num_query, num_heads, num_levels * K)}")
+    return batch, spatial_size, num_heads, channels, num_levels, num_query
+
+
+def flash_deform_attn_forward_split(value, spatial_shapes, level_start_index, sampling_locations, attention_logits,
+                                    im2col_step=64, K=8, d_stride=8, block_thread=0):
+    """:func:`flash_deform_attn_forward` on un-packed rows: ``sampling_locations`` (N, Lq, M, L*K*2) or (N, Lq, M, L,
+    K, 2) in float32 or the value's dtype, rounded through fp16 inside the kernel as the reference's module rounds
+    them before packing (DCNv4_op/DCNv4/modules/flash_deform_attn.py:132-133); ``attention_logits`` (N, Lq, M, L*K)."""
+    batch, spatial_size, num_heads, channels, num_levels, num_query = _fda_split_common(
+        value, spatial_shapes, level_start_index, sampling_locations, attention_logits, K)
+    code = _dtype_code(value, "value")
+    with torch.cuda.device(value.device):
+        output = torch.empty((batch, num_query, num_heads * channels), dtype=value.dtype, device=value.device)
+        _lib.check(_L.flash_deform_attn_gfx950_forward_split(
+            value.data_ptr(), spatial_shapes.data_ptr(), level_start_index.data_ptr(), sampling_locations.data_ptr(),
+            attention_logits.data_ptr(), output.data_ptr(), code, _DTYPES[sampling_locations.dtype], batch, spatial_size,
+            num_heads, channels, num_levels, num_query, int(K), int(im2col_step), _hint(d_stride), _hint(block_thread),
+            _stream()))
+    return output
+
+
+def flash_deform_attn_backward_split(value, spatial_shapes, level_start_index, sampling_locations, attention_logits,
+                                     grad_output, im2col_step=64, K=8, d_stride=2, block_thread=0):
+    """``[grad_value, grad_sampling_locations, grad_attention_logits]`` of :func:`flash_deform_attn_forward_split`."""
+    batch, spatial_size, num_heads, channels, num_levels, num_query = _fda_split_common(
+        value, spatial_shapes, level_start_index, sampling_locations, attention_logits, K)
+    _check(grad_output, "grad_output", value.dtype)
+    if grad_output.numel() != batch * num_query * num_heads * channels:
+        raise RuntimeError("grad_output shape does not match the output")
+    code = _dtype_code(value, "value")
+    with torch.cuda.device(value.device):
+        grad_value = torch.empty_like(value)
+        grad_loc = torch.empty_like(sampling_locations)
+        grad_logits = torch.empty_like(attention_logits)
+        ws_bytes = _L.flash_deform_attn_gfx950_backward_workspace_bytes(code, batch, spatial_size, num_heads, channels,
+                                                                        num_levels, num_query, int(K))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=value.device) if ws_bytes else None
+        _lib.check(_L.flash_deform_attn_gfx950_backward_split(
+            value.data_ptr(), spatial_shapes.data_ptr(), level_start_index.data_ptr(), sampling_locations.data_ptr(),
+            attention_logits.data_ptr(), grad_output.data_ptr(), grad_value.data_ptr(), grad_loc.data_ptr(),
+            grad_logits.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes, code,
+            _DTYPES[sampling_locations.dtype], batch, spatial_size, num_heads, channels, num_levels, num_query, int(K),
+            int(im2col_step), _hint(d_stride), _hint(block_thread), _stream()))
+    return [grad_value, grad_loc, grad_logits]

@@ -1,22 +1,34 @@
 """Centre-feature blend of a DCNv4 layer (DCNv4_op/DCNv4/modules/dcnv4.py:17-26,142-147): a per-(pixel, group) gate
 ``s = sigmoid(W y + b)`` computed from the sampled features ``y`` mixes them with the un-sampled projection ``x``:
-``out = y * (1 - s) + x * s``, every channel using its group's gate.
+``out = y * (1 - s) + x * s``, every channel using its group's gate.  Forward and backward each run as one kernel of
+libdcnv4_gfx950.so; the two parameter gradients are a matrix product of the kernel's logit gradients with ``y``.
 """
 import torch
-import torch.nn.functional as F
+from torch.autograd import Function
+from torch.autograd.function import once_differentiable
+
+from .. import ext
 
 
-def blend_reference(y, x, weight, bias):
-    """The blend composed from torch operators."""
-    groups = weight.shape[0]
-    gate = torch.sigmoid(F.linear(y, weight, bias))                       # (N,H,W,G)
-    gate = gate.unsqueeze(-1).expand(*gate.shape, y.shape[-1] // groups).reshape(y.shape)
-    return y * (1 - gate) + x * gate
-
-
-class CenterFeatureBlendFunction:
-    """apply(y (N,H,W,C), x (N,H,W,C), weight (G,C), bias (G,)) -> (N,H,W,C)."""
+class CenterFeatureBlendFunction(Function):
+    """apply(y (..., C), x (..., C), weight (G, C), bias (G,)) -> (..., C)."""
 
     @staticmethod
-    def apply(y, x, weight, bias):
-        return blend_reference(y, x, weight, bias)
+    def forward(ctx, y, x, weight, bias):
+        y, x, weight, bias = y.contiguous(), x.contiguous(), weight.contiguous(), bias.contiguous()
+        dtype = y.dtype
+        x, weight, bias = x.to(dtype), weight.to(dtype), bias.to(dtype)
+        ctx.save_for_backward(y, x, weight, bias)
+        return ext.center_feature_blend_forward(y, x, weight, bias)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_out):
+        y, x, weight, bias = ctx.saved_tensors
+        grad_y, grad_x, grad_logits = ext.center_feature_blend_backward(grad_out.contiguous().to(y.dtype), y, x, weight, bias)
+        grad_weight = grad_bias = None
+        if ctx.needs_input_grad[2]:
+            grad_weight = (grad_logits.t() @ y.reshape(-1, y.shape[-1]).float()).to(weight.dtype)
+        if ctx.needs_input_grad[3]:
+            grad_bias = grad_logits.sum(0).to(bias.dtype)
+        return grad_y, grad_x, grad_weight, grad_bias

@@ -1,25 +1,17 @@
 """``layer_norm_residual``: the tail of a FlashInternImage block, ``residual + gamma * LayerNorm(y)``
 (classification/models/flash_intern_image.py:425-440), as one kernel instead of the framework's three.
 
-The forward runs on the library's kernel whenever the tensors allow it (one floating dtype for activations and
-parameters, contiguous, channel count a whole number of 16-byte vectors, no autocast in force); otherwise, and for
-every backward, the same expression is evaluated with torch's own operators, so gradients are exactly autograd's.
+Forward and backward run on the library's kernels whenever the tensors allow it (one floating dtype for activations
+and parameters, contiguous, channel count a whole number of 16-byte vectors, no autocast in force); otherwise the
+expression is left to torch's own operators and autograd.
 """
 import torch
-import torch.nn.functional as F
 from torch.autograd import Function
 from torch.autograd.function import once_differentiable
 
 from .. import ext
 
 _MAX_VECTORS = 512
-
-
-def _compose(y, residual, weight, bias, gamma, eps):
-    out = F.layer_norm(y, (y.shape[-1],), weight, bias, eps)
-    if gamma is not None:
-        out = gamma * out
-    return out if residual is None else residual + out
 
 
 class LayerNormResidualFunction(Function):
@@ -35,11 +27,10 @@ class LayerNormResidualFunction(Function):
     def backward(ctx, grad_out):
         y, weight, bias, gamma = ctx.saved_tensors
         has_residual, has_gamma = ctx.has
-        leaves = [t.detach().requires_grad_(True) for t in ((y, weight, bias, gamma) if has_gamma else (y, weight, bias))]
-        with torch.enable_grad():
-            z = _compose(leaves[0], None, leaves[1], leaves[2], leaves[3] if has_gamma else None, ctx.eps)
-        grads = torch.autograd.grad(z, leaves, grad_out)
-        return (grads[0], grad_out if has_residual else None, grads[1], grads[2], grads[3] if has_gamma else None, None)
+        need_params = any(ctx.needs_input_grad[2:5])
+        grad_y, grad_weight, grad_bias, grad_gamma = ext.layer_norm_residual_backward(
+            grad_out.contiguous(), y, weight, bias, gamma if has_gamma else None, ctx.eps, need_params)
+        return (grad_y, grad_out if has_residual else None, grad_weight, grad_bias, grad_gamma if has_gamma else None, None)
 
 
 def _fusable(y, residual, weight, bias, gamma):

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define DCNV4_GFX950_ABI_VERSION 4
+#define DCNV4_GFX950_ABI_VERSION 5
 
 #define DCNV4_DTYPE_F32 0
 #define DCNV4_DTYPE_F16 1
@@ -175,6 +175,44 @@ int flash_deform_attn_gfx950_backward(const void *value, const int64_t *spatial_
                                       int block_thread, void *stream);
 
 /*
+ * Flash deformable attention with the rows of a (query, head) given as two tensors instead of one packed row.
+ * Replaces, together with the operator itself, the packing the reference's module does in front of it
+ * (DCNv4_op/DCNv4/modules/flash_deform_attn.py:132-133: `sampling_locations.flatten(-3).half()` followed by
+ * `torch.cat([sampling_locations, attention_weights], dim=-1)`, two passes over the largest tensor of the layer):
+ * every location passes through fp16 while it is staged, exactly as `.half()` rounds it, and is then used as the
+ * packed operator uses it.
+ *   sampling_locations  [batch, num_query, num_heads, num_levels*num_points*2] normalised (x,y); dtype
+ *                       `location_dtype`: DCNV4_DTYPE_F32 or the same as `dtype`
+ *   attention_logits    [batch, num_query, num_heads, num_levels*num_points], dtype `dtype`
+ *   other arguments and the result as flash_deform_attn_gfx950_forward
+ */
+int flash_deform_attn_gfx950_forward_split(const void *value, const int64_t *spatial_shapes,
+                                           const int64_t *level_start_index,
+                                           const void *sampling_locations, const void *attention_logits,
+                                           void *output, int dtype, int location_dtype, int batch,
+                                           int spatial_size, int num_heads, int head_channels,
+                                           int num_levels, int num_query, int num_points,
+                                           int im2col_step, int d_stride, int block_thread, void *stream);
+
+/*
+ * Backward of flash_deform_attn_gfx950_forward_split: flash_deform_attn_gfx950_backward with the row gradient
+ * written as two tensors (the split that autograd derives from the reference's `cat` and `.half()`,
+ * DCNv4_op/DCNv4/modules/flash_deform_attn.py:132-133; the cast passes the gradient through unchanged).
+ *   grad_sampling_locations like sampling_locations (dtype `location_dtype`), grad_attention_logits like
+ *   attention_logits; both fully overwritten.  Workspace as flash_deform_attn_gfx950_backward_workspace_bytes.
+ */
+int flash_deform_attn_gfx950_backward_split(const void *value, const int64_t *spatial_shapes,
+                                            const int64_t *level_start_index,
+                                            const void *sampling_locations, const void *attention_logits,
+                                            const void *grad_output, void *grad_value,
+                                            void *grad_sampling_locations, void *grad_attention_logits,
+                                            void *workspace, size_t workspace_bytes, int dtype,
+                                            int location_dtype, int batch, int spatial_size, int num_heads,
+                                            int head_channels, int num_levels, int num_query,
+                                            int num_points, int im2col_step, int d_stride,
+                                            int block_thread, void *stream);
+
+/*
  * Depthwise convolution over channels-last tensors, stride 1, dilation 1, square kernel of size
  * 1, 3, 5 or 7: the `offset_mask_dw` layer of a DCNv4 block.  Replaces the nn.Conv2d call and the
  * NHWC -> NCHW -> NHWC permutes around it (DCNv4_op/DCNv4/modules/dcnv4.py:67-75 and :121-123).
@@ -224,6 +262,53 @@ int dcnv4_gfx950_layer_norm_residual_forward(const void *input, const void *resi
                                              const void *bias, const void *gamma, void *output,
                                              int dtype, long long rows, int channels, float eps,
                                              void *stream);
+
+/*
+ * Bytes of device scratch dcnv4_gfx950_layer_norm_residual_backward needs (partial column sums of the parameter
+ * gradients, one row per workgroup; no initialisation needed).
+ */
+size_t dcnv4_gfx950_layer_norm_residual_backward_workspace_bytes(int dtype, long long rows, int channels);
+
+/*
+ * Backward of dcnv4_gfx950_layer_norm_residual_forward: what autograd derives for the block tail
+ * `x + drop_path(gamma1 * norm1(dcn(x)))` (classification/models/flash_intern_image.py:425-440) through
+ * layer_norm, the broadcast multiply and the add, in two kernels.  The row statistics are recomputed from
+ * `input`; the parameter gradients are column sums added in a fixed order (no atomics).
+ *   grad_output, input, grad_input  [rows, channels];  weight, bias, gamma  [channels]
+ *   grad_weight, grad_bias, grad_gamma  [channels], each may be NULL (not wanted)
+ *   bias is needed only with gamma (it enters grad_gamma); gamma may be NULL.
+ *   The gradient of the residual is grad_output itself and is not written.
+ */
+int dcnv4_gfx950_layer_norm_residual_backward(const void *grad_output, const void *input, const void *weight,
+                                              const void *bias, const void *gamma, void *grad_input,
+                                              void *grad_weight, void *grad_bias, void *grad_gamma,
+                                              void *workspace, size_t workspace_bytes, int dtype,
+                                              long long rows, int channels, float eps, void *stream);
+
+/*
+ * Centre-feature blend of a DCNv4 layer (DCNv4_op/DCNv4/modules/dcnv4.py:17-26 CenterFeatureScaleModule and
+ * :142-147): gate = sigmoid(sampled . weight^T + bias) per (row, group), then
+ * output = sampled * (1 - gate) + projected * gate with every channel using its group's gate - the reference's
+ * linear, sigmoid, `repeat`, and three element-wise kernels in one pass.
+ *   sampled, projected, output  [rows, channels];  weight [groups, channels];  bias [groups]
+ *   channels / groups must be a whole number of 16-byte vectors.
+ */
+int dcnv4_gfx950_center_feature_blend_forward(const void *sampled, const void *projected, const void *weight,
+                                              const void *bias, void *output, int dtype, long long rows,
+                                              int channels, int groups, void *stream);
+
+/*
+ * Backward of the centre-feature blend (autograd through DCNv4_op/DCNv4/modules/dcnv4.py:142-147).
+ *   grad_sampled, grad_projected  [rows, channels], fully overwritten
+ *   grad_gate_logits  [rows, groups] fp32: the gradient of the gates' pre-sigmoid values; the parameter
+ *   gradients are grad_weight = grad_gate_logits^T . sampled and grad_bias = its column sums, a plain matrix
+ *   product left to the caller's GEMM library.
+ */
+int dcnv4_gfx950_center_feature_blend_backward(const void *grad_output, const void *sampled,
+                                               const void *projected, const void *weight, const void *bias,
+                                               void *grad_sampled, void *grad_projected,
+                                               float *grad_gate_logits, int dtype, long long rows,
+                                               int channels, int groups, void *stream);
 
 #ifdef __cplusplus
 }

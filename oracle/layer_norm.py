@@ -17,3 +17,23 @@ def layer_norm_residual(y, weight, bias, eps, gamma=None, residual=None):
     if residual is not None:
         out = out + np.asarray(residual, dtype=np.float64)
     return out
+
+
+def layer_norm_residual_backward(grad_out, y, weight, bias, eps, gamma=None):
+    """Gradients of ``layer_norm_residual`` for ``grad_out``: (grad_y, grad_weight, grad_bias, grad_gamma or None); the
+    gradient of the residual is ``grad_out`` itself.  Chain rule through out = residual + gamma * (xhat * weight + bias),
+    xhat = (y - mean) / sqrt(var + eps): what autograd derives for flash_intern_image.py:425-440.  Pinned against
+    torch autograd and finite differences in tests/test_oracle_pins.py."""
+    g = np.asarray(grad_out, dtype=np.float64)
+    y = np.asarray(y, dtype=np.float64)
+    w = np.asarray(weight, dtype=np.float64)
+    b = np.asarray(bias, dtype=np.float64)
+    mean = y.mean(axis=-1, keepdims=True)
+    rstd = 1.0 / np.sqrt(((y - mean) ** 2).mean(axis=-1, keepdims=True) + eps)
+    xhat = (y - mean) * rstd
+    gg = g if gamma is None else g * np.asarray(gamma, dtype=np.float64)       # gradient of the normalisation's output
+    a = gg * w
+    grad_y = rstd * (a - a.mean(axis=-1, keepdims=True) - xhat * (a * xhat).mean(axis=-1, keepdims=True))
+    flat = lambda t: t.reshape(-1, t.shape[-1]).sum(axis=0)
+    grad_gamma = None if gamma is None else flat(g * (xhat * w + b))
+    return grad_y, flat(gg * xhat), flat(gg), grad_gamma

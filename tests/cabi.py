@@ -136,3 +136,68 @@ def dcnv4_backward_static_scratch(value, om, go, geom, G, D, scale, rc=0, softma
                                                  om.shape[-1], softmax, 0, 0, _stream())
     _lib.check(rc_)
     return gv, gom
+
+
+def layer_norm_residual_backward(go, y, weight, bias, gamma, eps, want_params=True):
+    L = _lib.load()
+    C = y.shape[-1]
+    rows = y.numel() // C
+    gy = torch.full_like(y, float("nan"))
+    new = lambda: torch.full((C,), float("nan"), dtype=y.dtype, device=y.device)
+    gw, gb = (new(), new()) if want_params else (None, None)
+    gg = new() if (want_params and gamma is not None) else None
+    nbytes = L.dcnv4_gfx950_layer_norm_residual_backward_workspace_bytes(CODES[y.dtype], rows, C)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=y.device)
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    _lib.check(L.dcnv4_gfx950_layer_norm_residual_backward(go.data_ptr(), y.data_ptr(), weight.data_ptr(), ptr(bias), ptr(gamma),
+                                                            gy.data_ptr(), ptr(gw), ptr(gb), ptr(gg), ws.data_ptr(), nbytes,
+                                                            CODES[y.dtype], rows, C, float(eps), _stream()))
+    return gy, gw, gb, gg
+
+
+def center_feature_blend_forward(y, x, weight, bias):
+    L = _lib.load()
+    C = y.shape[-1]
+    out = torch.full_like(y, float("nan"))
+    _lib.check(L.dcnv4_gfx950_center_feature_blend_forward(y.data_ptr(), x.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                                            out.data_ptr(), CODES[y.dtype], y.numel() // C, C, bias.numel(), _stream()))
+    return out
+
+
+def center_feature_blend_backward(go, y, x, weight, bias):
+    L = _lib.load()
+    C = y.shape[-1]
+    rows = y.numel() // C
+    gy, gx = torch.full_like(y, float("nan")), torch.full_like(y, float("nan"))
+    gl = torch.full((rows, bias.numel()), float("nan"), dtype=torch.float32, device=y.device)
+    _lib.check(L.dcnv4_gfx950_center_feature_blend_backward(go.data_ptr(), y.data_ptr(), x.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                                             gy.data_ptr(), gx.data_ptr(), gl.data_ptr(), CODES[y.dtype], rows, C,
+                                                             bias.numel(), _stream()))
+    return gy, gx, gl
+
+
+def fda_forward_split(value, shapes, starts, loc, logits, K, im2col_step=64):
+    L = _lib.load()
+    B, N, G, D = value.shape
+    Q = logits.shape[1]
+    out = torch.full((B, Q, G * D), float("nan"), dtype=value.dtype, device=value.device)
+    _lib.check(L.flash_deform_attn_gfx950_forward_split(value.data_ptr(), shapes.data_ptr(), starts.data_ptr(), loc.data_ptr(),
+                                                         logits.data_ptr(), out.data_ptr(), CODES[value.dtype], CODES[loc.dtype], B, N,
+                                                         G, D, shapes.shape[0], Q, K, im2col_step, 0, 0, _stream()))
+    return out
+
+
+def fda_backward_split(value, shapes, starts, loc, logits, go, K, im2col_step=64):
+    L = _lib.load()
+    B, N, G, D = value.shape
+    Q = logits.shape[1]
+    gv = torch.full_like(value, float("nan"))
+    gloc = torch.full_like(loc, float("nan"))
+    glog = torch.full_like(logits, float("nan"))
+    nbytes = L.flash_deform_attn_gfx950_backward_workspace_bytes(CODES[value.dtype], B, N, G, D, shapes.shape[0], Q, K)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=value.device)
+    _lib.check(L.flash_deform_attn_gfx950_backward_split(value.data_ptr(), shapes.data_ptr(), starts.data_ptr(), loc.data_ptr(),
+                                                          logits.data_ptr(), go.data_ptr(), gv.data_ptr(), gloc.data_ptr(),
+                                                          glog.data_ptr(), ws.data_ptr(), nbytes, CODES[value.dtype], CODES[loc.dtype],
+                                                          B, N, G, D, shapes.shape[0], Q, K, im2col_step, 0, 0, _stream()))
+    return gv, gloc, glog

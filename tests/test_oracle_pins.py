@@ -340,3 +340,66 @@ def test_layer_norm_oracle_matches_torch_and_normalises_rows():
     np.testing.assert_allclose((plain ** 2).mean(-1), 1.0, rtol=1e-12)          # biased variance
     shifted = layer_norm.layer_norm_residual(y.numpy() + 100.0, np.ones(24), np.zeros(24), 0.0)
     np.testing.assert_allclose(shifted, plain, atol=1e-9)
+
+
+@pytest.mark.parametrize("use_gamma", [True, False])
+def test_layer_norm_backward_oracle_matches_autograd_and_finite_differences(use_gamma):
+    from oracle import layer_norm
+    g = torch.Generator().manual_seed(22)
+    y = (torch.randn(4, 6, 24, dtype=torch.float64, generator=g) * 2 + 0.7).requires_grad_(True)
+    w, b, gamma = (torch.randn(24, dtype=torch.float64, generator=g).requires_grad_(True) for _ in range(3))
+    res = torch.randn(4, 6, 24, dtype=torch.float64, generator=g).requires_grad_(True)
+    go = torch.randn(4, 6, 24, dtype=torch.float64, generator=g)
+    z = F.layer_norm(y, (24,), w, b, 1e-6)
+    out = res + (gamma * z if use_gamma else z)
+    leaves = [y, w, b, res] + ([gamma] if use_gamma else [])
+    want = torch.autograd.grad(out, leaves, go)
+    gy, gw, gb, gg = layer_norm.layer_norm_residual_backward(go.numpy(), y.detach().numpy(), w.detach().numpy(), b.detach().numpy(),
+                                                             1e-6, gamma.detach().numpy() if use_gamma else None)
+    np.testing.assert_allclose(gy, want[0].numpy(), rtol=1e-10, atol=1e-11)
+    np.testing.assert_allclose(gw, want[1].numpy(), rtol=1e-10, atol=1e-11)
+    np.testing.assert_allclose(gb, want[2].numpy(), rtol=1e-10, atol=1e-11)
+    np.testing.assert_array_equal(want[3].numpy(), go.numpy())          # the residual's gradient is grad_out itself
+    if use_gamma:
+        np.testing.assert_allclose(gg, want[4].numpy(), rtol=1e-10, atol=1e-11)
+    else:
+        assert gg is None
+    # central differences of the oracle's own forward along a random direction of y
+    d = torch.randn(4, 6, 24, dtype=torch.float64, generator=g).numpy()
+    f = lambda t: (layer_norm.layer_norm_residual(t, w.detach().numpy(), b.detach().numpy(), 1e-6,
+                                                  gamma.detach().numpy() if use_gamma else None) * go.numpy()).sum()
+    h = 1e-6
+    num = (f(y.detach().numpy() + h * d) - f(y.detach().numpy() - h * d)) / (2 * h)
+    assert abs(num - (gy * d).sum()) < 1e-6 * max(1.0, abs(num))
+    # rows of grad_y are orthogonal to the constant vector and to the normalised row (the two directions LayerNorm ignores)
+    assert np.abs(gy.sum(-1)).max() < 1e-10
+
+
+def test_center_feature_oracle_matches_the_reference_expression_autograd_and_limits():
+    """The expression of DCNv4_op/DCNv4/modules/dcnv4.py:17-26,142-147 written with the reference's own torch calls."""
+    from oracle import center_feature
+    g = torch.Generator().manual_seed(23)
+    y = torch.randn(2, 3, 4, 32, dtype=torch.float64, generator=g).requires_grad_(True)
+    x = torch.randn(2, 3, 4, 32, dtype=torch.float64, generator=g).requires_grad_(True)
+    w = (0.4 * torch.randn(2, 32, dtype=torch.float64, generator=g)).requires_grad_(True)
+    b = torch.randn(2, dtype=torch.float64, generator=g).requires_grad_(True)
+    go = torch.randn(2, 3, 4, 32, dtype=torch.float64, generator=g)
+    s = F.linear(y, weight=w, bias=b).sigmoid()
+    s = s[..., None].repeat(1, 1, 1, 1, 32 // 2).flatten(-2)
+    want = y * (1 - s) + x * s
+    np_ = lambda t: t.detach().numpy()
+    got = center_feature.blend_forward(np_(y), np_(x), np_(w), np_(b))
+    np.testing.assert_allclose(got, np_(want), rtol=1e-12, atol=1e-12)
+    wy, wx, ww, wb = torch.autograd.grad(want, [y, x, w, b], go)
+    gy, gx, gw, gb, gl = center_feature.blend_backward(go.numpy(), np_(y), np_(x), np_(w), np_(b))
+    for a, e in ((gy, wy), (gx, wx), (gw, ww), (gb, wb)):
+        np.testing.assert_allclose(a, e.numpy(), rtol=1e-10, atol=1e-11)
+    np.testing.assert_allclose(gl.reshape(-1, 2).sum(0), gb, rtol=1e-12)
+    # limits: a very negative bias closes the gate (out = y), a very positive one opens it (out = x)
+    np.testing.assert_allclose(center_feature.blend_forward(np_(y), np_(x), np_(w), np.full(2, -80.0)), np_(y), atol=1e-12)
+    np.testing.assert_allclose(center_feature.blend_forward(np_(y), np_(x), np_(w), np.full(2, 80.0)), np_(x), atol=1e-12)
+    # one-hot weight on a channel of group 1 only: group 0's gate is sigmoid(b0) everywhere
+    w1 = np.zeros((2, 32)); w1[1, 20] = 1.0
+    out = center_feature.blend_forward(np_(y), np_(x), w1, np.array([0.3, 0.0]))
+    s0 = 1 / (1 + np.exp(-0.3))
+    np.testing.assert_allclose(out[..., :16], np_(y)[..., :16] * (1 - s0) + np_(x)[..., :16] * s0, rtol=1e-12)
