@@ -39,6 +39,8 @@ CFG3 = [("L-dense1", 2, 256, 256, 160, 10), ("L-dense2", 2, 128, 128, 320, 20),
 CFG5 = [("B-stage1", 128, 56, 56, 112, 7), ("B-stage2", 128, 28, 28, 224, 14),
         ("B-stage3", 128, 14, 14, 448, 28), ("B-stage4", 128, 7, 7, 896, 56)]
 CFG4_SHAPES = [(128, 128), (64, 64), (32, 32), (16, 16)]
+# the shape of the reference's only timing note (DCNv4_op/scripts/test_dcnv4_bwd.py:94-106: 64 x 56 x 56 x 128, 4 groups of 32)
+DEVNOTE = [("ref-note-56x56-C128-G4", 64, 56, 56, 128, 4)]
 
 
 def p_pad(G, K=9):
@@ -130,13 +132,18 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / iters      # ms per call
 
+    def stream_ceiling(mb, iters, warm):
+        """GB/s (bytes read + bytes written) of the library's own streaming copy over `mb` MB."""
+        n = int(mb * 1e6) // 16 * 4
+        src, dst = torch.randn(n, device=dev), torch.empty(n, device=dev)
+        ms = time_op(lambda: ext.stream_copy(src, dst), iters, warm=warm)
+        return ms, n * 4, 2 * n * 4 / (ms * 1e-3) / 1e9
+
     if args.only_op and args.only_op.startswith("copy:"):
         # plain copy of known size: calibrates FETCH_SIZE / WRITE_SIZE counters and shows the HBM ceiling
-        n = int(float(args.only_op.split(":")[1]) * 1e6) // 4
-        src, dst = torch.randn(n, device=dev), torch.empty(n, device=dev)
-        ms = time_op(lambda: dst.copy_(src), args.steps, warm=args.warmup)
-        print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "read_MB": n * 4 / 1e6, "write_MB": n * 4 / 1e6,
-                          "GBps_read_plus_write": round(2 * n * 4 / (ms * 1e-3) / 1e9, 1)}))
+        ms, nbytes, gbps = stream_ceiling(float(args.only_op.split(":")[1]), args.steps, args.warmup)
+        print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "read_MB": nbytes / 1e6, "write_MB": nbytes / 1e6,
+                          "GBps_read_plus_write": round(gbps, 1)}))
         return
 
     def fda_inputs(dtype):
@@ -190,7 +197,7 @@ def main():
                                   "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)}))
                 return
             sys.exit(f"--only-op {args.only_op}: no such shape")
-        for table, off in ((CFG2, 3.0), (CFG3, 4.0), (CFG5, 3.0)):
+        for table, off in ((CFG2, 3.0), (CFG3, 4.0), (CFG5, 3.0), (DEVNOTE, 3.0)):
             for name, B, H, W, C, G in table:
                 if name != shape_name:
                     continue
@@ -243,6 +250,12 @@ def main():
     if not args.no_detail:
         for name, B, H, W, C, G in CFG3:
             t = dcn_inputs(B, H, W, C, G, torch.float16, 4.0)
+            fb, bb = dcn_bytes(2, B, H, W, C, G)
+            add("dcnv4_fwd", name, torch.float16, time_op(lambda: dcn_fwd(t, G, C), args.op_iters), fb)
+            add("dcnv4_bwd", name, torch.float16, time_op(lambda: dcn_bwd(t, G, C), args.op_iters), bb)
+            del t
+        for name, B, H, W, C, G in DEVNOTE:
+            t = dcn_inputs(B, H, W, C, G, torch.float16, 3.0)
             fb, bb = dcn_bytes(2, B, H, W, C, G)
             add("dcnv4_fwd", name, torch.float16, time_op(lambda: dcn_fwd(t, G, C), args.op_iters), fb)
             add("dcnv4_bwd", name, torch.float16, time_op(lambda: dcn_bwd(t, G, C), args.op_iters), bb)
@@ -314,42 +327,74 @@ def main():
     # ------------------------------------------------------------------ roofline of the dominant operator
     dom = max(step_ops, key=lambda d: d["ms"])
     dom_bytes = dom["MB"] * 1e6
+    _, _, ceiling = stream_ceiling(512, 50, 10)
     roofline = {
         "bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
         "traffic": MEASURED_TRAFFIC_BYTES.get(f'{dom["op"]}:{dom["shape"]}:{dom["dtype"]}'),
         "kernel": f'{dom["op"]} {dom["shape"]} {dom["dtype"]}', "ms": dom["ms"],
         "algorithmic_bytes": int(dom_bytes),
-        "note": "HIP events around whole operator calls (backward = state reset + grad_offset_mask kernel + tiled grad_value kernel + fallback); traffic = rocprofv3 FETCH_SIZE/WRITE_SIZE per call, scaled by a copy of known size (profiles/)",
+        "measured_ceiling": round(ceiling, 1), "frac_of_measured_ceiling": round(dom["GBps"] / ceiling, 4),
+        "note": "HIP events around whole operator calls (backward = state reset + grad_offset_mask kernel + tiled grad_value kernel); measured_ceiling = read+write GB/s of the library's own streaming copy over 512 MB in this run; traffic = rocprofv3 FETCH_SIZE/WRITE_SIZE per call, scaled by a copy of known size (profiles/)",
     }
 
     # ------------------------------------------------------------------ CPU baseline (rank 0, bounded sample)
+    # The pure-PyTorch grid_sample formulation on the host cores: 2 warm-ups, median of 5, forward and
+    # forward+backward separately.  `value` is the forward+backward rate over the step's own four shapes on a batch
+    # sample; `detail` adds configs[0] (its full size, batch 2) and one image of the attention configuration.
     cpu = None
     if not args.no_cpu_baseline:
+        import statistics
         from oracle import torch_core
         cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
         torch.set_num_threads(cores)
+
+        def cpu_times(fwd_fn, leaves, go):
+            def f():
+                with torch.no_grad():
+                    fwd_fn()
+
+            def fb():
+                out = fwd_fn()
+                out.backward(go)
+                for t in leaves:
+                    t.grad = None
+            res = []
+            for fn in (f, fb):
+                for _ in range(2):
+                    fn()
+                ts = []
+                for _ in range(5):
+                    t0 = time.perf_counter()
+                    fn()
+                    ts.append(time.perf_counter() - t0)
+                res.append(statistics.median(ts))
+            return res      # seconds: forward, forward+backward
+
+        cpu_detail = []
         Bc = 8
         cpu_bytes, cpu_time = 0, 0.0
-        for name, B, H, W, C, G in CFG2:
-            v, om, go = (x.cpu().float()[:Bc].contiguous() for x in dcn_inputs(Bc, H, W, C, G, torch.float32, 3.0))
-            v.requires_grad_(True)
-            om.requires_grad_(True)
-
-            def run():
-                out = torch_core.dcnv4_core_torch(v, om, *GEOM, G, C // G, 1.0)
-                out.backward(go)
-                v.grad = om.grad = None
-            run()
-            reps = 3
-            t0 = time.perf_counter()
-            for _ in range(reps):
-                run()
-            cpu_time += (time.perf_counter() - t0) / reps
-            cpu_bytes += sum(dcn_bytes(4, Bc, H, W, C, G))
+        for cfg_name, table, Bs, off in (("cfg1", [("56x56 C64 G4", 2, 56, 56, 64, 4)], None, 2.0), ("cfg2", CFG2, Bc, 3.0)):
+            for name, B, H, W, C, G in table:
+                Bn = B if Bs is None else Bs
+                v, om, go = (x.cpu().float().contiguous() for x in dcn_inputs(Bn, H, W, C, G, torch.float32, off))
+                v.requires_grad_(True)
+                om.requires_grad_(True)
+                tf, tfb = cpu_times(lambda: torch_core.dcnv4_core_torch(v, om, *GEOM, G, C // G, 1.0), (v, om), go)
+                cpu_detail.append({"config": cfg_name, "shape": name, "batch": Bn, "fwd_ms": round(tf * 1e3, 2), "fwd_bwd_ms": round(tfb * 1e3, 2)})
+                if cfg_name == "cfg2":
+                    cpu_time += tfb
+                    cpu_bytes += sum(dcn_bytes(4, Bn, H, W, C, G))
+        (B4, N4, G4, D4, L4, K4), shapes4, starts4, v4, sla4, go4 = fda_inputs(torch.float32)
+        v1, s1, g1 = v4[:1].cpu().contiguous().requires_grad_(True), sla4[:1].cpu().contiguous().requires_grad_(True), go4[:1].cpu().contiguous()
+        tf, tfb = cpu_times(lambda: torch_core.msda_core_torch(v1, CFG4_SHAPES, [int(x) for x in starts4.cpu()], s1, K4), (v1, s1), g1)
+        cpu_detail.append({"config": "cfg4", "shape": "DETR-enc 4lvl Q=21760", "batch": 1, "fwd_ms": round(tf * 1e3, 2), "fwd_bwd_ms": round(tfb * 1e3, 2)})
+        del v4, sla4, go4
         cpu = {"value": round(cpu_bytes / cpu_time / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-               "sample": f"DCNv4 fwd+bwd, four FlashInternImage-T stage shapes at batch {Bc} (of 64), fp32, "
-                         f"torch grid_sample formulation + autograd, {cpu_time * 1e3:.0f} ms per pass"}
+               "sample": f"DCNv4 fwd+bwd, four FlashInternImage-T stage shapes at batch {Bc} (of 64), fp32, torch grid_sample "
+                         f"formulation + autograd, median of 5 after 2 warm-ups, {cpu_time * 1e3:.0f} ms per pass; detail: "
+                         "configs[0] at its full batch 2, configs[1] at batch 8, configs[3] one image of 4",
+               "detail": cpu_detail}
 
     line = {
         "metric": "DCNv4 fwd+bwd achieved HBM GB/s (algorithmic bytes / time)", "value": round(value, 1), "unit": "GB/s",

@@ -38,6 +38,7 @@ SIGNATURES = {
     "dcnv4_gfx950_layer_norm_residual_backward_workspace_bytes": (_sz, [_i, ctypes.c_longlong, _i]),
     "dcnv4_gfx950_layer_norm_residual_backward": (_i, [_vp] * 10 + [_sz, _i, ctypes.c_longlong, _i, _f, _vp]),
     "dcnv4_gfx950_center_feature_blend_forward": (_i, [_vp] * 5 + [_i, ctypes.c_longlong, _i, _i, _vp]),
+    "dcnv4_gfx950_stream_copy": (_i, [_vp, _vp, _sz, _vp]),
     "dcnv4_gfx950_center_feature_blend_backward": (_i, [_vp] * 8 + [_i, ctypes.c_longlong, _i, _i, _vp]),
 }
 

@@ -89,6 +89,18 @@ __global__ void __launch_bounds__(256) narrow_kernel(const float *src, void *dst
   }
 }
 
+// Plain streaming copy, four 16-byte vectors per lane: the yardstick for what the memory system sustains.
+__global__ void __launch_bounds__(256) stream_copy_kernel(const u32x4 *src, u32x4 *dst, size_t n16) {
+  const size_t base = (size_t)blockIdx.x * (256 * 4) + threadIdx.x;
+  u32x4 v[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+    if (base + u * 256 < n16) v[u] = __builtin_nontemporal_load(src + base + u * 256);
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+    if (base + u * 256 < n16) __builtin_nontemporal_store(v[u], dst + base + u * 256);
+}
+
 int grid_for(size_t work_items) {
   const size_t blocks = (work_items + 255) / 256;
   return (int)std::min<size_t>(std::max<size_t>(blocks, 1), 256 * 32);
@@ -130,6 +142,7 @@ struct LaunchOptions {
   int scatter = kOptAuto;      // attention grad_value: binned LDS accumulation / global atomics
   int reach = -1;              // input pixels around a reference point that the tiled gathers stage; -1: default
   int tile = 0;                // largest side of a grad_value tile (8, 16, 32); 0: default
+  int gather_tile = 0;         // largest side of an output tile of the tiled gathers (4, 8, 16); 0: default (16)
   int fda_order = kOptAuto;    // attention forward: 1 whole query rows per workgroup, 2 one head per workgroup
 };
 thread_local LaunchOptions g_opt;
@@ -199,27 +212,42 @@ bool plan_gather_tiles(DcnLaunch *L, int s) {
   if (nv != 1 && nv != 2 && nv != 4 && nv != 8) return false;
   if (L->Kp > 64) return false;
   L->gt_lpg = nv >= 4 ? 2 : 1;      // wide groups: two lanes each, for twice the waves per workgroup
-  const int Ho = L->Q / L->Wo, Wo = L->Wo, R = L->gt_reach;
+  const int Ho = L->Q / L->Wo, Wo = L->Wo;
   auto even_split = [](int extent, int cap) { const int n = (extent + cap - 1) / cap; return (extent + n - 1) / n; };
-  // two workgroups per CU when the window allows it, so that one stages while the other computes
-  const size_t budgets[2] = {kMaxLdsPerWorkgroup / 2 - 512, kMaxLdsPerWorkgroup - 1024};
-  for (size_t budget : budgets) {
-    for (int cap_h = 16, cap_w = 16; cap_h >= 4 && cap_w >= 4;) {
+  const int cap0 = g_opt.gather_tile > 0 ? g_opt.gather_tile : 16;
+  // The largest tile and group chunk that fit `budget` bytes of LDS with `reach`, with at least `min_lanes` lanes.
+  auto fit = [&](size_t budget, int reach, int min_lanes) {
+    for (int cap_h = cap0, cap_w = cap0; cap_h >= 4 && cap_w >= 4;) {
+      L->gt_reach = reach;
       L->gt_h = even_split(Ho, cap_h);
       L->gt_w = even_split(Wo, cap_w);
-      L->gt_wh = std::min((L->gt_h - 1) * L->sh + 2 * R + 1, L->H + 2);
-      L->gt_ww = std::min((L->gt_w - 1) * L->sw + 2 * R + 1, L->W + 2);
+      L->gt_wh = std::min((L->gt_h - 1) * L->sh + 2 * reach + 1, L->H + 2);
+      L->gt_ww = std::min((L->gt_w - 1) * L->sw + 2 * reach + 1, L->W + 2);
       const int px = L->gt_h * L->gt_w;
       for (int ng = std::min(L->G, kTiledGatherThreads / (px * L->gt_lpg)); ng >= 1; --ng) {
         // 16-bit tensors: keep the offset_mask slices dword-aligned when the tap count is odd
         if (s == 2 && ((ng * 3 * L->Kp) & 1) && ng > 1) continue;
+        if (px * ng * L->gt_lpg < min_lanes) break;
         L->gt_ng = ng;
         if (dcnv4_tiled_gather_lds_bytes(*L, s) <= budget) return true;
       }
       if (cap_h >= cap_w) cap_h /= 2; else cap_w /= 2;
     }
-  }
+    return false;
+  };
+  // Two workgroups per CU when the window allows it, so that one stages while the other computes, and workgroups of
+  // 384 lanes or more (a small workgroup stages its window in short pieces and leaves the CU short of waves).  A
+  // shape too wide for that with the full reach stages a window one or two pixels shorter - the sampling points
+  // beyond it are served from memory - before it settles for a small workgroup or a whole CU's LDS.
+  const size_t half = kMaxLdsPerWorkgroup / 2 - 512, whole = kMaxLdsPerWorkgroup - 1024;
+  const int R = L->gt_reach;
+  const int want_lanes = std::min(384, Ho * Wo * L->G * L->gt_lpg);
+  const int shorter = g_opt.reach < 0 ? 2 : 0;        // an explicit reach is kept
+  for (int d = 0; d <= shorter && d <= R - 2; ++d)
+    if (fit(half, R - d, want_lanes)) return true;
+  if (fit(half, R, 1) || fit(whole, R, 1)) return true;
   L->gt_h = L->gt_w = L->gt_ng = L->gt_wh = L->gt_ww = 0;
+  L->gt_reach = R;
   return false;
 }
 
@@ -488,6 +516,7 @@ static int *launch_option_slot(const char *name) {
   if (std::strcmp(name, "scatter") == 0) return &g_opt.scatter;
   if (std::strcmp(name, "reach") == 0) return &g_opt.reach;
   if (std::strcmp(name, "tile") == 0) return &g_opt.tile;
+  if (std::strcmp(name, "gather_tile") == 0) return &g_opt.gather_tile;
   if (std::strcmp(name, "fda_order") == 0) return &g_opt.fda_order;
   return nullptr;
 }
@@ -498,6 +527,7 @@ int dcnv4_gfx950_set_launch_option(const char *name, int value) {
   const bool family = value == kOptAuto || value == kOptTiled || value == kOptPlain;
   const bool ok = slot == &g_opt.reach ? (value >= -1 && value <= 64)
                   : slot == &g_opt.tile ? (value == 0 || value == 8 || value == 16 || value == 32)
+                  : slot == &g_opt.gather_tile ? (value == 0 || value == 4 || value == 8 || value == 16)
                                         : family;
   if (!ok) return fail(DCNV4_ERR_INVALID_ARGUMENT, "launch option %s does not take the value %d", name, value);
   *slot = value;
@@ -1060,6 +1090,19 @@ int dcnv4_gfx950_center_feature_blend_backward(const void *grad_output, const vo
   L.grad_y = grad_sampled; L.grad_x = grad_projected; L.grad_logits = grad_gate_logits;
   if (hipError_t e = launch_center_feature_blend(dtype, L, true, static_cast<hipStream_t>(stream)))
     return hip_fail("centre-feature blend backward launch", e);
+  return DCNV4_OK;
+}
+
+int dcnv4_gfx950_stream_copy(const void *src, void *dst, size_t bytes, void *stream) {
+  if (int rc = check_ptrs({src, dst})) return rc;
+  if (bytes % 16 != 0) return fail(DCNV4_ERR_INVALID_ARGUMENT, "stream copy takes a multiple of 16 bytes, got %zu", bytes);
+  const size_t n16 = bytes / 16;
+  if (n16 == 0) return DCNV4_OK;
+  const size_t blocks = (n16 + 1023) / 1024;
+  if (blocks > 0x7fffffffull) return fail(DCNV4_ERR_RUNTIME, "stream copy of %zu bytes is too large for one launch", bytes);
+  hipLaunchKernelGGL(stream_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const u32x4 *>(src), static_cast<u32x4 *>(dst), n16);
+  if (hipError_t e = hipGetLastError()) return hip_fail("stream copy launch", e);
   return DCNV4_OK;
 }
 

@@ -47,12 +47,12 @@ _ORDER = {"auto": 0, "rows": 1, "heads": 2}
 class launch_options:
     """Context manager over the calling thread's launch options (include/dcnv4_gfx950.h,
     ``dcnv4_gfx950_set_launch_option``): ``gather`` in auto / tiled / direct, ``scatter`` in auto / tiled / atomic,
-    ``reach`` an int or None, ``tile`` 8 / 16 / 32 or None, ``fda_order`` in auto / rows / heads.  Used by the tuner,
+    ``reach`` an int or None, ``tile`` 8 / 16 / 32 or None, ``gather_tile`` 4 / 8 / 16 or None, ``fda_order`` in auto / rows / heads.  Used by the tuner,
     by dispatch-table entries that carry options and by tests that force a kernel family; on exit every option is
     back at the value it had on entry, so contexts nest.  Results do not depend on the options beyond the rounding
     of sums."""
 
-    def __init__(self, gather=None, scatter=None, reach=None, tile=None, fda_order=None):
+    def __init__(self, gather=None, scatter=None, reach=None, tile=None, fda_order=None, gather_tile=None):
         self.values = {}
         if gather is not None:
             self.values["gather"] = _FAMILY[gather]
@@ -62,6 +62,8 @@ class launch_options:
             self.values["reach"] = int(reach)
         if tile is not None:
             self.values["tile"] = int(tile)
+        if gather_tile is not None:
+            self.values["gather_tile"] = int(gather_tile)
         if fda_order is not None:
             self.values["fda_order"] = _ORDER[fda_order]
         self.saved = {}
@@ -414,3 +416,16 @@ def flash_deform_attn_backward_split(value, spatial_shapes, level_start_index, s
             _DTYPES[sampling_locations.dtype], batch, spatial_size, num_heads, channels, num_levels, num_query, int(K),
             int(im2col_step), _hint(d_stride), _hint(block_thread), _stream()))
     return [grad_value, grad_loc, grad_logits]
+
+
+def stream_copy(src, dst):
+    """Copies ``src`` into ``dst`` (same byte size, a multiple of 16) with the library's streaming kernel: the measured
+    memory ceiling of the benchmark and the known-size workload that calibrates byte counters."""
+    _check(src, "src")
+    _check(dst, "dst")
+    nbytes = src.numel() * src.element_size()
+    if nbytes != dst.numel() * dst.element_size():
+        raise RuntimeError("src and dst differ in size")
+    with torch.cuda.device(src.device):
+        _lib.check(_L.dcnv4_gfx950_stream_copy(src.data_ptr(), dst.data_ptr(), nbytes, _stream()))
+    return dst

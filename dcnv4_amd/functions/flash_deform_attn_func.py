@@ -9,7 +9,7 @@ from torch.autograd import Function
 from torch.autograd.function import once_differentiable
 
 from .. import ext
-from .launch_spec import findspec_attn, findspec_attn_bwd
+from .launch_spec import attn_launch_options_for, findspec_attn, findspec_attn_bwd
 
 
 class FlashDeformAttnFunction(Function):
@@ -23,8 +23,11 @@ class FlashDeformAttnFunction(Function):
         es = value.element_size()
         d_stride, block_thread = findspec_attn(B, Q, G, C, es)
         ctx.d_stride_backward, ctx.blockthread_backward = findspec_attn_bwd(B, Q, G, C, es)
-        output = ext.flash_deform_attn_forward(value, value_spatial_shapes, value_level_start_index,
-                                               sampling_loc_attn, im2col_step, K, d_stride, block_thread)
+        L = value_spatial_shapes.shape[0]
+        ctx.backward_options = attn_launch_options_for(B, Q, G, C, L, K, es, "bwd")
+        with ext.launch_options(**attn_launch_options_for(B, Q, G, C, L, K, es, "fwd")):
+            output = ext.flash_deform_attn_forward(value, value_spatial_shapes, value_level_start_index,
+                                                   sampling_loc_attn, im2col_step, K, d_stride, block_thread)
         ctx.save_for_backward(value, value_spatial_shapes, value_level_start_index, sampling_loc_attn)
         return output
 
@@ -32,9 +35,10 @@ class FlashDeformAttnFunction(Function):
     @once_differentiable
     def backward(ctx, grad_output):
         value, value_spatial_shapes, value_level_start_index, sampling_loc_attn = ctx.saved_tensors
-        grad_value, grad_sampling_loc_attn = ext.flash_deform_attn_backward(
-            value, value_spatial_shapes, value_level_start_index, sampling_loc_attn, grad_output.contiguous(),
-            ctx.im2col_step, ctx.K, ctx.d_stride_backward, ctx.blockthread_backward)
+        with ext.launch_options(**ctx.backward_options):
+            grad_value, grad_sampling_loc_attn = ext.flash_deform_attn_backward(
+                value, value_spatial_shapes, value_level_start_index, sampling_loc_attn, grad_output.contiguous(),
+                ctx.im2col_step, ctx.K, ctx.d_stride_backward, ctx.blockthread_backward)
         return grad_value, None, None, grad_sampling_loc_attn, None, None
 
 
@@ -56,9 +60,12 @@ class FlashDeformAttnSplitFunction(Function):
         es = value.element_size()
         d_stride, block_thread = findspec_attn(B, Q, G, C, es)
         ctx.d_stride_backward, ctx.blockthread_backward = findspec_attn_bwd(B, Q, G, C, es)
-        output = ext.flash_deform_attn_forward_split(value, value_spatial_shapes, value_level_start_index,
-                                                     sampling_locations, attention_logits, im2col_step, K, d_stride,
-                                                     block_thread)
+        L = value_spatial_shapes.shape[0]
+        ctx.backward_options = attn_launch_options_for(B, Q, G, C, L, K, es, "bwd")
+        with ext.launch_options(**attn_launch_options_for(B, Q, G, C, L, K, es, "fwd")):
+            output = ext.flash_deform_attn_forward_split(value, value_spatial_shapes, value_level_start_index,
+                                                         sampling_locations, attention_logits, im2col_step, K, d_stride,
+                                                         block_thread)
         ctx.save_for_backward(value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_logits)
         return output
 
@@ -66,7 +73,8 @@ class FlashDeformAttnSplitFunction(Function):
     @once_differentiable
     def backward(ctx, grad_output):
         value, shapes, starts, locations, logits = ctx.saved_tensors
-        grad_value, grad_locations, grad_logits = ext.flash_deform_attn_backward_split(
-            value, shapes, starts, locations, logits, grad_output.contiguous(), ctx.im2col_step, ctx.K,
-            ctx.d_stride_backward, ctx.blockthread_backward)
+        with ext.launch_options(**ctx.backward_options):
+            grad_value, grad_locations, grad_logits = ext.flash_deform_attn_backward_split(
+                value, shapes, starts, locations, logits, grad_output.contiguous(), ctx.im2col_step, ctx.K,
+                ctx.d_stride_backward, ctx.blockthread_backward)
         return grad_value, None, None, grad_locations, grad_logits, None, None

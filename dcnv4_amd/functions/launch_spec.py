@@ -11,8 +11,10 @@ B*H*W on every call).
 Measured overrides live in ``gfx950_table.json`` next to this file, written by ``python -m dcnv4_amd.tune``
 (the counterpart of DCNv4_op/scripts/search_dcnv4.py, search_dcnv4_bwd.py and find_best.py).  Its keys are the
 reference's ``"BxHxWxGxC"`` plus the element size and the direction; an entry holds the two hints and, optionally,
-launch options (``gather`` = tiled / direct, ``tile`` = 8 / 16 / 32, ``reach`` = pixels), which
-:func:`launch_options_for` hands to the library as thread-local launch options around the call.
+launch options (``gather`` = tiled / direct, ``tile`` = 8 / 16 / 32, ``reach`` = pixels, ``gather_tile`` = 4 / 8 / 16;
+for the attention operator ``fda_order`` = rows / heads and ``scatter`` = tiled / atomic), which
+:func:`launch_options_for` hands to the library as thread-local launch options around the call.  Attention keys are
+``"attn:BxQxGxC:LxK"`` plus element size and direction.
 """
 import functools
 import json
@@ -31,7 +33,7 @@ def _load_table(path=TABLE_PATH):
 
 
 # key -> {"d_stride": int, "n_thread": int, and optionally "gather": str, "tile": int, "reach": int}
-OPTION_KEYS = ("gather", "tile", "reach")
+OPTION_KEYS = ("gather", "scatter", "tile", "reach", "gather_tile", "fda_order")
 GFX950_TABLE = _load_table()
 
 
@@ -86,3 +88,16 @@ def findspec_attn(B, Q, G, C, elem_bytes=2):
 
 def findspec_attn_bwd(B, Q, G, C, elem_bytes=2):
     return _spec(G, C, elem_bytes, scatter=True)
+
+
+def attn_table_key(B, Q, G, C, L, K, elem_bytes, direction):
+    return f"attn:{B}x{Q}x{G}x{C}:{L}x{K}:{elem_bytes}:{direction}"
+
+
+@functools.lru_cache(maxsize=None)
+def attn_launch_options_for(B, Q, G, C, L, K, elem_bytes, direction):
+    """Options a table entry asks for around a flash-deformable-attention call ({}: the library chooses)."""
+    entry = GFX950_TABLE.get(attn_table_key(B, Q, G, C, L, K, elem_bytes, direction))
+    if entry is None:
+        return {}
+    return {k: entry[k] for k in OPTION_KEYS if entry.get(k, "auto") not in ("auto", None)}

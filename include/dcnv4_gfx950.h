@@ -61,6 +61,8 @@ const char *dcnv4_gfx950_last_error(void);
  *                the LDS-tiled DCNv4 gathers stage; sampling points beyond it are fetched from memory
  *   "tile"       0 library's choice (32), else 8, 16 or 32: largest side of the input tile a workgroup of the
  *                DCNv4 grad_value kernel owns
+ *   "gather_tile" 0 library's choice (16), else 4, 8 or 16: largest side of the output tile a workgroup of the
+ *                LDS-tiled DCNv4 gathers owns
  *   "fda_order"  0 library's choice, 1 whole query rows per workgroup, 2 one head per workgroup
  *                (flash deformable attention forward and grad_sampling_loc_attn kernels)
  * dcnv4_gfx950_get_launch_option reads a value back, so that a caller can restore what it found.
@@ -309,6 +311,13 @@ int dcnv4_gfx950_center_feature_blend_backward(const void *grad_output, const vo
                                                void *grad_sampled, void *grad_projected,
                                                float *grad_gate_logits, int dtype, long long rows,
                                                int channels, int groups, void *stream);
+
+/*
+ * Measurement aid without a counterpart in the reference: copies `bytes` (a multiple of 16) from src to dst with
+ * the library's own streaming kernel (16-byte non-temporal loads and stores).  Its rate is the ceiling the
+ * benchmark quotes beside the nominal HBM peak, and its known traffic calibrates hardware byte counters.
+ */
+int dcnv4_gfx950_stream_copy(const void *src, void *dst, size_t bytes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -659,3 +659,28 @@ def test_flash_intern_image_b_in_fp16_matches_the_same_weights_on_the_torch_core
         want = ref(x.half().float())
     assert got.shape == (8, 1000) and torch.isfinite(got).all()
     assert _rel_err(got, want) < 3e-2
+
+
+def test_every_committed_table_entry_still_beats_the_library_choice():
+    """The dispatch table is measured data: an entry that no longer wins against the library's own planner (the kernels
+    have changed since it was measured) must be deleted or re-measured with `python -m dcnv4_amd.tune`."""
+    import re
+    from dcnv4_amd import ext, tune
+    from dcnv4_amd.functions import launch_spec as ls
+    for key, entry in ls.GFX950_TABLE.items():
+        options = {k: entry[k] for k in ls.OPTION_KEYS if k in entry}
+        m = re.fullmatch(r"(\d+)x(\d+)x(\d+)x(\d+)x(\d+):(\d):(fwd|bwd)", key)
+        if m is None:
+            continue                  # attention entries are timed by the tuner only
+        B, H, W, G, D, es, direction = (int(x) if x.isdigit() else x for x in m.groups())
+        dtype = torch.float16 if es == 2 else torch.float32
+        v, om, go = (t.cuda() for t in make_dcnv4_inputs(B, H, W, G, D, offset_range=3.0, seed=1, dtype=dtype))
+        def call(d, n):
+            if direction == "fwd":
+                return ext.dcnv4_forward(v, om, *GEOM, G, D, 1.0, 64, 0, d, n, False)
+            return ext.dcnv4_backward(v, om, *GEOM, G, D, 1.0, 64, go, 0, d, n, False)
+        base = min(tune._time(lambda: call(0, 0), 30, 10) for _ in range(3))
+        with ext.launch_options(**options):
+            tuned = min(tune._time(lambda: call(entry["d_stride"], entry["n_thread"]), 30, 10) for _ in range(3))
+        print(f"table entry {key}: library {base * 1e3:.1f} us, entry {tuned * 1e3:.1f} us", flush=True)
+        assert tuned <= base, f"{key}: the entry ({tuned * 1e3:.1f} us) lost to the library's choice ({base * 1e3:.1f} us); re-run the tuner"

@@ -24,7 +24,7 @@ def test_library_exports_every_symbol_the_header_declares():
     from dcnv4_amd import _lib
     lib = ctypes.CDLL(_lib.LIB_PATH)
     declared = _declared_functions()
-    assert len(declared) == 21, sorted(declared)
+    assert len(declared) == 22, sorted(declared)
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in include/dcnv4_gfx950.h but not exported"
     assert set(declared) == set(_lib.SIGNATURES), "ctypes table and header list different functions"
@@ -261,10 +261,29 @@ def test_tuner_candidates_are_valid_hints_and_start_with_the_library_choice():
         fwd = tune.candidates(G, D, es, "fwd")
         assert fwd[0] == ("library", {}, 0, 0)
         for _, options, d_stride, n_thread in fwd[1:]:
-            assert options == {"gather": "direct"} and D % d_stride == 0 and d_stride * es <= 16 and n_thread in (128, 256, 512)
+            if options == {"gather": "direct"}:
+                assert D % d_stride == 0 and d_stride * es <= 16 and n_thread in (128, 256, 512)
+            else:       # parameters of the tiled family: hints stay with the library
+                assert set(options) <= {"reach", "gather_tile"} and (d_stride, n_thread) == (0, 0)
+        assert {"reach": 3} in [c[1] for c in fwd] and {"gather_tile": 8} in [c[1] for c in fwd]
         bwd = tune.candidates(G, D, es, "bwd")
-        assert bwd[0] == ("library", {}, 0, 0) and {"tile": 16} in [c[1] for c in bwd]
+        assert bwd[0] == ("library", {}, 0, 0) and {"tile": 16} in [c[1] for c in bwd] and {"reach": 2} in [c[1] for c in bwd]
     assert set(tune.SHAPES) == {"t", "b", "dense"} and all(len(v) == 4 for v in tune.SHAPES.values())
+    att = tune.attention_candidates("bwd")
+    assert att[0] == ("library", {}) and {"scatter": "atomic"} in [c[1] for c in att] and {"fda_order": "heads"} in [c[1] for c in att]
+    # every option the tuner may write is one the table loader passes on
+    from dcnv4_amd.functions import launch_spec
+    used = {k for c in tune.candidates(4, 16, 2, "fwd") + tune.candidates(4, 16, 2, "bwd") for k in c[1]} | {k for c in att for k in c[1]}
+    assert used <= set(launch_spec.OPTION_KEYS)
+
+
+def test_committed_table_entries_are_well_formed():
+    from dcnv4_amd.functions import launch_spec
+    for key, entry in launch_spec.GFX950_TABLE.items():
+        assert key.split(":")[-1] in ("fwd", "bwd")
+        assert set(entry) <= set(launch_spec.OPTION_KEYS) | {"d_stride", "n_thread"}, key
+        if not key.startswith("attn:"):
+            assert entry["d_stride"] in (1, 2, 4, 8, 16) and entry["n_thread"] > 0
 
 
 def test_module_initial_values_follow_the_reference_recipe():
