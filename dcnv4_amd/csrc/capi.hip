@@ -165,23 +165,28 @@ bool fda_tiled_enabled() { return g_opt.scatter != kOptPlain; }
 // at most one (cell, group, channel part) per lane and its LDS footprint fits.
 int plan_grad_value_tiles(DcnLaunch *L, int dtype) {
   const int D = L->D;
-  L->gv_cw = D <= 8 ? 8 : (D <= 16 ? 16 : 32);
+  L->gv_cw = D <= 8 ? 8 : 16;
   L->gv_lps_log2 = 0;
   while ((L->gv_cw << L->gv_lps_log2) < D) ++L->gv_lps_log2;
-  const int max_slots = 1024 >> L->gv_lps_log2;
-  const int cap_log2 = g_opt.tile == 8 ? 3 : (g_opt.tile == 16 ? 4 : 5);
-  L->tile_h_log2 = L->tile_w_log2 = cap_log2;
-  while (L->tile_h_log2 > 0 && (1 << (L->tile_h_log2 - 1)) >= L->H) --L->tile_h_log2;
-  while (L->tile_w_log2 > 0 && (1 << (L->tile_w_log2 - 1)) >= L->W) --L->tile_w_log2;
-  while ((1 << (L->tile_h_log2 + L->tile_w_log2)) > max_slots) {
-    if (L->tile_h_log2 >= L->tile_w_log2) --L->tile_h_log2; else --L->tile_w_log2;
+  const int max_lists = dcnv4_grad_value_max_lists() >> L->gv_lps_log2;      // a lane per (anchor, group, channel part)
+  const int cap = g_opt.tile == 8 ? 8 : (g_opt.tile == 16 ? 16 : 31);
+  // the image is split evenly into tiles of at most cap x cap cells (all workgroups then carry the same load); the
+  // anchors of a tile, one row and one column more than its cells, must fit the workgroup
+  auto even_split = [](int extent, int c) { const int n = (extent + c - 1) / c; return (extent + n - 1) / n; };
+  int cap_h = cap, cap_w = cap;
+  for (;;) {
+    L->tile_h = even_split(L->H, cap_h);
+    L->tile_w = even_split(L->W, cap_w);
+    if ((L->tile_h + 1) * (L->tile_w + 1) <= max_lists) break;
+    if (cap_h == 1 && cap_w == 1) return fail(DCNV4_ERR_RUNTIME, "groups of %d channels are too wide for the tiled backward", D);
+    if (cap_h >= cap_w) cap_h = std::max(1, cap_h * 3 / 4); else cap_w = std::max(1, cap_w * 3 / 4);
   }
-  L->tile_h = 1 << L->tile_h_log2;
-  L->tile_w = 1 << L->tile_w_log2;
-  const int cells = L->tile_h * L->tile_w;
+  L->tile_h_log2 = ceil_log2(L->tile_h);
+  L->tile_w_log2 = ceil_log2(L->tile_w);
+  const int anchors = (L->tile_h + 1) * (L->tile_w + 1);
   const int max_items = dcnv4_grad_value_rounds(L->gv_cw) * 1024;
   const int park_bytes = dtype == DCNV4_DTYPE_F16 ? 2 : 4;
-  for (int ng = std::min({L->G, max_slots / cells, 63, max_items / L->Kp}); ng >= 1; --ng) {
+  for (int ng = std::min({L->G, max_lists / anchors, 63, max_items / L->Kp}); ng >= 1; --ng) {
     L->ng_chunk = ng;
     int units = (ng * (L->gv_cw << L->gv_lps_log2) * park_bytes + 15) / 16;
     units |= 1;                                     // an odd number of 16-byte units spreads the rows over the LDS banks

@@ -70,8 +70,8 @@ struct DcnLaunch {
   void *grad_value;         // [n_img, H, W, G*D] in the tensor dtype
   GradState *state;
   int n_img;
-  int tile_h, tile_w;       // input-space tile one workgroup owns (powers of two)
-  int tile_h_log2, tile_w_log2;
+  int tile_h, tile_w;       // input-space tile one workgroup owns (an even split of the image, at most 32 x 32)
+  int tile_h_log2, tile_w_log2;   // log2 of the tile extents rounded up to powers of two: the stride of the cell index
   int ng_chunk;             // groups per workgroup (channel chunk = ng_chunk * D)
   int strip_pix;            // output pixels staged per strip
   int gv_cw;                // channels a lane accumulates: 8, 16 or 32
@@ -87,7 +87,8 @@ struct DcnLaunch {
 
 // Sampling points a lane of the tiled grad_value kernel handles per strip, at most (it keeps them in registers next to
 // cw running sums): a strip holds at most 1024 * rounds of them.
-constexpr int dcnv4_grad_value_rounds(int cw) { return cw <= 16 ? 4 : 2; }
+constexpr int dcnv4_grad_value_rounds(int) { return 6; }
+int dcnv4_grad_value_max_lists();      // (anchor, group) lists a workgroup of the grad_value kernel can hold
 
 // Flash deformable attention (reference: DCNv4_op/src/cuda/flash_deform_im2col_cuda.cuh:211-272)
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
