@@ -143,6 +143,7 @@ struct LaunchOptions {
   int reach = -1;              // input pixels around a reference point that the tiled gathers stage; -1: default
   int tile = 0;                // largest side of a grad_value tile (8, 16, 32); 0: default
   int gather_tile = 0;         // largest side of an output tile of the tiled gathers (4, 8, 16); 0: default (16)
+  int gv_threads = 0;          // lanes per workgroup of the grad_value kernel (512, 1024); 0: default
   int fda_order = kOptAuto;    // attention forward: 1 whole query rows per workgroup, 2 one head per workgroup
 };
 thread_local LaunchOptions g_opt;
@@ -163,37 +164,54 @@ bool fda_tiled_enabled() { return g_opt.scatter != kOptPlain; }
 
 // Tile, group chunk, lanes per slot and strip of the tiled grad_value kernel such that a workgroup of 1024 lanes has
 // at most one (cell, group, channel part) per lane and its LDS footprint fits.
-int plan_grad_value_tiles(DcnLaunch *L, int dtype) {
+int plan_grad_value_tiles(DcnLaunch *L, int dtype, int batch) {
   const int D = L->D;
   L->gv_cw = D <= 8 ? 8 : 16;
   L->gv_lps_log2 = 0;
   while ((L->gv_cw << L->gv_lps_log2) < D) ++L->gv_lps_log2;
-  const int max_lists = dcnv4_grad_value_max_lists() >> L->gv_lps_log2;      // a lane per (anchor, group, channel part)
-  const int cap = g_opt.tile == 8 ? 8 : (g_opt.tile == 16 ? 16 : 31);
-  // the image is split evenly into tiles of at most cap x cap cells (all workgroups then carry the same load); the
-  // anchors of a tile, one row and one column more than its cells, must fit the workgroup
+  // Workgroups of 1024 lanes with a CU's whole LDS (measured faster than two of 512 sharing a CU on every shape with
+  // enough tiles), unless that leaves CUs without a workgroup: then 512 lanes and half the groups each.  The launch
+  // option "gv_threads" overrides.
   auto even_split = [](int extent, int c) { const int n = (extent + c - 1) / c; return (extent + n - 1) / n; };
-  int cap_h = cap, cap_w = cap;
-  for (;;) {
-    L->tile_h = even_split(L->H, cap_h);
-    L->tile_w = even_split(L->W, cap_w);
-    if ((L->tile_h + 1) * (L->tile_w + 1) <= max_lists) break;
-    if (cap_h == 1 && cap_w == 1) return fail(DCNV4_ERR_RUNTIME, "groups of %d channels are too wide for the tiled backward", D);
-    if (cap_h >= cap_w) cap_h = std::max(1, cap_h * 3 / 4); else cap_w = std::max(1, cap_w * 3 / 4);
-  }
-  L->tile_h_log2 = ceil_log2(L->tile_h);
-  L->tile_w_log2 = ceil_log2(L->tile_w);
-  const int anchors = (L->tile_h + 1) * (L->tile_w + 1);
-  const int max_items = dcnv4_grad_value_rounds(L->gv_cw) * 1024;
   const int park_bytes = dtype == DCNV4_DTYPE_F16 ? 2 : 4;
-  for (int ng = std::min({L->G, max_lists / anchors, 63, max_items / L->Kp}); ng >= 1; --ng) {
-    L->ng_chunk = ng;
-    int units = (ng * (L->gv_cw << L->gv_lps_log2) * park_bytes + 15) / 16;
-    units |= 1;                                     // an odd number of 16-byte units spreads the rows over the LDS banks
-    L->gv_go_stride = units * 16;
-    for (int s = std::min(1023, max_items / (L->Kp * ng)); s >= 1; s = s > 64 ? s - 16 : s - 1) {
-      L->strip_pix = s;
-      if (dcnv4_grad_value_lds_bytes(*L) <= kMaxLdsPerWorkgroup - 512) return DCNV4_OK;
+  int threads_first = g_opt.gv_threads == 512 ? 512 : 1024;
+  if (g_opt.gv_threads == 0) {
+    const int lists_1024 = 1024 >> L->gv_lps_log2;
+    const int th = even_split(L->H, 31), tw = even_split(L->W, 31);
+    if ((th + 1) * (tw + 1) <= lists_1024) {
+      const int ng = std::max(1, std::min(L->G, lists_1024 / ((th + 1) * (tw + 1))));
+      const long long wgs = (long long)batch * ((L->H + th - 1) / th) * ((L->W + tw - 1) / tw) * ((L->G + ng - 1) / ng);
+      if (wgs < 256) threads_first = 512;
+    }
+  }
+  for (int threads = threads_first; threads <= 1024; threads *= 2) {
+    L->gv_threads = threads;
+    const size_t budget = threads == 512 ? kMaxLdsPerWorkgroup / 2 - 512 : kMaxLdsPerWorkgroup - 512;
+    const int max_lists = threads >> L->gv_lps_log2;      // a lane per (anchor, group, channel part)
+    if (max_lists < 4) continue;
+    const int cap = g_opt.tile == 8 ? 8 : (g_opt.tile == 16 ? 16 : 31);
+    // the image is split evenly into tiles of at most cap x cap cells (all workgroups then carry the same load); the
+    // anchors of a tile, one row and one column more than its cells, must fit the workgroup
+    int cap_h = cap, cap_w = cap;
+    for (;;) {
+      L->tile_h = even_split(L->H, cap_h);
+      L->tile_w = even_split(L->W, cap_w);
+      if ((L->tile_h + 1) * (L->tile_w + 1) <= max_lists) break;
+      if (cap_h >= cap_w) cap_h = std::max(1, cap_h - 1); else cap_w = std::max(1, cap_w - 1);
+    }
+    L->tile_h_log2 = ceil_log2(L->tile_h);
+    L->tile_w_log2 = ceil_log2(L->tile_w);
+    const int anchors = (L->tile_h + 1) * (L->tile_w + 1);
+    const int max_items = kGradValueRounds * threads;
+    for (int ng = std::min({L->G, max_lists / anchors, 63, max_items / L->Kp}); ng >= 1; --ng) {
+      L->ng_chunk = ng;
+      int units = (ng * (L->gv_cw << L->gv_lps_log2) * park_bytes + 15) / 16;
+      units |= 1;                                     // an odd number of 16-byte units spreads the rows over the LDS banks
+      L->gv_go_stride = units * 16;
+      for (int s = std::min(1023, max_items / (L->Kp * ng)); s >= 1; s = s > 64 ? s - 16 : s - 1) {
+        L->strip_pix = s;
+        if (dcnv4_grad_value_lds_bytes(*L) <= budget) return DCNV4_OK;
+      }
     }
   }
   return fail(DCNV4_ERR_RUNTIME, "kernel with %d taps and %d group channels does not fit the tiled backward", L->Kp, D);
@@ -522,6 +540,7 @@ static int *launch_option_slot(const char *name) {
   if (std::strcmp(name, "reach") == 0) return &g_opt.reach;
   if (std::strcmp(name, "tile") == 0) return &g_opt.tile;
   if (std::strcmp(name, "gather_tile") == 0) return &g_opt.gather_tile;
+  if (std::strcmp(name, "gv_threads") == 0) return &g_opt.gv_threads;
   if (std::strcmp(name, "fda_order") == 0) return &g_opt.fda_order;
   return nullptr;
 }
@@ -533,6 +552,7 @@ int dcnv4_gfx950_set_launch_option(const char *name, int value) {
   const bool ok = slot == &g_opt.reach ? (value >= -1 && value <= 64)
                   : slot == &g_opt.tile ? (value == 0 || value == 8 || value == 16 || value == 32)
                   : slot == &g_opt.gather_tile ? (value == 0 || value == 4 || value == 8 || value == 16)
+                  : slot == &g_opt.gv_threads ? (value == 0 || value == 512 || value == 1024)
                                         : family;
   if (!ok) return fail(DCNV4_ERR_INVALID_ARGUMENT, "launch option %s does not take the value %d", name, value);
   *slot = value;
@@ -602,7 +622,7 @@ static int dcn_backward_impl(const void *value, const void *offset_mask, const v
 
   // state reset, then 1. grad_offset_mask + the reach the sampling points need  2. tiled grad_value (plain stores)
   DcnLaunch base = pr.launch;
-  if (int rc = plan_grad_value_tiles(&base, dtype)) return rc;
+  if (int rc = plan_grad_value_tiles(&base, dtype, batch)) return rc;
   // the grad_value kernel addresses one image's offset_mask and grad_out with 32-bit element offsets
   if (base.Q >= (1 << 24) || (uint64_t)base.Q * (uint64_t)base.P_pad >= (1ull << 31) ||
       (uint64_t)base.Q * (uint64_t)(base.G * base.D) >= (1ull << 31))

@@ -39,7 +39,6 @@
 namespace dcn {
 namespace {
 
-constexpr int kValThreads = 1024;
 
 // grad_out is parked in LDS as it is for fp32 and fp16 tensors (fp16 feeds mixed-precision FMAs directly)
 // and widened to fp32 for bf16.
@@ -48,13 +47,14 @@ template <> struct ParkType<F16> { typedef _Float16 type; };
 
 __device__ __forceinline__ int fdiv_small(int n, float inv) { return (int)(((float)n + 0.5f) * inv); }   // exact for n < 2^20
 
-// One (anchor, group) list per lane at most.
-constexpr int kMaxAnchorSlots = kValThreads;
 
 // CW: channels a lane accumulates for each of the four corners (8 or 16): the group width rounded up, or 16 with
 // several lanes per (anchor, group).
-template <typename Tag, int KP, int CW, int ROUNDS>
-__global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const DcnLaunch p) {
+// NT: lanes per workgroup (512: two workgroups share a CU and overlap each other's phases; 1024: one workgroup with
+// the whole LDS); one (anchor, group) list per lane at most.
+template <typename Tag, int KP, int CW, int ROUNDS, int NT>
+__global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p) {
+  constexpr int kValThreads = NT, kMaxAnchorSlots = NT;
   extern __shared__ __align__(16) uint32_t lds32[];
   typedef typename ParkType<Tag>::type park_t;
   typedef typename RawWord<Tag::kBytes>::type elem_t;
@@ -292,7 +292,7 @@ __global__ void __launch_bounds__(kValThreads) dcnv4_grad_value_kernel(const Dcn
   // same cell, so plain LDS stores and read-modify-writes suffice.  Corner 0 reaches every cell of the tile and so
   // initialises the image.
   float *s_sum = reinterpret_cast<float *>(lds32);
-  const int row_floats = p.ng_chunk * Dp;                        // floats per cell
+  const int row_floats = dcnv4_grad_value_image_stride(p.ng_chunk * Dp);      // floats between cells (an odd number of 16-byte units)
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     const int cy = my_ay - 1 + (k >> 1), cx = my_ax - 1 + (k & 1);
@@ -344,7 +344,7 @@ template <typename Tag>
 hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
   const int n_chunks = (p.G + p.ng_chunk - 1) / p.ng_chunk;
   const int nty = (p.H + p.tile_h - 1) / p.tile_h, ntx = (p.W + p.tile_w - 1) / p.tile_w;
-  const dim3 grid((unsigned)(p.n_img * nty * ntx * n_chunks)), block(kValThreads);
+  const dim3 grid((unsigned)(p.n_img * nty * ntx * n_chunks)), block((unsigned)p.gv_threads);
   const size_t lds = dcnv4_grad_value_lds_bytes(p);
   const bool k3 = p.kh == 3 && p.kw == 3;
   auto go = [&](auto kernel) -> hipError_t {
@@ -354,8 +354,12 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
   };
 #define GV_CASE(KPV)                                                                \
   do {                                                                              \
-    if (p.gv_cw == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, dcnv4_grad_value_rounds(8)>);      \
-    return go(dcnv4_grad_value_kernel<Tag, KPV, 16, dcnv4_grad_value_rounds(16)>);  \
+    if (p.gv_threads == 512) {                                                      \
+      if (p.gv_cw == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, kGradValueRounds, 512>);      \
+      return go(dcnv4_grad_value_kernel<Tag, KPV, 16, kGradValueRounds, 512>);      \
+    }                                                                               \
+    if (p.gv_cw == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, kGradValueRounds, 1024>);       \
+    return go(dcnv4_grad_value_kernel<Tag, KPV, 16, kGradValueRounds, 1024>);       \
   } while (0)
   if (k3 && !p.remove_center) GV_CASE(9);
   if (k3 && p.remove_center) GV_CASE(8);
@@ -369,12 +373,10 @@ size_t dcnv4_grad_value_lds_bytes(const DcnLaunch &p) {
   const size_t items = (size_t)p.strip_pix * p.Kp * p.ng_chunk;
   // list heads (two sets), parked grad_out, entries + the dummy entry that ends every list; at the end the fp32 image
   // of the tile takes the place of all of it
-  const size_t strip = 2 * kMaxAnchorSlots * sizeof(uint32_t) + (size_t)p.strip_pix * p.gv_go_stride + (items + 1) * sizeof(u32x4);
-  const size_t image = (size_t)p.tile_h * p.tile_w * p.ng_chunk * (p.gv_cw << p.gv_lps_log2) * sizeof(float);
+  const size_t strip = 2 * (size_t)p.gv_threads * sizeof(uint32_t) + (size_t)p.strip_pix * p.gv_go_stride + (items + 1) * sizeof(u32x4);
+  const size_t image = (size_t)p.tile_h * p.tile_w * dcnv4_grad_value_image_stride(p.ng_chunk * (p.gv_cw << p.gv_lps_log2)) * sizeof(float);
   return std::max(strip, image);
 }
-
-int dcnv4_grad_value_max_lists() { return kMaxAnchorSlots; }
 
 hipError_t launch_dcnv4_grad_value(int dtype, const DcnLaunch &p, hipStream_t stream) {
   switch (dtype) {

@@ -74,7 +74,8 @@ struct DcnLaunch {
   int tile_h_log2, tile_w_log2;   // log2 of the tile extents rounded up to powers of two: the stride of the cell index
   int ng_chunk;             // groups per workgroup (channel chunk = ng_chunk * D)
   int strip_pix;            // output pixels staged per strip
-  int gv_cw;                // channels a lane accumulates: 8, 16 or 32
+  int gv_threads;           // lanes per workgroup of the grad_value kernel: 512 or 1024
+  int gv_cw;                // channels a lane accumulates per corner: 8 or 16
   int gv_lps_log2;          // log2 of the lanes that share one (cell, group): group width / gv_cw, rounded up to a power of two
   int gv_go_stride;         // bytes between the parked grad_out rows of consecutive pixels (an odd number of 16-byte units)
   // LDS-tiled gather path (forward and grad_offset_mask); gt_h == 0: not planned
@@ -85,10 +86,12 @@ struct DcnLaunch {
   int gt_reach;             // input pixels around an output pixel's reference point that the window covers
 };
 
-// Sampling points a lane of the tiled grad_value kernel handles per strip, at most (it keeps them in registers next to
-// cw running sums): a strip holds at most 1024 * rounds of them.
-constexpr int dcnv4_grad_value_rounds(int) { return 6; }
-int dcnv4_grad_value_max_lists();      // (anchor, group) lists a workgroup of the grad_value kernel can hold
+// Sampling points a lane of the tiled grad_value kernel handles per strip, at most: a strip holds at most
+// gv_threads * kGradValueRounds of them.
+constexpr int kGradValueRounds = 6;
+// floats between the cells of the fp32 tile image in which the corner sums meet: the cell's channels rounded up to an odd
+// number of 16-byte units, so that the lanes of one LDS instruction (consecutive cells) fall into different banks
+__host__ __device__ inline int dcnv4_grad_value_image_stride(int channels) { return ((((channels + 3) / 4) | 1) * 4); }
 
 // Flash deformable attention (reference: DCNv4_op/src/cuda/flash_deform_im2col_cuda.cuh:211-272)
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
