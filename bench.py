@@ -120,6 +120,18 @@ def main():
         t = B * H * W * C * s
         return 2 * t, 3 * t
 
+    def tail_inputs(B, H, W, C, dtype):
+        # the tail of a FlashInternImage block: x + gamma * LayerNorm(y) over rows of C channels
+        rows = B * H * W
+        return (torch.randn(rows, C, device=dev).to(dtype), torch.randn(rows, C, device=dev).to(dtype),
+                (1 + 0.1 * torch.randn(C, device=dev)).to(dtype), (0.1 * torch.randn(C, device=dev)).to(dtype),
+                torch.randn(C, device=dev).to(dtype), torch.randn(rows, C, device=dev).to(dtype))
+
+    def tail_bytes(s, B, H, W, C):
+        # forward: y and the residual read, the result written; backward: y and grad_out read, grad_y written
+        t = B * H * W * C * s
+        return 3 * t, 3 * t
+
     def time_op(fn, iters, warm=20):
         for _ in range(warm):
             fn()
@@ -184,6 +196,19 @@ def main():
             print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "algorithmic_MB": round(nbytes / 1e6, 2),
                               "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)}))
             return
+        if op.startswith("block_tail"):      # residual + gamma * LayerNorm(y), forward / backward
+            for name, B, H, W, C, G in CFG2 + CFG5:
+                if name != shape_name:
+                    continue
+                y, x, w, b, gamma, go = tail_inputs(B, H, W, C, dtype)
+                fn = (lambda: ext.layer_norm_residual_forward(y, x, w, b, gamma, 1e-6)) if op == "block_tail_fwd" else \
+                     (lambda: ext.layer_norm_residual_backward(go, y, w, b, gamma, 1e-6))
+                ms = time_op(fn, args.steps, warm=args.warmup)
+                nbytes = tail_bytes(y.element_size(), B, H, W, C)[0 if op == "block_tail_fwd" else 1]
+                print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "algorithmic_MB": round(nbytes / 1e6, 2),
+                                  "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)}))
+                return
+            sys.exit(f"--only-op {args.only_op}: no such shape")
         if op.startswith("depthwise"):       # the offset_mask_dw layer of a DCNv4 block, 3x3, NHWC
             for name, B, H, W, C, G in CFG2 + CFG5:
                 if name != shape_name:
@@ -270,6 +295,13 @@ def main():
             add("depthwise_bwd", name, torch.float16, time_op(lambda: ext.depthwise_conv_backward(x, w, go, 1), args.op_iters),
                 dw_bytes(2, B, H, W, C)[1])
             del x, w, b, go
+            if name == "B-stage1":
+                y, x, w, b, gamma, go = tail_inputs(B, H, W, C, torch.float16)
+                add("block_tail_fwd", name, torch.float16, time_op(lambda: ext.layer_norm_residual_forward(y, x, w, b, gamma, 1e-6), args.op_iters),
+                    tail_bytes(2, B, H, W, C)[0])
+                add("block_tail_bwd", name, torch.float16, time_op(lambda: ext.layer_norm_residual_backward(go, y, w, b, gamma, 1e-6), args.op_iters),
+                    tail_bytes(2, B, H, W, C)[1])
+                del y, x, w, b, gamma, go
         for dtype, s in ((torch.float16, 2), (torch.float32, 4)):
             (B, N, G, D, L, K), shapes, starts, v, sla, go = fda_inputs(dtype)
             fb, bb = fda_bytes(s, B, N, N, G, D, L, K)

@@ -441,14 +441,16 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
   __syncthreads();
 
   uint32_t reach_needed = 0;
+  float reach_f = 0.f;
   if (active) {
     float go[NV][EPV];
 #pragma unroll
     for (int v = 0; v < NV; ++v) pack::decode(go_raw[v], go[v]);
     const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
     const int p0y = half_h - p.ph + ho * p.sh, p0x = half_w - p.pw + wo * p.sw;      // reference point
-    const float x_base = sub_rn((float)p0x, mul_rn((float)half_w, p.offset_scale));
-    const float y_base = sub_rn((float)p0y, mul_rn((float)half_h, p.offset_scale));
+    const float p0xf = (float)p0x, p0yf = (float)p0y;
+    const float x_base = sub_rn(p0xf, mul_rn((float)half_w, p.offset_scale));
+    const float y_base = sub_rn(p0yf, mul_rn((float)half_h, p.offset_scale));
     elem_t *om = s_om + unit * 3 * Kp;
     const int zero_base = t.wh * t.ww * cell_stride, row_bytes = t.ww * cell_stride;
     const int lane_bytes = gl * p.D * Tag::kBytes + part * NV * 16;
@@ -475,12 +477,9 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
       const float m = lds_elem<Tag>(om, 2 * Kp + k);
       const WinTap wt = window_tap(y, x, p.H, p.W, t, cell_stride, lane_bytes, zero_base);
       far_mask |= (mask_t)(wt.inside && !wt.ok) << k;
-      if (wt.inside) {      // distance of the weighted, in-image part of the 2x2 corner block from the reference point
-        const int y0 = wt.ry + t.wy0, x0 = wt.rx + t.wx0;
-        const int y1 = y0 + (wt.ly > 0.f ? 1 : 0), x1 = x0 + (wt.lx > 0.f ? 1 : 0);
-        const int d = max(max(p0y - max(y0, 0), min(y1, p.H - 1) - p0y), max(p0x - max(x0, 0), min(x1, p.W - 1) - p0x));
-        reach_needed = max(reach_needed, (uint32_t)max(d, 0));
-      }
+      // Chebyshev distance of the point from the reference point; its ceiling is how far the weighted corners of
+      // the 2x2 block lie from it at most (a point at an integer distance k has its far corners at weight 0)
+      if (wt.inside) reach_f = fmaxf(reach_f, fmaxf(fabsf(x - p0xf), fabsf(y - p0yf)));
       u32x4 raw[4][NV];
 #pragma unroll
       for (int cn = 0; cn < 4; ++cn) {
@@ -579,7 +578,7 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
 
   // the reach the grad_value kernel has to cover: fold in LDS, then touch the global word only when it would grow
   // (same-address global atomics retire slowly)
-  reach_needed = wave_max_u32(reach_needed);
+  reach_needed = wave_max_u32((uint32_t)min(ceilf(reach_f), 1048576.f));
   if ((threadIdx.x & (kWave - 1)) == 0 && reach_needed != 0) atomicMax(&s_reach, reach_needed);
   __syncthreads();
   if (threadIdx.x == 0) {
