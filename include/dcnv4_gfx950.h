@@ -149,8 +149,9 @@ int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_s
 
 /*
  * Bytes of device scratch flash_deform_attn_gfx950_backward needs for this problem (16-byte aligned;
- * contents need no initialisation).  Head widths that are multiples of 8 up to 32 take about 22 bytes
- * per sampling point (key, probability, and list space for binning the points by tile) plus a tile table; other widths take an fp32 image of value for 16-bit
+ * contents need no initialisation).  Head widths that are multiples of 8 up to 32 take about 34 bytes
+ * per sampling point (a key, a position-and-probability record, and list space for binning the points by
+ * tile) plus grad_output once more and a tile table; other widths take an fp32 image of value for 16-bit
  * tensors.  The reference allocates its fp32 gradient buffers itself
  * (DCNv4_op/src/cuda/flash_deform_attn_cuda.cu:127-133).
  */
