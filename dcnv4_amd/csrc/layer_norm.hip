@@ -140,26 +140,36 @@ __global__ void __launch_bounds__(kLnThreads) layer_norm_residual_backward_kerne
 
   const long long row_begin = (long long)blockIdx.x * p.slab;
   const long long row_end = row_begin + p.slab < p.rows ? row_begin + p.slab : p.rows;
+  // the rows of the next pass are requested before the current pass is worked on
+  raw_t next_y[VPL], next_g[VPL];
+  auto request = [&](long long row0) {
+    const long long row = row0 + team_id;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      const int i = lane_in_team + u * team;
+      if (row < row_end && col_live[u]) {
+        next_y[u] = reinterpret_cast<const raw_t *>(p.y)[row * nvec + i];
+        next_g[u] = reinterpret_cast<const raw_t *>(p.grad_out)[row * nvec + i];
+      } else {
+        next_y[u] = raw_t{};
+        next_g[u] = raw_t{};
+      }
+    }
+  };
+  request(row_begin);
   for (long long row0 = row_begin; row0 < row_end; row0 += teams_per_block) {
     const long long row = row0 + team_id;
     const bool row_live = row < row_end;
-    const raw_t *y = reinterpret_cast<const raw_t *>(p.y) + row * nvec;
-    const raw_t *go = reinterpret_cast<const raw_t *>(p.grad_out) + row * nvec;
     float v[VPL][V], g[VPL][V];
     float sum = 0.f;
 #pragma unroll
     for (int u = 0; u < VPL; ++u) {
-      const int i = lane_in_team + u * team;
-      if (row_live && col_live[u]) {
-        pack::decode(y[i], v[u]);
-        pack::decode(go[i], g[u]);
-      } else {
-#pragma unroll
-        for (int c = 0; c < V; ++c) v[u][c] = g[u][c] = 0.f;
-      }
+      pack::decode(next_y[u], v[u]);
+      pack::decode(next_g[u], g[u]);
 #pragma unroll
       for (int c = 0; c < V; ++c) sum += v[u][c];
     }
+    request(row0 + teams_per_block);
     for (int o = team >> 1; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
     const float mean = sum * inv_c;
     float sq = 0.f;
@@ -227,17 +237,28 @@ __global__ void __launch_bounds__(kLnThreads) layer_norm_residual_backward_kerne
   }
 }
 
-// partial [n_part][3][C] -> grad_weight, grad_bias, grad_gamma, added in the order of the workgroups
+// partial [n_part][3][C] -> grad_weight, grad_bias, grad_gamma.  A workgroup takes 8 columns; its 128 row lanes each add
+// every 128th partial row (independent loads, many in flight), then the row lanes meet through LDS in lane order: a fixed
+// summation tree, so the result does not depend on scheduling.
+constexpr int kPgCols = 8, kPgRows = 128;
 template <typename Tag>
-__global__ void __launch_bounds__(kLnThreads) layer_norm_param_grad_kernel(const LnLaunch p) {
-  const int idx = blockIdx.x * kLnThreads + threadIdx.x;
-  if (idx >= 3 * p.C) return;
+__global__ void __launch_bounds__(kPgCols * kPgRows) layer_norm_param_grad_kernel(const LnLaunch p) {
+  __shared__ float s_part[kPgRows][kPgCols + 1];
+  const int col = threadIdx.x % kPgCols, rl = threadIdx.x / kPgCols;
+  const int idx = blockIdx.x * kPgCols + col;                   // column of the [3][C] row
+  float acc = 0.f;
+  if (idx < 3 * p.C)
+    for (int w = rl; w < p.n_part; w += kPgRows) acc += p.partial[(size_t)w * 3 * p.C + idx];
+  s_part[rl][col] = acc;
+  __syncthreads();
+  if (rl != 0 || idx >= 3 * p.C) return;
+  float total = 0.f;
+#pragma unroll
+  for (int r = 0; r < kPgRows; ++r) total += s_part[r][col];
   const int q = idx / p.C, c = idx - q * p.C;
   void *dst = q == 0 ? p.grad_weight : (q == 1 ? p.grad_bias : p.grad_gamma);
   if (dst == nullptr) return;
-  float acc = 0.f;
-  for (int w = 0; w < p.n_part; ++w) acc += p.partial[(size_t)w * 3 * p.C + idx];
-  const float f[1] = {acc};
+  const float f[1] = {total};
   reinterpret_cast<typename RawWord<Tag::kBytes>::type *>(dst)[c] = Pack<Tag, 1>::encode(f);
 }
 
@@ -254,7 +275,7 @@ hipError_t launch_bwd_t(const LnLaunch &p, hipStream_t stream) {
     default: return hipErrorInvalidValue;
   }
   if (hipError_t e = hipGetLastError()) return e;
-  hipLaunchKernelGGL((layer_norm_param_grad_kernel<Tag>), dim3((unsigned)((3 * p.C + kLnThreads - 1) / kLnThreads)), block, 0, stream, p);
+  hipLaunchKernelGGL((layer_norm_param_grad_kernel<Tag>), dim3((unsigned)((3 * p.C + kPgCols - 1) / kPgCols)), dim3(kPgCols * kPgRows), 0, stream, p);
   return hipGetLastError();
 }
 
