@@ -196,6 +196,21 @@ def main():
             print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "algorithmic_MB": round(nbytes / 1e6, 2),
                               "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)}))
             return
+        if op.startswith("center_blend"):    # gate = sigmoid(y W^T + b) per (pixel, group); y (1 - gate) + x gate
+            for name, B, H, W, C, G in CFG2 + CFG5:
+                if name != shape_name:
+                    continue
+                y, x, _, _, _, go = tail_inputs(B, H, W, C, dtype)
+                w, b = (torch.randn(G, C, device=dev) / C ** 0.5).to(dtype), torch.randn(G, device=dev).to(dtype)
+                fn = (lambda: ext.center_feature_blend_forward(y, x, w, b)) if op == "center_blend_fwd" else \
+                     (lambda: ext.center_feature_blend_backward(go, y, x, w, b))
+                ms = time_op(fn, args.steps, warm=args.warmup)
+                t = B * H * W * C * y.element_size()
+                nbytes = 3 * t if op == "center_blend_fwd" else 5 * t      # y, x in, out; backward: grad_out, y, x in, two gradients out
+                print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "algorithmic_MB": round(nbytes / 1e6, 2),
+                                  "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)}))
+                return
+            sys.exit(f"--only-op {args.only_op}: no such shape")
         if op.startswith("block_tail"):      # residual + gamma * LayerNorm(y), forward / backward
             for name, B, H, W, C, G in CFG2 + CFG5:
                 if name != shape_name:

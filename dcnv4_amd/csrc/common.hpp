@@ -15,7 +15,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
 
 // dtype tags; the numeric values are the dtype codes of the C ABI
 struct F32 { static constexpr int kBytes = 4; static constexpr int kCode = 0; };
@@ -169,29 +168,6 @@ __device__ __forceinline__ Tap make_tap(float y, float x, int H, int W, uint32_t
   return t;
 }
 
-// ---------------------------------------------------------------- tiled grad_value: reach rule
-// grad_value is accumulated by workgroups that each own a 2^th x 2^tw tile of the input and
-// visit every output pixel whose reference point p0 (the centre tap at zero offset) lies within
-// `reach` pixels of the tile.  A corner is "near" when the tile that owns it visits the output
-// pixel it comes from; all other in-image corners are left to the fallback scatter.  For one
-// output pixel the near corners form a box: the union of the tiles that visit it.  Both the
-// statistics pass and the fallback pass must use exactly this box.
-struct NearBox { int y_lo, y_hi, x_lo, x_hi; };     // half-open, in input pixels
-
-__device__ __forceinline__ NearBox near_box(int p0y, int p0x, int tile_h_log2, int tile_w_log2, int reach) {
-  // tiles t with t*T - reach <= p0 < (t+1)*T + reach  <=>  floor((p0-reach-T)/T)+1 <= t <= floor((p0+reach)/T)
-  NearBox b;
-  b.y_lo = (((p0y - reach) >> tile_h_log2)) << tile_h_log2;            // arithmetic shifts = floor division
-  b.y_hi = (((p0y + reach) >> tile_h_log2) + 1) << tile_h_log2;
-  b.x_lo = (((p0x - reach) >> tile_w_log2)) << tile_w_log2;
-  b.x_hi = (((p0x + reach) >> tile_w_log2) + 1) << tile_w_log2;
-  return b;
-}
-
-__device__ __forceinline__ bool corner_is_near(const NearBox &b, int cy, int cx) {
-  return cy >= b.y_lo && cy < b.y_hi && cx >= b.x_lo && cx < b.x_hi;
-}
-
 __device__ __forceinline__ int ceil_div_signed(int a, int b) {    // b > 0
   return a >= 0 ? (a + b - 1) / b : -((-a) / b);
 }
@@ -247,34 +223,6 @@ __device__ __forceinline__ void atomic_add_element(void *base, size_t elem, floa
       __builtin_amdgcn_global_atomic_fadd_v2bf16((__attribute__((address_space(1))) bf16x2 *)addr,
                                                  __builtin_convertvector(pair, bf16x2));
   }
-}
-
-// round-to-nearest-even(a * b) as a two's-complement 64-bit integer, for |a * b| < 2^51.  The exact
-// product is formed inside a double-precision fma whose addend, 1.5 * 2^52, pushes the integer part
-// into the low mantissa bits; the addend's bit pattern has a zero low word, so removing it is one
-// 32-bit add.  Two VALU instructions per term (fp64 fma is full rate on this GPU) once the factors
-// are widened.
-__device__ __forceinline__ unsigned long long fixed_product(double a, double b) {
-  const double d = __builtin_fma(a, b, 6755399441055744.0);
-  return __builtin_bit_cast(unsigned long long, d) - 0x4338000000000000ull;
-}
-
-// round-to-nearest-even(a * b) for |a * b| < 2^22, two instructions: the product is formed inside an
-// fma whose addend pushes the integer part into the low mantissa bits.
-__device__ __forceinline__ int to_fixed32(float a, float b) {
-  return (int)(__builtin_bit_cast(uint32_t, fmaf(a, b, 12582912.f)) - 0x4B400000u);
-}
-
-// Two signed 32-bit fixed-point terms in one 64-bit addend: the sum of such words is hi * 2^32 + lo with both
-// halves signed, so the low term is sign-extended into the high word before the add.
-__device__ __forceinline__ unsigned long long pack_fixed32(int lo, int hi) {
-  return ((unsigned long long)(uint32_t)(hi + (lo >> 31)) << 32) | (uint32_t)lo;
-}
-
-// the two fields of a sum of pack_fixed32 words
-__device__ __forceinline__ int packed_field(unsigned long long a, int high) {
-  const int lo = (int)(uint32_t)a;
-  return high ? (int)(uint32_t)(a >> 32) + (lo < 0 ? 1 : 0) : lo;
 }
 
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {

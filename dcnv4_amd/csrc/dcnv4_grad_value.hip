@@ -100,9 +100,12 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
   // this lane's list: (anchor row, group of the chunk, anchor column), and its part of the group's channels
   const int n_lists = (eh + 1) * p.ng_chunk * aw;
   const int my_list = tid >> lps_log2, my_part = tid & ((1 << lps_log2) - 1);
-  const int my_row = fdiv_small(my_list, 1.f / (float)aw), my_ax = my_list - my_row * aw;      // row = anchor row * ng + group
-  const int my_ay = fdiv_small(my_row, 1.f / (float)p.ng_chunk), my_gl = my_row - my_ay * p.ng_chunk;
-  const bool list_live = my_list < n_lists && my_ay <= th && my_ax <= tw && my_gl < ng;
+  bool list_live;
+  {
+    const int row = fdiv_small(my_list, 1.f / (float)aw), ax = my_list - row * aw;      // row = anchor row * ng + group
+    const int ay = fdiv_small(row, 1.f / (float)p.ng_chunk), gl = row - ay * p.ng_chunk;
+    list_live = my_list < n_lists && ay <= th && ax <= tw && gl < ng;
+  }
   float acc[4][CW];
 #pragma unroll
   for (int k = 0; k < 4; ++k)
@@ -155,21 +158,21 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
     const int vpp = vec_park ? ng * D / kVec : ng * Dp;                 // vectors (elements) per parked pixel
     const float inv_vpp = 1.f / (float)vpp;
 
-    // a lane's offsets and modulation scalars of a strip, requested one strip ahead (before the previous strip's
-    // phase B) so that their latency hides there
-    elem_t pf_x[ROUNDS], pf_y[ROUNDS], pf_m[ROUNDS];
+    // a lane's offsets of a strip, requested one strip ahead (before the previous strip's phase B) so that their
+    // latency hides there; the modulation scalar lies in the same row and is read when it is needed
+    elem_t pf_x[ROUNDS], pf_y[ROUNDS];
     auto prefetch = [&](int s) {
       const int rows_s = (n_rows - s + n_strips - 1) / n_strips;
 #pragma unroll
       for (int v = 0; v < ROUNDS; ++v) {
-        pf_x[v] = pf_y[v] = pf_m[v] = elem_t(0);
+        pf_x[v] = pf_y[v] = elem_t(0);
         uint32_t it = item[v];
         asm volatile("" : "+v"(it));        // decoded afresh every strip: hoisted out of the loop, the fields of all rounds stay in registers
         const int r = (int)(it & 0x3ffu), col = (int)((it >> 10) & 0x3ffu), gl = (int)((it >> 20) & 0x3fu), t = (int)(it >> 26);
         if (it == ~0u || r >= rows_s) continue;
         const int ho = ho_lo + s + r * n_strips, wo = wo_lo + col;
         const elem_t *om = om_img + ((uint32_t)(ho * p.Wo + wo) * (uint32_t)p.P_pad + (uint32_t)((g0 + gl) * 3 * Kp));
-        pf_x[v] = om[2 * t]; pf_y[v] = om[2 * t + 1]; pf_m[v] = om[2 * Kp + t];
+        pf_x[v] = om[2 * t]; pf_y[v] = om[2 * t + 1];
       }
     };
     prefetch(0);
@@ -236,9 +239,9 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
         // anchor relative to the anchor grid, whose first row and column lie one cell outside the tile
         const int ay = (int)fy - ty0 + 1, ax = (int)fx - tx0 + 1;
         if ((unsigned)ay > (unsigned)th || (unsigned)ax > (unsigned)tw) continue;
-        float m = to_f(pf_m[v]);
+        const elem_t *om = om_img + ((uint32_t)(ho * p.Wo + wo) * (uint32_t)p.P_pad + (uint32_t)((g0 + gl) * 3 * Kp));
+        float m = load_f(om + 2 * Kp + t);
         if (p.softmax) {          // rare: normalise over this group's taps
-          const elem_t *om = om_img + ((uint32_t)(ho * p.Wo + wo) * (uint32_t)p.P_pad + (uint32_t)((g0 + gl) * 3 * Kp));
           float mx = load_f(om + 2 * Kp), sum = 0.f;
           for (int k = 1; k < Kp; ++k) mx = fmaxf(mx, load_f(om + 2 * Kp + k));
           for (int k = 0; k < Kp; ++k) sum += __expf(load_f(om + 2 * Kp + k) - mx);
@@ -272,14 +275,21 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
           const float fxv = __builtin_bit_cast(float, fx_bits), hxv = 1.f - fxv;
           const float w4[4] = {wa * hxv, wa * fxv, wb * hxv, wb * fxv};
           const char *g = go_lane + ((ent.w & 0x3fffu) << 4);
-          park_t gv[CW];
+          // the row in pieces of at most 32 bytes, one piece in registers at a time
+          constexpr int kPieceBytes = kLaneBytes < 32 ? kLaneBytes : 32;
+          constexpr int kPiece = kPieceBytes / kParkBytes;       // channels per piece
 #pragma unroll
-          for (int q = 0; q < kLaneBytes / 16; ++q)
-            *reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(gv) + 16 * q) = *reinterpret_cast<const u32x4 *>(g + 16 * q);
+          for (int h = 0; h < CW / kPiece; ++h) {
+            park_t gv[kPiece];
 #pragma unroll
-          for (int k = 0; k < 4; ++k)
+            for (int q = 0; q < kPieceBytes / 16; ++q)
+              *reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(gv) + 16 * q) = *reinterpret_cast<const u32x4 *>(g + kPieceBytes * h + 16 * q);
 #pragma unroll
-            for (int c = 0; c < CW; ++c) acc[k][c] = fmaf(w4[k], (float)gv[c], acc[k][c]);
+            for (int k = 0; k < 4; ++k)
+#pragma unroll
+              for (int c = 0; c < kPiece; ++c) acc[k][h * kPiece + c] = fmaf(w4[k], (float)gv[c], acc[k][h * kPiece + c]);
+            if (h + 1 < CW / kPiece) __builtin_amdgcn_sched_barrier(0);
+          }
           ent = next;
         }
       }
@@ -292,6 +302,10 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
   // same cell, so plain LDS stores and read-modify-writes suffice.  Corner 0 reaches every cell of the tile and so
   // initialises the image.
   float *s_sum = reinterpret_cast<float *>(lds32);
+  int list_now = my_list;
+  asm volatile("" : "+v"(list_now));      // the list's coordinates are decoded here, not kept in registers from the start
+  const int my_row = fdiv_small(list_now, 1.f / (float)aw), my_ax = list_now - my_row * aw;
+  const int my_ay = fdiv_small(my_row, 1.f / (float)p.ng_chunk), my_gl = my_row - my_ay * p.ng_chunk;
   const int row_floats = dcnv4_grad_value_image_stride(p.ng_chunk * Dp);      // floats between cells (an odd number of 16-byte units)
 #pragma unroll
   for (int k = 0; k < 4; ++k) {

@@ -22,7 +22,7 @@ constexpr size_t kMaxLdsPerWorkgroup = 160 * 1024;  // gfx950
 struct GradState {
   uint32_t unused0;
   uint32_t unused1;
-  uint32_t reach_needed;   // DCNv4: largest Chebyshev distance (pixels) of an in-image corner of non-zero weight from its output pixel's reference point
+  uint32_t reach_needed;   // DCNv4: ceiling of the largest Chebyshev distance (pixels) of an in-range sampling point from its output pixel's reference point
   uint32_t reserved;       // attention backward: set when a level has more tiles than the binning kernel can count
 };
 
@@ -88,7 +88,7 @@ struct DcnLaunch {
 
 // Sampling points a lane of the tiled grad_value kernel handles per strip, at most: a strip holds at most
 // gv_threads * kGradValueRounds of them.
-constexpr int kGradValueRounds = 6;
+constexpr int kGradValueRounds = 5;
 // floats between the cells of the fp32 tile image in which the corner sums meet: the cell's channels rounded up to an odd
 // number of 16-byte units, so that the lanes of one LDS instruction (consecutive cells) fall into different banks
 __host__ __device__ inline int dcnv4_grad_value_image_stride(int channels) { return ((((channels + 3) / 4) | 1) * 4); }

@@ -182,3 +182,17 @@ def test_flash_deform_attn_split_rejects_mismatched_location_dtype():
     with pytest.raises(RuntimeError, match="fp32 or of the value's dtype"):
         cabi.fda_forward_split(v, shp, st, torch.zeros(1, 3, 2, 8, device="cuda", dtype=torch.float16),
                                torch.zeros(1, 3, 2, 4, device="cuda"), 4)
+
+
+def test_stream_copy_copies_and_rejects_odd_sizes():
+    from dcnv4_amd import ext
+    src = torch.randn(1 << 20, device="cuda")
+    dst = torch.zeros_like(src)
+    ext.stream_copy(src, dst)
+    assert torch.equal(src, dst)
+    small = torch.arange(12, device="cuda", dtype=torch.float32)         # 48 bytes: three vectors, less than one workgroup
+    out = torch.zeros_like(small)
+    ext.stream_copy(small, out)
+    assert torch.equal(small, out)
+    with pytest.raises(ValueError, match="multiple of 16"):
+        ext.stream_copy(torch.zeros(3, device="cuda"), torch.zeros(3, device="cuda"))

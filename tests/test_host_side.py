@@ -209,9 +209,35 @@ def test_launch_options_are_validated_without_a_gpu():
     assert lib.dcnv4_gfx950_set_launch_option(b"reach", 7) == 0 and lib.dcnv4_gfx950_set_launch_option(b"reach", -1) == 0
     assert lib.dcnv4_gfx950_set_launch_option(b"tile", 16) == 0 and lib.dcnv4_gfx950_set_launch_option(b"tile", 0) == 0
     assert lib.dcnv4_gfx950_set_launch_option(b"tile", 12) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.dcnv4_gfx950_set_launch_option(b"gather_tile", 8) == 0 and lib.dcnv4_gfx950_set_launch_option(b"gather_tile", 0) == 0
+    assert lib.dcnv4_gfx950_set_launch_option(b"gather_tile", 5) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.dcnv4_gfx950_set_launch_option(b"gv_threads", 512) == 0 and lib.dcnv4_gfx950_set_launch_option(b"gv_threads", 0) == 0
+    assert lib.dcnv4_gfx950_set_launch_option(b"gv_threads", 256) == _lib.ERR_INVALID_ARGUMENT
     assert lib.dcnv4_gfx950_set_launch_option(b"gather", 5) == _lib.ERR_INVALID_ARGUMENT
     assert lib.dcnv4_gfx950_set_launch_option(b"nonsense", 1) == _lib.ERR_INVALID_ARGUMENT
     assert b"nonsense" in lib.dcnv4_gfx950_last_error()
+
+
+def test_layer_level_entry_points_check_their_arguments_without_a_gpu():
+    from dcnv4_amd import _lib
+    lib = _lib.load()
+    # centre-feature blend: group widths must be whole 16-byte vectors, channels a multiple of the groups
+    rc = lib.dcnv4_gfx950_center_feature_blend_forward(None, None, None, None, None, 1, 10, 24, 6, None)
+    assert rc == _lib.ERR_INVALID_ARGUMENT and b"group width" in lib.dcnv4_gfx950_last_error()
+    rc = lib.dcnv4_gfx950_center_feature_blend_forward(None, None, None, None, None, 1, 10, 64, 5, None)
+    assert rc == _lib.ERR_INVALID_ARGUMENT and b"equal groups" in lib.dcnv4_gfx950_last_error()
+    rc = lib.dcnv4_gfx950_center_feature_blend_forward(None, None, None, None, None, 1, 10, 64, 4, None)
+    assert rc == _lib.ERR_RUNTIME and b"null" in lib.dcnv4_gfx950_last_error()
+    # block tail backward: bias is needed with gamma; workspace is checked
+    rc = lib.dcnv4_gfx950_layer_norm_residual_backward(None, None, None, None, None, None, None, None, None, None, 0, 7, 10, 64, 1e-6, None)
+    assert rc == _lib.ERR_RUNTIME and b"dtype" in lib.dcnv4_gfx950_last_error()
+    # attention on un-packed rows: locations are fp32 or of the value's dtype
+    rc = lib.flash_deform_attn_gfx950_forward_split(None, None, None, None, None, None, 0, 1, 1, 16, 1, 16, 1, 4, 4, 64, 0, 0, None)
+    assert rc == _lib.ERR_RUNTIME and b"fp32 or of the value's dtype" in lib.dcnv4_gfx950_last_error()
+    rc = lib.flash_deform_attn_gfx950_forward_split(None, None, None, None, None, None, 1, 0, 1, 16, 1, 16, 6, 4, 16, 64, 0, 0, None)
+    assert rc == _lib.ERR_INVALID_ARGUMENT and b"points" in lib.dcnv4_gfx950_last_error()
+    # the streaming copy wants whole 16-byte vectors (checked after the pointers)
+    assert lib.dcnv4_gfx950_stream_copy(None, None, 32, None) == _lib.ERR_RUNTIME
 
 
 def test_launch_option_contexts_nest_and_restore_what_they_found():
@@ -244,7 +270,10 @@ def test_workspace_sizes_do_not_depend_on_launch_options_or_threads():
     fda = lambda: lib.flash_deform_attn_gfx950_backward_workspace_bytes(1, 2, 80, 4, 32, 2, 50, 4)
     base = (dcn(), fda())
     assert base[0] == 256 and base[1] > 0
-    for options in (dict(scatter="atomic"), dict(gather="direct", tile=8), dict(fda_order="rows", reach=0)):
+    ln = lambda: lib.dcnv4_gfx950_layer_norm_residual_backward_workspace_bytes(1, 5000, 112)
+    assert ln() > 0 and ln() % 16 == 0 and ln() <= 2048 * 3 * 112 * 4
+    assert lib.dcnv4_gfx950_layer_norm_residual_backward_workspace_bytes(1, 5000, 12) == 0      # not whole 16-byte vectors
+    for options in (dict(scatter="atomic"), dict(gather="direct", tile=8), dict(fda_order="rows", reach=0), dict(gv_threads=512, gather_tile=8)):
         with ext.launch_options(**options):
             assert (dcn(), fda()) == base
     seen = []
