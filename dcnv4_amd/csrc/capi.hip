@@ -145,6 +145,7 @@ struct LaunchOptions {
   int gather_tile = 0;         // largest side of an output tile of the tiled gathers (4, 8, 16); 0: default (16)
   int gv_threads = 0;          // lanes per workgroup of the grad_value kernel (512, 1024); 0: default
   int fda_order = kOptAuto;    // attention forward: 1 whole query rows per workgroup, 2 one head per workgroup
+  int fda_stage = kOptAuto;    // attention forward: 1 stage the smallest levels of a head in LDS, 2 never
 };
 thread_local LaunchOptions g_opt;
 
@@ -413,6 +414,22 @@ void fda_choose_order(FdaLaunch *F, const FdaProblem &pr, int N, int G, int D, i
   const int width = 1 << F->lanes.tpgp_log2;
   const size_t lds_per_row = (size_t)3 * L * K * sizeof(float) * (backward ? 2 : 1);
   F->nq_block = std::max(1, std::min(kBlockThreads / width, (int)(kMaxDynamicLds / lds_per_row)));
+  // Forward: the smallest levels of the head's value slice in LDS.  The level shapes live in device memory, so the
+  // choice goes by what a pyramid with a factor of two between levels would need: its last two levels hold about
+  // 6 % of the pixels.  The kernel stages whatever really fits; with nothing staged it only runs at lower occupancy.
+  F->stage_budget = 0;
+  if (backward || g_opt.fda_stage == kOptPlain || (head_bytes % 16) != 0 || width > 64) return;
+  const size_t rows_bytes = (size_t)(kFdaStagedThreads / width) * lds_per_row;
+  if (rows_bytes + 4096 > kMaxLdsPerWorkgroup - 2048) return;
+  const size_t budget = std::min<size_t>(kMaxLdsPerWorkgroup - 2048 - rows_bytes, 112 * 1024);
+  const bool pyramid_fits = L >= 3 && (size_t)N * head_bytes * 8 / 100 + 64 <= budget;
+  if (g_opt.fda_stage != kOptTiled && !pyramid_fits) return;
+  F->stage_budget = (int)(budget & ~size_t(15));
+  const int pairs = (int)(F->n_row / F->Q) * G;
+  const int sub_q = kFdaStagedThreads / width;
+  F->stage_blocks = std::max(1, std::min((256 + pairs - 1) / pairs, (F->Q + sub_q - 1) / sub_q));
+  F->stage_nq = ((F->Q + F->stage_blocks - 1) / F->stage_blocks + sub_q - 1) / sub_q * sub_q;
+  F->stage_blocks = (F->Q + F->stage_nq - 1) / F->stage_nq;
 }
 
 int images_per_launch(const FdaProblem &pr, bool backward) {
@@ -542,6 +559,7 @@ static int *launch_option_slot(const char *name) {
   if (std::strcmp(name, "gather_tile") == 0) return &g_opt.gather_tile;
   if (std::strcmp(name, "gv_threads") == 0) return &g_opt.gv_threads;
   if (std::strcmp(name, "fda_order") == 0) return &g_opt.fda_order;
+  if (std::strcmp(name, "fda_stage") == 0) return &g_opt.fda_stage;
   return nullptr;
 }
 

@@ -190,6 +190,147 @@ __global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLau
   }
 }
 
+// ------------------------------------------------------------------------------- forward, small levels in LDS
+// The gathers of the forward are bound by the rate at which the L2 answers 64- or 128-byte requests at random
+// addresses.  In a feature pyramid half of the sampling points fall on the two smallest levels, whose slice for one
+// head is a few tens of KB: a workgroup of 1024 lanes that works on ONE (image, head) copies the last levels that fit
+// its LDS budget into LDS once; then its waves walk the workgroup's queries independently, each staging the rows of its
+// own 64 lanes' queries (no workgroup barriers); sampling points on a staged level are served from LDS, the others from
+// memory as in fda_forward_kernel.  Same arithmetic in the same order per
+// (query, head): identical results.  Which levels fit is decided on the device from spatial_shapes.
+template <typename Tag, int CPT, int KT>
+__global__ void __launch_bounds__(kFdaStagedThreads) fda_forward_staged_kernel(const FdaLaunch p) {
+  extern __shared__ float lds[];
+  __shared__ int s_level_off[kMaxLevels];       // byte offset of a staged level in the stage area, -1: not staged
+  typedef Pack<Tag, CPT> pack;
+  const int LK = p.L * p.K, row_len = 3 * LK;
+  const int tpgp_log2 = p.lanes.tpgp_log2;
+  const int sub_q = kFdaStagedThreads >> tpgp_log2;       // queries per pass
+  const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
+  const int rb = (int)(blk % (uint32_t)p.stage_blocks), bg = (int)(blk / (uint32_t)p.stage_blocks);
+  const int b = bg / p.G, g = bg - b * p.G;
+  const int q_begin = rb * p.stage_nq, q_end = min(p.Q, q_begin + p.stage_nq);
+  const uint32_t head_bytes = (uint32_t)p.D * Tag::kBytes, pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
+  char *s_stage = reinterpret_cast<char *>(lds + (size_t)sub_q * row_len);      // 64 zero bytes, then the staged levels
+  const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
+
+  if (threadIdx.x == 0) {
+    int used = 64;
+    bool open = true;
+    for (int l = p.L - 1; l >= 0; --l) {
+      const Level lv = load_level(p, l);
+      const long long bytes = (long long)lv.H * lv.W * head_bytes;
+      open = open && lv.H > 0 && lv.W > 0 && used + bytes <= p.stage_budget;
+      s_level_off[l] = open ? used : -1;
+      if (open) used += (int)bytes;
+    }
+  }
+  if (threadIdx.x < 4) reinterpret_cast<u32x4 *>(s_stage)[threadIdx.x] = u32x4{0u, 0u, 0u, 0u};
+  __syncthreads();
+  for (int l = 0; l < p.L; ++l) {
+    const int off = s_level_off[l];
+    if (off < 0) continue;
+    const Level lv = load_level(p, l);
+    const int vpr = (int)head_bytes / 16, n_vec = lv.H * lv.W * vpr;
+    const float inv_vpr = 1.f / (float)vpr;
+    const uint32_t base = (uint32_t)(b * p.N + lv.start) * pix_bytes + (uint32_t)g * head_bytes;
+    for (int i = threadIdx.x; i < n_vec; i += kFdaStagedThreads) {
+      const int n = fdiv20(i, inv_vpr), v = i - n * vpr;
+      *reinterpret_cast<u32x4 *>(s_stage + off + i * 16) = buffer_load<16>(value, base + (uint32_t)n * pix_bytes + 16u * v);
+    }
+  }
+
+  __syncthreads();                        // the levels are in place; from here on the waves go their own ways
+
+  // Every wave walks its own passes of 64 / lanes-per-(query, head) queries: it stages their rows in its own slice of
+  // the row area and works on them, with no workgroup barrier (a wave's LDS operations complete in program order).
+  const int K = KT > 0 ? KT : p.K;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int qpw = kWave >> tpgp_log2;
+  const int chunk = lane & ((1 << tpgp_log2) - 1), lr = lane >> tpgp_log2;
+  const uint32_t lane_off = (uint32_t)(chunk * CPT) * Tag::kBytes;
+  float *rows = lds + (size_t)wave * qpw * row_len;
+  constexpr int EPV = 16 / Tag::kBytes;
+  const bool vec_rows = p.loc == nullptr && (row_len % EPV) == 0;
+  const int vpr = row_len / EPV;                                     // 16-byte vectors per row (vec_rows)
+  const float inv_vpr = 1.f / (float)max(vpr, 1), inv_len = 1.f / (float)row_len;
+  const float inv_2lk = 1.f / (float)(2 * LK), inv_lk = 1.f / (float)LK;
+  for (int q0 = q_begin + wave * qpw; q0 < q_end; q0 += (kFdaStagedThreads / kWave) * qpw) {
+    const int nrow = min(qpw, q_end - q0), row0 = b * p.Q + q0;
+    __builtin_amdgcn_wave_barrier();      // the previous pass has read its rows
+    if (vec_rows) {
+      const u32x4 *src = reinterpret_cast<const u32x4 *>(p.sla);
+      for (int i = lane; i < nrow * vpr; i += kWave) {
+        const int r = fdiv20(i, inv_vpr), v = i - r * vpr;
+        float f[EPV];
+        Pack<Tag, EPV>::decode(src[((size_t)(row0 + r) * p.G + g) * vpr + v], f);
+#pragma unroll
+        for (int j = 0; j < EPV; j += 4)
+          *reinterpret_cast<f32x4 *>(rows + r * row_len + v * EPV + j) = f32x4{f[j], f[j + 1], f[j + 2], f[j + 3]};
+      }
+    } else if (p.loc == nullptr) {
+      for (int i = lane; i < nrow * row_len; i += kWave) {
+        const int r = fdiv20(i, inv_len), e = i - r * row_len;
+        rows[i] = elem_f32<Tag>(p.sla, ((size_t)(row0 + r) * p.G + g) * row_len + e);
+      }
+    } else {      // locations (rounded through fp16) and logits from their own tensors
+      for (int i = lane; i < nrow * 2 * LK; i += kWave) {
+        const int r = fdiv20(i, inv_2lk), e = i - r * 2 * LK;
+        const size_t at = ((size_t)(row0 + r) * p.G + g) * (2 * LK) + e;
+        const float v = p.loc_f32 ? reinterpret_cast<const float *>(p.loc)[at] : elem_f32<Tag>(p.loc, at);
+        rows[r * row_len + e] = (float)(_Float16)v;
+      }
+      for (int i = lane; i < nrow * LK; i += kWave) {
+        const int r = fdiv20(i, inv_lk), e = i - r * LK;
+        rows[r * row_len + 2 * LK + e] = elem_f32<Tag>(p.logits, ((size_t)(row0 + r) * p.G + g) * LK + e);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (lr >= nrow || chunk >= p.lanes.tpg) continue;
+    const float *s = rows + lr * row_len;
+    float mx, inv;
+    softmax_stats(s + 2 * LK, LK, mx, inv);
+    float acc[CPT];
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) acc[c] = 0.f;
+    for (int l = 0; l < p.L; ++l) {
+      const Level lv = load_level(p, l);
+      const int off = s_level_off[l];
+      const bool staged = off >= 0;
+      // staged: byte offsets into the stage area, a corner outside the level reads the zero bytes at its start
+      const uint32_t base = staged ? (uint32_t)off + lane_off : (uint32_t)(b * p.N + lv.start) * pix_bytes + (uint32_t)g * head_bytes + lane_off;
+      const uint32_t step = staged ? head_bytes : pix_bytes;
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        const int t = l * K + k;
+        const float x = sub_rn(mul_rn(s[2 * t], (float)lv.W), 0.5f);       // flash_deform_im2col_cuda.cuh:188-189
+        const float y = sub_rn(mul_rn(s[2 * t + 1], (float)lv.H), 0.5f);
+        const float pr = __expf(s[2 * LK + t] - mx) * inv;
+        const Tap tp = make_tap(y, x, lv.H, lv.W, base, step);
+        typename pack::raw_t raw[4];
+        if (staged) {
+#pragma unroll
+          for (int cn = 0; cn < 4; ++cn)
+            raw[cn] = *reinterpret_cast<const typename pack::raw_t *>(s_stage + ((tp.valid >> cn) & 1u ? tp.off[cn] : 0u));
+        } else {
+#pragma unroll
+          for (int cn = 0; cn < 4; ++cn) raw[cn] = buffer_load<pack::kBytes>(value, tp.off[cn]);
+        }
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn) {
+          float v[CPT];
+          pack::decode(raw[cn], v);
+          const float w = pr * tp.w[cn];
+#pragma unroll
+          for (int c = 0; c < CPT; ++c) acc[c] = fmaf(w, v[c], acc[c]);
+        }
+      }
+    }
+    char *dst = (char *)p.out + ((size_t)(row0 + lr) * (p.G * p.D) + g * p.D + chunk * CPT) * Tag::kBytes;
+    *reinterpret_cast<typename pack::raw_t *>(dst) = pack::encode(acc);
+  }
+}
+
 // ------------------------------------------------------------------------------- backward
 // One kernel body, three roles (FdaBackwardMode):
 //   kFdaFull       grad_sampling_loc_attn, and grad_value scattered with fp32 buffer atomics into a
@@ -345,8 +486,25 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
   fda_unstage_grads<Tag>(s_grad, p, row0, nrow, g_fixed, heads_here);
 }
 
+template <typename Tag, int CPT>
+hipError_t launch_staged(const FdaLaunch &p, hipStream_t stream) {
+  const dim3 grid((unsigned)((p.n_row / p.Q) * p.G * p.stage_blocks)), block(kFdaStagedThreads);
+  const size_t lds = (size_t)(kFdaStagedThreads >> p.lanes.tpgp_log2) * 3 * p.L * p.K * sizeof(float) + (size_t)p.stage_budget;
+  auto go = [&](auto kernel) -> hipError_t {
+    if (hipError_t e = ensure_dynamic_lds_limit(reinterpret_cast<const void *>(kernel), kMaxLdsPerWorkgroup - 1024)) return e;
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
+    return hipGetLastError();
+  };
+  if (p.K == 4) return go(fda_forward_staged_kernel<Tag, CPT, 4>);
+  if (p.K == 8) return go(fda_forward_staged_kernel<Tag, CPT, 8>);
+  return go(fda_forward_staged_kernel<Tag, CPT, 0>);
+}
+
 template <typename Tag, int CPT, int MODE>      // MODE -1: forward
 hipError_t launch_k(const FdaLaunch &p, hipStream_t stream, dim3 grid, dim3 block, size_t lds) {
+  if constexpr (MODE < 0) {
+    if (p.stage_budget > 0) return launch_staged<Tag, CPT>(p, stream);
+  }
 #define FDA_LAUNCH(KT)                                                                                     \
   do {                                                                                                     \
     if constexpr (MODE >= 0) hipLaunchKernelGGL((fda_backward_kernel<Tag, CPT, KT, MODE>), grid, block, lds, stream, p); \

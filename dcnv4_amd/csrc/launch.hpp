@@ -116,6 +116,10 @@ struct FdaLaunch {
   int Q, N, G, D, L, K;
   int nq_block;             // queries per workgroup
   int head_major;           // forward: a workgroup takes nq_block queries of ONE head, workgroups ordered [image][head][block]
+  // forward with the smallest levels of one head's value slice staged in LDS (stage_budget > 0; implies head_major)
+  int stage_budget;         // bytes of LDS for staged levels, behind the rows; the kernel stages the last levels that fit
+  int stage_nq;             // queries one workgroup walks (in passes of as many queries as its lanes hold)
+  int stage_blocks;         // workgroups per (image, head)
   LaneMap lanes;
   // tiled grad_value path
   void *grad_value;         // [n_img, N, G, D] in the tensor dtype
@@ -216,6 +220,7 @@ hipError_t launch_dcnv4_forward_tiled(int dtype, const DcnLaunch &p, hipStream_t
 hipError_t launch_dcnv4_offset_mask_grad_tiled(int dtype, const DcnLaunch &p, hipStream_t stream);
 size_t dcnv4_tiled_gather_lds_bytes(const DcnLaunch &p, int elem_bytes);
 hipError_t launch_fda_forward(int dtype, const FdaLaunch &p, hipStream_t stream);
+constexpr int kFdaStagedThreads = 1024;      // lanes of a workgroup of the staged forward
 hipError_t launch_fda_backward(int dtype, const FdaLaunch &p, int mode, hipStream_t stream);
 hipError_t launch_fda_grad_value(int dtype, const FdaLaunch &p, hipStream_t stream);
 size_t fda_grad_value_lds_bytes(const FdaLaunch &p, int elem_bytes);

@@ -47,12 +47,13 @@ _ORDER = {"auto": 0, "rows": 1, "heads": 2}
 class launch_options:
     """Context manager over the calling thread's launch options (include/dcnv4_gfx950.h,
     ``dcnv4_gfx950_set_launch_option``): ``gather`` in auto / tiled / direct, ``scatter`` in auto / tiled / atomic,
-    ``reach`` an int or None, ``tile`` 8 / 16 / 32 or None, ``gather_tile`` 4 / 8 / 16 or None, ``gv_threads`` 512 / 1024 or None, ``fda_order`` in auto / rows / heads.  Used by the tuner,
+    ``reach`` an int or None, ``tile`` 8 / 16 / 32 or None, ``gather_tile`` 4 / 8 / 16 or None, ``gv_threads`` 512 / 1024 or None, ``fda_order`` in auto / rows / heads, ``fda_stage`` in auto / on / off.  Used by the tuner,
     by dispatch-table entries that carry options and by tests that force a kernel family; on exit every option is
     back at the value it had on entry, so contexts nest.  Results do not depend on the options beyond the rounding
     of sums."""
 
-    def __init__(self, gather=None, scatter=None, reach=None, tile=None, fda_order=None, gather_tile=None, gv_threads=None):
+    def __init__(self, gather=None, scatter=None, reach=None, tile=None, fda_order=None, gather_tile=None, gv_threads=None,
+                 fda_stage=None):
         self.values = {}
         if gather is not None:
             self.values["gather"] = _FAMILY[gather]
@@ -68,6 +69,8 @@ class launch_options:
             self.values["gv_threads"] = int(gv_threads)
         if fda_order is not None:
             self.values["fda_order"] = _ORDER[fda_order]
+        if fda_stage is not None:
+            self.values["fda_stage"] = {"auto": 0, "on": 1, "off": 2}[fda_stage]
         self.saved = {}
 
     def __enter__(self):

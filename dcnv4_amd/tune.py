@@ -67,6 +67,9 @@ def attention_candidates(direction):
     out = [("library", {})]
     for order in ("rows", "heads"):
         out.append((f"order {order}", {"fda_order": order}))
+    if direction == "fwd":
+        out.append(("heads, small levels in LDS", {"fda_order": "heads", "fda_stage": "on"}))
+        out.append(("heads, all levels from memory", {"fda_order": "heads", "fda_stage": "off"}))
     if direction == "bwd":
         out.append(("atomic scatter", {"scatter": "atomic"}))
         out.append(("atomic scatter, rows", {"scatter": "atomic", "fda_order": "rows"}))

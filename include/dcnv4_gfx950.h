@@ -65,6 +65,9 @@ const char *dcnv4_gfx950_last_error(void);
  *                LDS-tiled DCNv4 gathers owns
  *   "fda_order"  0 library's choice, 1 whole query rows per workgroup, 2 one head per workgroup
  *                (flash deformable attention forward and grad_sampling_loc_attn kernels)
+ *   "fda_stage"  0 library's choice, 1 stage the smallest levels of one head's value slice in LDS whenever the
+ *                one-head-per-workgroup order is used, 2 never (flash deformable attention forward)
+ *   "gv_threads" 0 library's choice, else 512 or 1024: lanes per workgroup of the DCNv4 grad_value kernel
  * dcnv4_gfx950_get_launch_option reads a value back, so that a caller can restore what it found.
  */
 int dcnv4_gfx950_set_launch_option(const char *name, int value);

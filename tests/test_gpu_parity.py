@@ -412,3 +412,27 @@ def test_flash_deform_attn_head_major_order_matches_oracle_and_row_order(oracle,
     cabi.assert_close(out, want, *FWD_TOL[dtype], what="output")
     cabi.assert_close(gv, wgv, *GRAD_TOL[dtype], what="grad_value")
     cabi.assert_close(gs, wgs, *GRAD_TOL[dtype], what="grad_sampling_loc_attn")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("name,B,shapes,G,D,K,Q,lo,hi", [
+    ("pyramid_two_levels_staged", 2, [(64, 64), (32, 32), (16, 16), (8, 8)], 8, 32, 4, 700, -0.05, 1.05),
+    ("all_levels_staged", 1, [(12, 20), (6, 10), (3, 5)], 3, 24, 4, 2100, -0.2, 1.2),
+    ("nothing_fits", 1, [(200, 160)], 2, 32, 8, 300, 0.0, 1.0),
+    ("k3_d8_five_levels", 2, [(9, 7), (5, 5), (4, 3), (2, 2), (1, 1)], 5, 8, 3, 1030, -0.3, 1.3),
+])
+def test_flash_deform_attn_forward_with_small_levels_staged_in_lds(oracle, name, B, shapes, G, D, K, Q, lo, hi, dtype):
+    """The forward that copies the smallest levels of one head's value slice into LDS, forced on: parity with the
+    oracle, and the same bits as the kernel that gathers everything from memory (same arithmetic per (query, head))."""
+    from dcnv4_amd import ext
+    v, shp, st, sla, _ = make_fda_inputs(B, shapes, G, D, K, Q, seed=zlib.crc32(name.encode()) % 1000, dtype=dtype, loc_lo=lo, loc_hi=hi)
+    args = (v.cuda(), shp.cuda(), st.cuda(), sla.cuda())
+    print(f"staged forward case {name} {dtype}", flush=True)
+    with ext.launch_options(fda_order="heads", fda_stage="on"):
+        out = cabi.fda_forward(*args, K)
+    with ext.launch_options(fda_order="heads", fda_stage="off"):
+        plain = cabi.fda_forward(*args, K)
+    torch.cuda.synchronize()
+    want = oracle.flash_deform_attn_forward(cabi.f64(v), shp.numpy(), st.numpy(), cabi.f64(sla), K, coord_f32=True)
+    cabi.assert_close(out, want, *FWD_TOL[dtype], what="output")
+    assert torch.equal(out, plain)
