@@ -160,6 +160,7 @@ bool fda_tiled_shape(int D, int L, int Q, int K) {
 }
 
 constexpr size_t kL2BytesPerXcd = 4u << 20;
+constexpr int kCusPerDevice = 256;      // MI355X: 8 XCDs of 32 CUs
 
 bool fda_tiled_enabled() { return g_opt.scatter != kOptPlain; }
 
@@ -423,11 +424,18 @@ void fda_choose_order(FdaLaunch *F, const FdaProblem &pr, int N, int G, int D, i
   if (rows_bytes + 4096 > kMaxLdsPerWorkgroup - 2048) return;
   const size_t budget = std::min<size_t>(kMaxLdsPerWorkgroup - 2048 - rows_bytes, 112 * 1024);
   const bool pyramid_fits = L >= 3 && (size_t)N * head_bytes * 8 / 100 + 64 <= budget;
-  if (g_opt.fda_stage != kOptTiled && !pyramid_fits) return;
-  F->stage_budget = (int)(budget & ~size_t(15));
+  // The workgroups of a launch - one per CU, 1024 lanes and most of the LDS each - should pass over the chip in two
+  // even rounds: measured on 128x128.. and 100x151.. pyramids (4 images, 8 heads of 32 fp16 channels), two rounds
+  // take 0.158 / 0.135 ms against 0.180 / 0.165 ms without staging, while counts that leave a partial last round
+  // or more rounds (every workgroup stages the levels again) lose the gain.  With few queries per workgroup, or
+  // heads wider than 64 bytes (half as many pixels fit), staging costs more than the LDS reads save.
   const int pairs = (int)(F->n_row / F->Q) * G;
   const int sub_q = kFdaStagedThreads / width;
-  F->stage_blocks = std::max(1, std::min((256 + pairs - 1) / pairs, (F->Q + sub_q - 1) / sub_q));
+  const int blocks = std::max(1, 2 * kCusPerDevice / std::max(1, pairs));
+  const bool pays = head_bytes <= 64 && (long long)F->Q >= (long long)blocks * 1024;
+  if (g_opt.fda_stage != kOptTiled && !(pyramid_fits && pays)) return;
+  F->stage_budget = (int)(budget & ~size_t(15));
+  F->stage_blocks = std::max(1, std::min(blocks, (F->Q + sub_q - 1) / sub_q));
   F->stage_nq = ((F->Q + F->stage_blocks - 1) / F->stage_blocks + sub_q - 1) / sub_q * sub_q;
   F->stage_blocks = (F->Q + F->stage_nq - 1) / F->stage_nq;
 }
