@@ -5,6 +5,7 @@
 // DCNv4_op/src/cuda/flash_deform_attn_cuda.cu:26-163, minus tensor allocation, which the
 // caller owns.
 #include <algorithm>
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -164,58 +165,69 @@ constexpr int kCusPerDevice = 256;      // MI355X: 8 XCDs of 32 CUs
 
 bool fda_tiled_enabled() { return g_opt.scatter != kOptPlain; }
 
-// Tile, group chunk, lanes per slot and strip of the tiled grad_value kernel such that a workgroup of 1024 lanes has
-// at most one (cell, group, channel part) per lane and its LDS footprint fits.
+// Tile, group chunk, lanes per slot and strip of the tiled grad_value kernel such that a workgroup has at most one
+// (anchor, group, channel part) per lane and its LDS footprint fits.
+static bool plan_grad_value_for(DcnLaunch *L, int threads, int park_bytes) {
+  auto even_split = [](int extent, int c) { const int n = (extent + c - 1) / c; return (extent + n - 1) / n; };
+  L->gv_threads = threads;
+  const size_t budget = kMaxLdsPerWorkgroup / (1024 / threads) - 512;
+  const int max_lists = threads >> L->gv_lps_log2;      // a lane per (anchor, group, channel part)
+  if (max_lists < 4) return false;
+  const int cap = g_opt.tile == 8 ? 8 : (g_opt.tile == 16 ? 16 : 31);
+  // the image is split evenly into tiles of at most cap x cap cells (all workgroups then carry the same load); the
+  // anchors of a tile, one row and one column more than its cells, must fit the workgroup
+  int cap_h = cap, cap_w = cap;
+  for (;;) {
+    L->tile_h = even_split(L->H, cap_h);
+    L->tile_w = even_split(L->W, cap_w);
+    if ((L->tile_h + 1) * (L->tile_w + 1) <= max_lists) break;
+    if (cap_h >= cap_w) cap_h = std::max(1, cap_h - 1); else cap_w = std::max(1, cap_w - 1);
+  }
+  L->tile_h_log2 = ceil_log2(L->tile_h);
+  L->tile_w_log2 = ceil_log2(L->tile_w);
+  const int anchors = (L->tile_h + 1) * (L->tile_w + 1);
+  const int max_items = kGradValueRounds * threads;
+  for (int ng = std::min({L->G, max_lists / anchors, 63, max_items / L->Kp}); ng >= 1; --ng) {
+    L->ng_chunk = ng;
+    int units = (ng * (L->gv_cw << L->gv_lps_log2) * park_bytes + 15) / 16;
+    units |= 1;                                     // an odd number of 16-byte units spreads the rows over the LDS banks
+    L->gv_go_stride = units * 16;
+    for (int s = std::min(1023, max_items / (L->Kp * ng)); s >= 1; s = s > 64 ? s - 16 : s - 1) {
+      L->strip_pix = s;
+      if (dcnv4_grad_value_lds_bytes(*L) <= budget) return true;
+    }
+  }
+  return false;
+}
+
 int plan_grad_value_tiles(DcnLaunch *L, int dtype, int batch) {
   const int D = L->D;
   L->gv_cw = D <= 8 ? 8 : 16;
   L->gv_lps_log2 = 0;
   while ((L->gv_cw << L->gv_lps_log2) < D) ++L->gv_lps_log2;
-  // Workgroups of 1024 lanes with a CU's whole LDS (measured faster than two of 512 sharing a CU on every shape with
-  // enough tiles), unless that leaves CUs without a workgroup: then 512 lanes and half the groups each.  The launch
-  // option "gv_threads" overrides.
-  auto even_split = [](int extent, int c) { const int n = (extent + c - 1) / c; return (extent + n - 1) / n; };
   const int park_bytes = dtype == DCNV4_DTYPE_F16 ? 2 : 4;
-  int threads_first = g_opt.gv_threads == 512 ? 512 : 1024;
-  if (g_opt.gv_threads == 0) {
-    const int lists_1024 = 1024 >> L->gv_lps_log2;
-    const int th = even_split(L->H, 31), tw = even_split(L->W, 31);
-    if ((th + 1) * (tw + 1) <= lists_1024) {
-      const int ng = std::max(1, std::min(L->G, lists_1024 / ((th + 1) * (tw + 1))));
-      const long long wgs = (long long)batch * ((L->H + th - 1) / th) * ((L->W + tw - 1) / tw) * ((L->G + ng - 1) / ng);
-      if (wgs < 256) threads_first = 512;
-    }
+  if (g_opt.gv_threads != 0) {
+    if (plan_grad_value_for(L, g_opt.gv_threads, park_bytes) || plan_grad_value_for(L, 1024, park_bytes)) return DCNV4_OK;
+    return fail(DCNV4_ERR_RUNTIME, "kernel with %d taps and %d group channels does not fit the tiled backward", L->Kp, D);
   }
-  for (int threads = threads_first; threads <= 1024; threads *= 2) {
-    L->gv_threads = threads;
-    const size_t budget = threads == 512 ? kMaxLdsPerWorkgroup / 2 - 512 : kMaxLdsPerWorkgroup - 512;
-    const int max_lists = threads >> L->gv_lps_log2;      // a lane per (anchor, group, channel part)
-    if (max_lists < 4) continue;
-    const int cap = g_opt.tile == 8 ? 8 : (g_opt.tile == 16 ? 16 : 31);
-    // the image is split evenly into tiles of at most cap x cap cells (all workgroups then carry the same load); the
-    // anchors of a tile, one row and one column more than its cells, must fit the workgroup
-    int cap_h = cap, cap_w = cap;
-    for (;;) {
-      L->tile_h = even_split(L->H, cap_h);
-      L->tile_w = even_split(L->W, cap_w);
-      if ((L->tile_h + 1) * (L->tile_w + 1) <= max_lists) break;
-      if (cap_h >= cap_w) cap_h = std::max(1, cap_h - 1); else cap_w = std::max(1, cap_w - 1);
-    }
-    L->tile_h_log2 = ceil_log2(L->tile_h);
-    L->tile_w_log2 = ceil_log2(L->tile_w);
-    const int anchors = (L->tile_h + 1) * (L->tile_w + 1);
-    const int max_items = kGradValueRounds * threads;
-    for (int ng = std::min({L->G, max_lists / anchors, 63, max_items / L->Kp}); ng >= 1; --ng) {
-      L->ng_chunk = ng;
-      int units = (ng * (L->gv_cw << L->gv_lps_log2) * park_bytes + 15) / 16;
-      units |= 1;                                     // an odd number of 16-byte units spreads the rows over the LDS banks
-      L->gv_go_stride = units * 16;
-      for (int s = std::min(1023, max_items / (L->Kp * ng)); s >= 1; s = s > 64 ? s - 16 : s - 1) {
-        L->strip_pix = s;
-        if (dcnv4_grad_value_lds_bytes(*L) <= budget) return DCNV4_OK;
-      }
-    }
+  // Workgroups of 1024 lanes (one per CU, the whole LDS) or of 512 (two per CU).  A workgroup takes about the same
+  // time either way - its lanes each own one anchor and walk lists of the same length - so the kernel's time goes
+  // with the number of passes the workgroups make over the chip, and a pass of 512-lane workgroups is a little
+  // shorter (two workgroups on a CU fill each other's barrier waits).  With few passes a partly filled last one
+  // counts in full.  Measured at batch 64: 56x56 with 4 groups, 1024 lanes: 4 passes, 96 us; 512 lanes: 4.5 passes,
+  // 102 us; 28x28 with 8 groups: 2 passes either way, 512 lanes 4 % faster; 256x256 with 10 groups, batch 2: 10 %.
+  double best_cost = 0.;
+  int best = 0;
+  for (int threads = 1024; threads >= 512; threads /= 2) {
+    DcnLaunch trial = *L;
+    if (!plan_grad_value_for(&trial, threads, park_bytes)) continue;
+    const double wgs = (double)batch * ((L->H + trial.tile_h - 1) / trial.tile_h) * ((L->W + trial.tile_w - 1) / trial.tile_w) *
+                       ((L->G + trial.ng_chunk - 1) / trial.ng_chunk);
+    const double passes = wgs / (double)(kCusPerDevice * (1024 / threads));
+    const double cost = (passes < 6. ? std::ceil(passes) : passes) * (threads == 512 ? 0.92 : 1.0);
+    if (best == 0 || cost < best_cost) { best = threads; best_cost = cost; }
   }
+  if (best != 0 && plan_grad_value_for(L, best, park_bytes)) return DCNV4_OK;
   return fail(DCNV4_ERR_RUNTIME, "kernel with %d taps and %d group channels does not fit the tiled backward", L->Kp, D);
 }
 

@@ -92,6 +92,8 @@ KERNEL_PATHS = {
     "reach9": dict(reach=9),
     "tile16": dict(tile=16),                                   # grad_value on 16x16 tiles, four groups each
     "tile8_reach1": dict(tile=8, reach=1),
+    "gv512": dict(gv_threads=512),                             # grad_value workgroups of 512 / 1024 lanes
+    "gv1024": dict(gv_threads=1024),
 }
 
 
