@@ -417,17 +417,6 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
 #pragma unroll
           for (int cn = 0; cn < 4; ++cn) tp.off[cn] = kDropOffset;
         }
-        if constexpr (MODE == kFdaNoScatter) {
-          if (chunk == 0) {
-            uint32_t key = kFdaKeyOutside;
-            if (tp.valid != 0)
-              key = (tp.y0 + 1 >= kFdaKeyFieldMax || tp.x0 + 1 >= kFdaKeyFieldMax) ? kFdaKeySaturated
-                                                                                  : ((uint32_t)(tp.y0 + 1) << 8) | (uint32_t)(tp.x0 + 1);
-            const size_t slot = (((size_t)b_local * p.G + g) * p.L + l) * fda_key_stride(p.Q, K) + (size_t)q * K + k;
-            p.keys[slot] = (uint16_t)key;
-            p.recs[slot] = f32x4_t{x, y, pr, 0.f};
-          }
-        }
         if constexpr (MODE == kFdaFallback) {
 #pragma unroll
           for (int cn = 0; cn < 4; ++cn) {
@@ -478,11 +467,38 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
       for (int t = 0; t < LK; ++t) {
         const float pr = __expf(s[2 * LK + t] - mx) * inv;
         gs[2 * LK + t] = pr * (gs[2 * LK + t] - dot_rg);
+        // the probability takes the logit's place for the record pass below (only this wave reads the row, and its
+        // lanes are past the tap loop)
+        if constexpr (MODE == kFdaNoScatter) const_cast<float *>(s)[2 * LK + t] = pr;
       }
     }
   }
   if constexpr (MODE == kFdaFallback) return;
   __syncthreads();
+  if constexpr (MODE == kFdaNoScatter) {
+    // Keys and records of the workgroup's sampling points, one lane per point in the order they lie in memory
+    // ([head][level][query][point]: whole 16-byte records side by side), from the staged rows.
+    const size_t stride = fda_key_stride(p.Q, K);
+    for (int hl = 0; hl < heads_here * p.L; ++hl) {
+      const int gh = hl / p.L, l = hl - gh * p.L, g = g_fixed + gh;
+      const Level lv = load_level(p, l);
+      for (int i = threadIdx.x; i < nrow * K; i += blockDim.x) {
+        const int lr = i / K, k = i - lr * K, t = l * K + k;
+        const float *s = s_in + (lr * heads_here + gh) * row_len;
+        const float x = sub_rn(mul_rn(s[2 * t], (float)lv.W), 0.5f);
+        const float y = sub_rn(mul_rn(s[2 * t + 1], (float)lv.H), 0.5f);
+        const Tap tp = make_tap(y, x, lv.H, lv.W, 0u, 0u);
+        uint32_t key = kFdaKeyOutside;
+        if (tp.valid != 0)
+          key = (tp.y0 + 1 >= kFdaKeyFieldMax || tp.x0 + 1 >= kFdaKeyFieldMax) ? kFdaKeySaturated
+                                                                              : ((uint32_t)(tp.y0 + 1) << 8) | (uint32_t)(tp.x0 + 1);
+        const int b_local = (row0 + lr) / p.Q, q = (row0 + lr) - b_local * p.Q;
+        const size_t slot = (((size_t)b_local * p.G + g) * p.L + l) * stride + (size_t)q * K + k;
+        p.keys[slot] = (uint16_t)key;
+        p.recs[slot] = f32x4_t{x, y, s[2 * LK + t], 0.f};
+      }
+    }
+  }
   fda_unstage_grads<Tag>(s_grad, p, row0, nrow, g_fixed, heads_here);
 }
 
