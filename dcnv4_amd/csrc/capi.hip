@@ -241,6 +241,7 @@ constexpr int kTiledGatherThreads = 512;     // launch bound of the tiled gather
 bool plan_gather_tiles(DcnLaunch *L, int s) {
   L->gt_h = L->gt_w = L->gt_ng = L->gt_wh = L->gt_ww = 0;
   L->gt_lpg = 1;
+  L->gt_pad = 16;
   L->gt_reach = reach_setting();
   if (!tiled_gather_enabled() || L->softmax) return false;
   const int lane_bytes = L->D * s;
@@ -281,7 +282,11 @@ bool plan_gather_tiles(DcnLaunch *L, int s) {
   const int want_lanes = std::min(384, Ho * Wo * L->G * L->gt_lpg);
   const int shorter = g_opt.reach < 0 ? 2 : 0;        // an explicit reach is kept
   for (int d = 0; d <= shorter && d <= R - 2; ++d)
-    if (fit(half, R - d, want_lanes)) return true;
+    for (int pad = 16; pad >= (d == 0 ? 0 : 16); pad -= 16) {       // the full reach is worth more than the padding between the cells
+      L->gt_pad = pad;
+      if (fit(half, R - d, want_lanes)) return true;
+    }
+  L->gt_pad = 16;
   if (fit(half, R, 1) || fit(whole, R, 1)) return true;
   L->gt_h = L->gt_w = L->gt_ng = L->gt_wh = L->gt_ww = 0;
   L->gt_reach = R;

@@ -24,10 +24,6 @@
 #include "common.hpp"
 #include "launch.hpp"
 
-#ifndef GT_PAD
-#define GT_PAD 16
-#endif
-
 namespace dcn {
 namespace {
 
@@ -274,7 +270,7 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_forward_tiled_kernel(cons
   typedef Pack<Tag, EPV> pack;
   const TileGeom t = tile_geometry(p);
   const int Kp = p.Kp;
-  const int cell_stride = p.gt_ng * p.D * Tag::kBytes + GT_PAD;
+  const int cell_stride = p.gt_ng * p.D * Tag::kBytes + p.gt_pad;
   char *s_win = reinterpret_cast<char *>(lds128);
   elem_t *s_om = reinterpret_cast<elem_t *>(s_win + (size_t)(p.gt_wh * p.gt_ww + p.gt_ww + 2) * cell_stride);
   stage_tile<Tag, NV>(p, t, s_win, s_om, cell_stride);
@@ -417,7 +413,7 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
   typedef Pack<Tag, EPV> pack;
   const TileGeom t = tile_geometry(p);
   const int Kp = p.Kp;
-  const int cell_stride = p.gt_ng * p.D * Tag::kBytes + GT_PAD;
+  const int cell_stride = p.gt_ng * p.D * Tag::kBytes + p.gt_pad;
   char *s_win = reinterpret_cast<char *>(lds128);
   elem_t *s_om = reinterpret_cast<elem_t *>(s_win + (size_t)(p.gt_wh * p.gt_ww + p.gt_ww + 2) * cell_stride);
   __shared__ uint32_t s_reach;
@@ -640,7 +636,7 @@ hipError_t launch_any(int dtype, const DcnLaunch &p, hipStream_t stream) {
 }  // namespace
 
 size_t dcnv4_tiled_gather_lds_bytes(const DcnLaunch &p, int elem_bytes) {
-  const size_t cell = (size_t)p.gt_ng * p.D * elem_bytes + GT_PAD;
+  const size_t cell = (size_t)p.gt_ng * p.D * elem_bytes + p.gt_pad;
   return (size_t)(p.gt_wh * p.gt_ww + p.gt_ww + 2) * cell +                     // window + zero cells
          (((size_t)p.gt_h * p.gt_w * p.gt_ng * 3 * p.Kp * elem_bytes + 15) & ~size_t(15));   // offset_mask slices
 }

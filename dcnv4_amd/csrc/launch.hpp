@@ -82,6 +82,7 @@ struct DcnLaunch {
   int gt_h, gt_w;           // output tile one workgroup owns
   int gt_ng;                // groups per workgroup
   int gt_lpg;               // lanes per (pixel, group): 1, or 2 when a group is 64 bytes or wider
+  int gt_pad;               // bytes between the cells of the staged window (16: fewer LDS bank conflicts; 0: a larger window fits)
   int gt_wh, gt_ww;         // largest input window (rows, columns of cells) a tile stages
   int gt_reach;             // input pixels around an output pixel's reference point that the window covers
 };
