@@ -512,8 +512,7 @@ hipError_t launch_staged(const FdaLaunch &p, hipStream_t stream) {
     return hipGetLastError();
   };
   if (p.K == 4) return go(fda_forward_staged_kernel<Tag, CPT, 4>);
-  if (p.K == 8) return go(fda_forward_staged_kernel<Tag, CPT, 8>);
-  return go(fda_forward_staged_kernel<Tag, CPT, 0>);
+  return go(fda_forward_staged_kernel<Tag, CPT, 0>);      // (unrolled for 8 points the kernel spills a hundred registers)
 }
 
 template <typename Tag, int CPT, int MODE>      // MODE -1: forward
