@@ -205,7 +205,7 @@ int plan_grad_value_tiles(DcnLaunch *L, int dtype, int batch) {
   L->gv_cw = D <= 8 ? 8 : 16;
   L->gv_lps_log2 = 0;
   while ((L->gv_cw << L->gv_lps_log2) < D) ++L->gv_lps_log2;
-  const int park_bytes = dtype == DCNV4_DTYPE_F16 ? 2 : 4;
+  const int park_bytes = 4;      // grad_out rows are parked as fp32 for every tensor dtype
   if (g_opt.gv_threads != 0) {
     if (plan_grad_value_for(L, g_opt.gv_threads, park_bytes) || plan_grad_value_for(L, 1024, park_bytes)) return DCNV4_OK;
     return fail(DCNV4_ERR_RUNTIME, "kernel with %d taps and %d group channels does not fit the tiled backward", L->Kp, D);

@@ -40,10 +40,9 @@ namespace dcn {
 namespace {
 
 
-// grad_out is parked in LDS as it is for fp32 and fp16 tensors (fp16 feeds mixed-precision FMAs directly)
-// and widened to fp32 for bf16.
+// grad_out is parked in LDS as fp32, also for 16-bit tensors: parked as fp16 and fed to mixed-precision FMAs it
+// takes half the LDS, but the kernel measured 5-8 % slower (T stage 1 fp16 backward 0.169 -> 0.156 ms with fp32 rows).
 template <typename Tag> struct ParkType { typedef float type; };
-template <> struct ParkType<F16> { typedef _Float16 type; };
 
 __device__ __forceinline__ int fdiv_small(int n, float inv) { return (int)(((float)n + 0.5f) * inv); }   // exact for n < 2^20
 
@@ -194,7 +193,7 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
         char *dst = s_go + px * go_stride;
         if (vec_park) {
           const vec_t raw = *reinterpret_cast<const vec_t *>(src + u * kVec);
-          if constexpr (Tag::kCode == BF16::kCode) {
+          if constexpr (Tag::kBytes == 2) {
             float f[kVec];
             Pack<Tag, kVec>::decode(raw, f);
             f32x4 *d4 = reinterpret_cast<f32x4 *>(dst + u * kVec * 4);
