@@ -224,7 +224,10 @@ int plan_grad_value_tiles(DcnLaunch *L, int dtype, int batch) {
     const double wgs = (double)batch * ((L->H + trial.tile_h - 1) / trial.tile_h) * ((L->W + trial.tile_w - 1) / trial.tile_w) *
                        ((L->G + trial.ng_chunk - 1) / trial.ng_chunk);
     const double passes = wgs / (double)(kCusPerDevice * (1024 / threads));
-    const double cost = (passes < 6. ? std::ceil(passes) : passes) * (threads == 512 ? 0.92 : 1.0);
+    // a tile that is a whole image revisits nothing and needs no reach statistic (28x28 with 8 groups at batch 64:
+    // 1024 lanes and whole images 2-3 % faster than 512 lanes and half images)
+    const bool whole = trial.tile_h >= L->H && trial.tile_w >= L->W;
+    const double cost = (passes < 6. ? std::ceil(passes) : passes) * (threads == 512 ? 0.92 : 1.0) * (whole ? 0.9 : 1.0);
     if (best == 0 || cost < best_cost) { best = threads; best_cost = cost; }
   }
   if (best != 0 && plan_grad_value_for(L, best, park_bytes)) return DCNV4_OK;
@@ -672,8 +675,13 @@ static int dcn_backward_impl(const void *value, const void *offset_mask, const v
     return fail(DCNV4_ERR_RUNTIME, "one image of %d output pixels is too large for the backward", base.Q);
   const bool gather_tiled = plan_gather_tiles(&base, pr.s);
   base.state = static_cast<GradState *>(workspace);
-  hipLaunchKernelGGL(init_state_kernel, dim3(1), dim3(64), 0, st, base.state);
-  if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);
+  // When a grad_value tile is a whole image its workgroups visit every output pixel whatever the reach: nobody reads
+  // the statistic that the first kernel folds into the state, and the launch that resets it is left out.
+  base.gv_whole = (base.tile_h >= base.H && base.tile_w >= base.W) ? 1 : 0;
+  if (!base.gv_whole) {
+    hipLaunchKernelGGL(init_state_kernel, dim3(1), dim3(64), 0, st, base.state);
+    if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);
+  }
   const int per = images_per_launch(pr, false);
   for (int pass = 0; pass < 2; ++pass) {
     for (int b0 = 0; b0 < batch; b0 += per) {

@@ -87,7 +87,7 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
   // output pixels this tile visits: reference point (centre tap at zero offset) within `reach` of the tile
   const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
   const int cy0 = half_h - p.ph, cx0 = half_w - p.pw, Ho = p.Q / p.Wo;
-  const int reach = (int)min(p.state->reach_needed, 1u << 20);
+  const int reach = p.gv_whole ? (1 << 20) : (int)min(p.state->reach_needed, 1u << 20);
   const int ho_lo = max(0, ceil_div_signed(ty0 - reach - cy0, p.sh));
   const int ho_hi = min(Ho, ceil_div_signed(ty0 + eh + reach - cy0, p.sh));
   const int wo_lo_all = max(0, ceil_div_signed(tx0 - reach - cx0, p.sw));

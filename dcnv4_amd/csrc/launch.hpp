@@ -77,6 +77,7 @@ struct DcnLaunch {
   int gv_threads;           // lanes per workgroup of the grad_value kernel: 512 or 1024
   int gv_cw;                // channels a lane accumulates per corner: 8 or 16
   int gv_lps_log2;          // log2 of the lanes that share one (cell, group): group width / gv_cw, rounded up to a power of two
+  int gv_whole;             // 1: a tile is a whole image, so every output pixel is visited and the reach statistic is not read
   int gv_go_stride;         // bytes between the parked grad_out rows of consecutive pixels (an odd number of 16-byte units)
   // LDS-tiled gather path (forward and grad_offset_mask); gt_h == 0: not planned
   int gt_h, gt_w;           // output tile one workgroup owns
