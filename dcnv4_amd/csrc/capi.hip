@@ -117,6 +117,26 @@ hipError_t clear_async(void *dst, size_t n_words, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// The same two, run only when the attention backward's binning kernel has raised its flag (GradState::reserved): the
+// fallback kernel then sums in an fp32 image that is cleared before it and narrowed after it.
+__global__ void __launch_bounds__(256) clear_if_flagged_kernel(const GradState *state, uint32_t *dst, size_t n16) {
+  if (state->reserved == 0u) return;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
+    reinterpret_cast<u32x4 *>(dst)[i] = u32x4{0, 0, 0, 0};
+}
+
+template <typename Tag>
+__global__ void __launch_bounds__(256) narrow_if_flagged_kernel(const GradState *state, const float *src, void *dst, size_t n8) {
+  if (state->reserved == 0u) return;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += stride) {
+    const f32x4 a = reinterpret_cast<const f32x4 *>(src)[2 * i], b = reinterpret_cast<const f32x4 *>(src)[2 * i + 1];
+    const float f[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    reinterpret_cast<u32x4 *>(dst)[i] = Pack<Tag, 8>::encode(f);
+  }
+}
+
 hipError_t narrow_async(int dtype, const float *src, void *dst, size_t n, hipStream_t stream) {
   if (n == 0) return hipSuccess;
   const size_t n8 = n / 8;
@@ -847,7 +867,8 @@ size_t flash_deform_attn_gfx950_backward_workspace_bytes(int dtype, int batch, i
                                                          int num_points) {
   if (elem_bytes(dtype) == 0 || batch <= 0 || spatial_size <= 0 || num_heads <= 0 || head_channels <= 0) return 0;
   size_t need = 0;
-  if (elem_bytes(dtype) == 2) need = round16((size_t)batch * spatial_size * num_heads * head_channels * sizeof(float));
+  // 16-bit tensors: an fp32 image of grad_value behind the state block (the atomic paths sum in fp32 and narrow once)
+  if (elem_bytes(dtype) == 2) need = kStateBytes + round16((size_t)batch * spatial_size * num_heads * head_channels * sizeof(float));
   if (fda_tiled_shape(head_channels, num_levels, num_query, num_points))
     need = std::max(need, fda_scratch(elem_bytes(dtype), batch, spatial_size, num_heads, head_channels, num_levels, num_query, num_points).total);
   return need;
@@ -918,7 +939,22 @@ static int fda_backward_impl(const void *value, const int64_t *spatial_shapes, c
         if (pass == 0) fda_choose_order(&F, pr, spatial_size, num_heads, head_channels, num_levels, num_points, true);
         if (pass == 0) e = launch_fda_backward(dtype, F, kFdaNoScatter, st);
         else if (pass == 1) e = launch_fda_grad_value(dtype, F, st);
-        else e = launch_fda_backward(dtype, F, kFdaFallback, st);
+        else {
+          // The fallback sums with fp32 atomics: straight into grad_value for fp32 tensors (the tiled kernel has left
+          // it zeroed), for 16-bit tensors into an fp32 image that takes the place of the - by now dead - keys and
+          // records, is cleared first and narrowed afterwards; all three launches return at once without the flag.
+          const size_t n = (size_t)nb * pr.img_elems;      // a multiple of 8: heads of 8, 16, 24 or 32 channels
+          float *acc = pr.s == 2 ? reinterpret_cast<float *>(ws + kStateBytes) + (size_t)b0 * pr.img_elems : static_cast<float *>(F.grad_value);
+          F.grad_value_acc = acc;
+          const dim3 grid((unsigned)std::min<size_t>((n / 8 + 255) / 256, 4096)), block(256);
+          if (pr.s == 2) hipLaunchKernelGGL(clear_if_flagged_kernel, grid, block, 0, st, base.state, reinterpret_cast<uint32_t *>(acc), n / 4);
+          e = launch_fda_backward(dtype, F, kFdaFallback, st);
+          if (e == hipSuccess && dtype == DCNV4_DTYPE_F16)
+            hipLaunchKernelGGL(narrow_if_flagged_kernel<F16>, grid, block, 0, st, base.state, acc, F.grad_value, n / 8);
+          if (e == hipSuccess && dtype == DCNV4_DTYPE_BF16)
+            hipLaunchKernelGGL(narrow_if_flagged_kernel<BF16>, grid, block, 0, st, base.state, acc, F.grad_value, n / 8);
+          if (e == hipSuccess) e = hipGetLastError();
+        }
         if (e) return hip_fail("flash_deform_attn backward launch", e);
       }
     }

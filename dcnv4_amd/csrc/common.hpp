@@ -205,26 +205,7 @@ __device__ __forceinline__ float cluster_sum(float v, int width) {
   return v;
 }
 
-// ---------------------------------------------------------------- atomics and wave reductions
-// Adds v to element `elem` of a tensor of dtype Tag with one hardware atomic (packed pair for the
-// 16-bit types, the untouched half gets +0).
-template <typename Tag>
-__device__ __forceinline__ void atomic_add_element(void *base, size_t elem, float v) {
-  if constexpr (Tag::kBytes == 4) {
-    unsafeAtomicAdd(reinterpret_cast<float *>(base) + elem, v);
-  } else {
-    char *addr = reinterpret_cast<char *>(base) + (elem & ~size_t(1)) * 2;
-    const bool hi = elem & 1;
-    const f32x2 pair = {hi ? 0.f : v, hi ? v : 0.f};
-    if constexpr (Tag::kCode == F16::kCode)
-      __builtin_amdgcn_global_atomic_fadd_v2f16((__attribute__((address_space(1))) f16x2 *)addr,
-                                                __builtin_convertvector(pair, f16x2));
-    else
-      __builtin_amdgcn_global_atomic_fadd_v2bf16((__attribute__((address_space(1))) bf16x2 *)addr,
-                                                 __builtin_convertvector(pair, bf16x2));
-  }
-}
-
+// ---------------------------------------------------------------- wave reductions
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
   for (int o = 32; o > 0; o >>= 1) v = max(v, (uint32_t)__shfl_xor((int)v, o, kWave));
   return v;

@@ -338,7 +338,7 @@ __global__ void __launch_bounds__(kFdaStagedThreads) fda_forward_staged_kernel(c
 //   kFdaNoScatter  grad_sampling_loc_attn, plus what the tiled grad_value kernel needs: per sampling point a key
 //                  and a (position, softmax probability) record, and grad_out regrouped by head
 //   kFdaFallback   exits at once unless the binning kernel flagged a level it cannot hold; then it scatters
-//                  with atomics in the tensor dtype into grad_value, which the tiled kernel has left zeroed
+//                  with fp32 atomics into an fp32 image (grad_value itself for fp32 tensors, left zeroed by the tiled kernel)
 template <typename Tag, int CPT, int KT, int MODE>
 __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLaunch p) {
   extern __shared__ float lds[];
@@ -417,14 +417,14 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
 #pragma unroll
           for (int cn = 0; cn < 4; ++cn) tp.off[cn] = kDropOffset;
         }
-        if constexpr (MODE == kFdaFallback) {
+        if constexpr (MODE == kFdaFallback) {      // fp32 atomics into the fp32 image (the tensor itself for fp32 tensors)
 #pragma unroll
           for (int cn = 0; cn < 4; ++cn) {
-            if (!(tp.valid & (1u << cn)) || !active) continue;
             const float w = pr * tp.w[cn];
-            const size_t e0 = ((((size_t)b * p.N + lv.start + (size_t)(tp.y0 + (cn >> 1)) * lv.W + tp.x0 + (cn & 1)) * p.G + g) * p.D) + chunk * CPT;
+            const uint32_t aoff = (tp.off[cn] == kDropOffset) ? kDropOffset : tp.off[cn] * (4 / Tag::kBytes);
 #pragma unroll
-            for (int c = 0; c < CPT; ++c) atomic_add_element<Tag>(p.grad_value, e0 + c, go[c] * w);
+            for (int c = 0; c < CPT; ++c)
+              __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(go[c] * w, gacc, aoff + 4 * c, 0, 0);
           }
           continue;
         }

@@ -149,7 +149,7 @@ __host__ __device__ inline size_t fda_key_stride(int Q, int K) { return ((size_t
 enum FdaBackwardMode {
   kFdaFull = 0,        // grad_sampling_loc_attn + fp32 atomic scatter of grad_value (any head width)
   kFdaNoScatter = 1,   // grad_sampling_loc_attn + keys + probabilities, no scatter
-  kFdaFallback = 2,    // scatter with atomics in the tensor dtype, only when the binning kernel gave up on a level
+  kFdaFallback = 2,    // scatter with fp32 atomics into an fp32 image, only when the binning kernel gave up on a level
 };
 
 // Accumulator channels per cell of the tiled flash-attention grad_value kernel (head width rounded up to

@@ -220,6 +220,11 @@ FDA_PATH_CASES = {
     "crowded_small_level": (1, [(3, 3), (20, 17)], 2, 16, 8, 6000, (0.0, 1.0)),
     # a level wider than the 16-bit fields of a key: the scan recomputes those positions
     "level_wider_than_a_key": (1, [(1, 65530), (2, 3)], 1, 8, 4, 300, (0.0, 1.0)),
+    # a level of more 8x8 tiles (8320) than the binning kernel counts: the binned kernels stand back and the atomic
+    # fallback kernel adds everything
+    "level_of_more_tiles_than_binned": (1, [(1024, 520), (4, 4)], 1, 8, 4, 300, (0.0, 1.0)),
+    # ... with 12000 points on a few cells of it: the fallback has to sum them in fp32 whatever the tensor dtype
+    "level_of_more_tiles_than_binned_crowded": (1, [(1024, 520), (4, 4)], 1, 8, 4, 3000, (0.5, 0.503)),
 }
 
 
@@ -239,7 +244,7 @@ def test_flash_deform_attn_backward_paths_match_oracle(oracle, name, scatter, dt
         gv, gs = cabi.fda_backward(v.cuda(), shp.cuda(), st.cuda(), sla.cuda(), go.cuda(), K)
     torch.cuda.synchronize()
     rtol, atol = GRAD_TOL[dtype]
-    if name == "crowded_small_level":       # thousands of terms per cell: the tolerance scales with the sum's magnitude
+    if name in ("crowded_small_level", "level_of_more_tiles_than_binned_crowded"):       # thousands of terms per cell: the tolerance scales with the sum's magnitude
         atol = atol * float(np.abs(wgv).max())
     cabi.assert_close(gv, wgv, rtol, atol, what="grad_value")
     cabi.assert_close(gs, wgs, *GRAD_TOL[dtype], what="grad_sampling_loc_attn")
