@@ -6,31 +6,29 @@
 // window around the query to exploit.  Instead the sampling points are first BINNED by the tile
 // of their level they touch, and then a workgroup that OWNS a tile adds them up in LDS:
 //
-//   * the grad_sampling_loc_attn kernel, which runs first, leaves one 16-bit key (integer position of
-//     the first corner, or "outside") and the softmax probability per sampling point, both laid out
-//     [image][head][level][query][point], and the maximum of |grad_out| in GradState;
+//   * the grad_sampling_loc_attn kernel, which runs first, leaves per sampling point a 16-bit key (integer position
+//     of the first corner, or "outside") and a 16-byte record (position, softmax probability), both laid out
+//     [image][head][level][query][point], and grad_out regrouped by head;
 //   * fda_bin_points_kernel: one workgroup per chunk of 8192 points of one (image, head, level)
 //     counting-sorts the chunk by tile in LDS (a point whose 2x2 corner block straddles tiles is
 //     listed under each of them) and writes the sorted point ids to the chunk's region of the
 //     workspace plus one (offset, count) word per tile to a table - no global atomics, no host
 //     round trip, every chunk independent;
-//   * fda_grad_value_kernel: persistent workgroups walk (tile, image, head) items, smallest level
-//     first.  An item collects its tile's slices of all chunk lists into LDS and applies them in
-//     batches: one lane per point rebuilds the position from sampling_loc_attn and, with the stored
-//     probability, the four corner weights, while the previous batch is being applied (two record
-//     buffers, one barrier per batch; all loads are requested one batch ahead); then a row of 8 lanes
-//     per point, each holding its own channels of the point's grad_out row in registers, adds the
-//     contributions to the tile's accumulators with 64-bit integer
-//     LDS atomics on fixed-point values (normalised by max |grad_out|; probability * bilinear weight
-//     <= 1), so the result does not depend on the order of arrival and is bit-reproducible;
+//   * fda_grad_value_kernel: persistent workgroups walk (tile, image, head) items, an XCD staying with one
+//     (image, head) pair and going through its levels coarsest first.  An item collects its tile's slices of all
+//     chunk lists into LDS and applies them in batches of 256 points: records and grad_out rows are requested one
+//     batch ahead; per batch every corner inside the tile draws a rank in its cell's list with an integer LDS
+//     atomic, a 64-entry scan gives every cell a segment, the (weight, parked row) entries are placed, and the
+//     lanes of a cell walk the cell's entries with fp32 sums in registers.  The arithmetic is the reference's
+//     (every term rounded to fp32, summed in fp32, rounded once to the tensor dtype); the order of the terms of a
+//     cell follows the ranks, which the atomics fix per run, like the reference's atomics do;
 //   * the finished tile is written to grad_value with plain stores in the tensor dtype.
 //
 // Tiles are at most 8x8 cells and every level is cut into 16 of them or more, so items stay
 // small (several workgroups share a CU and hide each other's latencies) and comparable in size.
 // Levels and tile shapes are derived on the device from the spatial_shapes tensor; the host never
 // reads it.  A level with more tiles than the binning kernel's LDS histogram holds raises a flag in
-// GradState: grad_value is then left zeroed for the atomic fallback kernel, like for non-finite
-// statistics.
+// GradState: this kernel then writes zeros and the atomic fallback kernel adds everything (in fp32).
 #include <algorithm>
 
 #include "common.hpp"
