@@ -11,7 +11,7 @@
 // contiguous kilobyte.  Corners outside the image are range-dropped by the buffer descriptor.
 // Backward: coordinate / modulation partials are summed over the lanes of a (pixel, group) with
 // DPP, parked in LDS and written back as whole rows (padding tail included, so the gradient
-// tensor needs no separate clearing); the value gradient is scattered with fp32 buffer atomics.
+// tensor needs no separate clearing); the value gradient is the tiled gather of dcnv4_grad_value.hip.
 #include <algorithm>
 
 #include "common.hpp"
