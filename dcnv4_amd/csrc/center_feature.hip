@@ -9,7 +9,7 @@
 // channels, a lane holds VPL 16-byte vectors of it; a vector lies inside one group (the entry point checks that
 // the group width is a whole number of vectors).  The G dot products are formed one group at a time: every
 // lane multiplies its channels with the matching piece of W[g, :] (the teams of a wave read the same addresses),
-// an xor-shuffle closes the sum inside the team, and the lanes whose vectors belong to group g keep the gate.
+// a butterfly of DPP moves (and shuffles beyond 16 lanes) closes the sum inside the team, and the lanes whose vectors belong to group g keep the gate.
 // fp32 arithmetic, one rounding.
 //
 // Backward, for grad_out q:  grad_x = q * gate;  d gate[g] = sum over the group's channels of q * (x - y);
@@ -79,10 +79,8 @@ __global__ void __launch_bounds__(kCfThreads) center_feature_blend_kernel(const 
         }
       }
     }
-    for (int o = team >> 1; o > 0; o >>= 1) {
-      z += __shfl_xor(z, o, kWave);
-      if constexpr (BWD) dgate += __shfl_xor(dgate, o, kWave);
-    }
+    z = cluster_sum(z, team);
+    if constexpr (BWD) dgate = cluster_sum(dgate, team);
     float bias_g[1];
     Pack<Tag, 1>::decode(reinterpret_cast<const typename RawWord<Tag::kBytes>::type *>(p.bias)[g], bias_g);
     const float s = sigmoid(z + bias_g[0]);

@@ -198,10 +198,21 @@ __device__ __forceinline__ float dpp_quad_xor1(float v) {
 __device__ __forceinline__ float dpp_quad_xor2(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true));
 }
+// Inside a row of 16 lanes the two further steps are DPP mirrors: once every lane holds its quad's sum, the lane
+// mirrored within 8 (then within 16) lies in the other quad (the other half), so adding it doubles the span just as
+// xor-4 (xor-8) would, without the LDS crossbar.
+__device__ __forceinline__ float dpp_row_half_mirror(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float dpp_row_mirror(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true));
+}
 __device__ __forceinline__ float cluster_sum(float v, int width) {
   if (width >= 2) v += dpp_quad_xor1(v);
   if (width >= 4) v += dpp_quad_xor2(v);
-  for (int o = 4; o < width; o <<= 1) v += __shfl_xor(v, o, kWave);
+  if (width >= 8) v += dpp_row_half_mirror(v);
+  if (width >= 16) v += dpp_row_mirror(v);
+  for (int o = 16; o < width; o <<= 1) v += __shfl_xor(v, o, kWave);
   return v;
 }
 

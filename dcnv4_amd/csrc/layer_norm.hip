@@ -47,7 +47,7 @@ __global__ void __launch_bounds__(kLnThreads) layer_norm_residual_kernel(const L
       for (int c = 0; c < V; ++c) v[u][c] = 0.f;
     }
   }
-  for (int o = team >> 1; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
+  sum = cluster_sum(sum, team);
   const float mean = sum / (float)p.C;
   float sq = 0.f;
 #pragma unroll
@@ -55,7 +55,7 @@ __global__ void __launch_bounds__(kLnThreads) layer_norm_residual_kernel(const L
     if (live[u])
 #pragma unroll
       for (int c = 0; c < V; ++c) sq = fmaf(v[u][c] - mean, v[u][c] - mean, sq);
-  for (int o = team >> 1; o > 0; o >>= 1) sq += __shfl_xor(sq, o, kWave);
+  sq = cluster_sum(sq, team);
   const float rstd = rsqrtf(sq / (float)p.C + p.eps);
 
 #pragma unroll
@@ -170,7 +170,7 @@ __global__ void __launch_bounds__(kLnThreads) layer_norm_residual_backward_kerne
       for (int c = 0; c < V; ++c) sum += v[u][c];
     }
     request(row0 + teams_per_block);
-    for (int o = team >> 1; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
+    sum = cluster_sum(sum, team);
     const float mean = sum * inv_c;
     float sq = 0.f;
 #pragma unroll
@@ -178,7 +178,7 @@ __global__ void __launch_bounds__(kLnThreads) layer_norm_residual_backward_kerne
       if (col_live[u])
 #pragma unroll
         for (int c = 0; c < V; ++c) sq = fmaf(v[u][c] - mean, v[u][c] - mean, sq);
-    for (int o = team >> 1; o > 0; o >>= 1) sq += __shfl_xor(sq, o, kWave);
+    sq = cluster_sum(sq, team);
     const float rstd = rsqrtf(sq * inv_c + p.eps);
 
     float s1 = 0.f, s2 = 0.f;
@@ -198,10 +198,8 @@ __global__ void __launch_bounds__(kLnThreads) layer_norm_residual_backward_kerne
         g[u][c] = a;
       }
     }
-    for (int o = team >> 1; o > 0; o >>= 1) {
-      s1 += __shfl_xor(s1, o, kWave);
-      s2 += __shfl_xor(s2, o, kWave);
-    }
+    s1 = cluster_sum(s1, team);
+    s2 = cluster_sum(s2, team);
     const float m1 = s1 * inv_c, m2 = s2 * inv_c;
     if (row_live) {
       raw_t *gy = reinterpret_cast<raw_t *>(p.grad_y) + row * nvec;
