@@ -316,7 +316,16 @@ def main():
                     tail_bytes(2, B, H, W, C)[0])
                 add("block_tail_bwd", name, torch.float16, time_op(lambda: ext.layer_norm_residual_backward(go, y, w, b, gamma, 1e-6), args.op_iters),
                     tail_bytes(2, B, H, W, C)[1])
-                del y, x, w, b, gamma, go
+                del w, b, gamma
+                # the centre-feature blend of a DCNv4 layer (off in the FlashInternImage configs): y, x in, out; backward
+                # grad_out, y, x in, two gradients out
+                G7 = G
+                w = (torch.randn(G7, C, device=dev) / C ** 0.5).to(torch.float16)
+                b = torch.randn(G7, device=dev).to(torch.float16)
+                t_bytes = B * H * W * C * 2
+                add("center_blend_fwd", name, torch.float16, time_op(lambda: ext.center_feature_blend_forward(y, x, w, b), args.op_iters), 3 * t_bytes)
+                add("center_blend_bwd", name, torch.float16, time_op(lambda: ext.center_feature_blend_backward(go, y, x, w, b), args.op_iters), 5 * t_bytes)
+                del y, x, w, b, go
         for dtype, s in ((torch.float16, 2), (torch.float32, 4)):
             (B, N, G, D, L, K), shapes, starts, v, sla, go = fda_inputs(dtype)
             fb, bb = fda_bytes(s, B, N, N, G, D, L, K)

@@ -81,6 +81,11 @@ __global__ void __launch_bounds__(kCfThreads) center_feature_blend_kernel(const 
     }
     z = cluster_sum(z, team);
     if constexpr (BWD) dgate = cluster_sum(dgate, team);
+    if constexpr (!BWD) {        // forward: a lane keeps the logit of its own group(s) and takes one sigmoid at the end
+#pragma unroll
+      for (int u = 0; u < VPL; ++u) gate[u] = grp[u] == g ? z : gate[u];
+      continue;
+    }
     float bias_g[1];
     Pack<Tag, 1>::decode(reinterpret_cast<const typename RawWord<Tag::kBytes>::type *>(p.bias)[g], bias_g);
     const float s = sigmoid(z + bias_g[0]);
@@ -96,6 +101,14 @@ __global__ void __launch_bounds__(kCfThreads) center_feature_blend_kernel(const 
     }
   }
 
+  if constexpr (!BWD) {
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      float bias_g[1];
+      Pack<Tag, 1>::decode(reinterpret_cast<const typename RawWord<Tag::kBytes>::type *>(p.bias)[min(grp[u], p.G - 1)], bias_g);
+      gate[u] = sigmoid(gate[u] + bias_g[0]);
+    }
+  }
 #pragma unroll
   for (int u = 0; u < VPL; ++u) {
     if (!live[u]) continue;
