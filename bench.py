@@ -132,7 +132,10 @@ def main():
         t = B * H * W * C * s
         return 3 * t, 3 * t
 
-    def time_op(fn, iters, warm=20):
+    def time_op(fn, iters, warm=None):
+        # per-operator timings warm up for as many launches as they time: some kernels (the attention forward with
+        # levels staged in LDS) settle only after ~120 launches, while the device's power management follows them
+        warm = iters if warm is None else warm
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
