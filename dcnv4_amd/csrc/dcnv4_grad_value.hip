@@ -228,6 +228,8 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
           ti = tt / p.kh; tj = tt - ti * p.kh;
         }
         const int ho = ho_lo + s + r * n_strips, wo = wo_lo + col;
+        const elem_t *om = om_img + ((uint32_t)(ho * p.Wo + wo) * (uint32_t)p.P_pad + (uint32_t)((g0 + gl) * 3 * Kp));
+        const elem_t m_raw = om[2 * Kp + t];      // requested before the position is formed: its latency hides behind that arithmetic
         const float off_x = to_f(pf_x[v]), off_y = to_f(pf_y[v]);
         const float x_base = sub_rn((float)(cx0 + wo * p.sw), x_sub), y_base = sub_rn((float)(cy0 + ho * p.sh), y_sub);
         const float x = add_rn(x_base, mul_rn(add_rn((float)(ti * p.dw), off_x), p.offset_scale));
@@ -238,8 +240,7 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
         // anchor relative to the anchor grid, whose first row and column lie one cell outside the tile
         const int ay = (int)fy - ty0 + 1, ax = (int)fx - tx0 + 1;
         if ((unsigned)ay > (unsigned)th || (unsigned)ax > (unsigned)tw) continue;
-        const elem_t *om = om_img + ((uint32_t)(ho * p.Wo + wo) * (uint32_t)p.P_pad + (uint32_t)((g0 + gl) * 3 * Kp));
-        float m = load_f(om + 2 * Kp + t);
+        float m = to_f(m_raw);
         if (p.softmax) {          // rare: normalise over this group's taps
           float mx = load_f(om + 2 * Kp), sum = 0.f;
           for (int k = 1; k < Kp; ++k) mx = fmaxf(mx, load_f(om + 2 * Kp + k));
