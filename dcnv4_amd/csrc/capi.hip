@@ -457,13 +457,14 @@ void fda_choose_order(FdaLaunch *F, const FdaProblem &pr, int N, int G, int D, i
   F->nq_block = std::max(1, std::min(kBlockThreads / width, (int)(kMaxDynamicLds / lds_per_row)));
   // Forward: the smallest levels of the head's value slice in LDS.  The level shapes live in device memory, so the
   // choice goes by what a pyramid with a factor of two between levels would need: its last two levels hold about
-  // 6 % of the pixels.  The kernel stages whatever really fits; with nothing staged it only runs at lower occupancy.
+  // 5.9 % of the pixels (6.5 % asked for).  The kernel stages whatever really fits; with nothing staged it only runs
+  // at lower occupancy.
   F->stage_budget = 0;
   if (backward || g_opt.fda_stage == kOptPlain || (head_bytes % 16) != 0 || width > 64) return;
   const size_t rows_bytes = (size_t)(kFdaStagedThreads / width) * lds_per_row;
   if (rows_bytes + 4096 > kMaxLdsPerWorkgroup - 2048) return;
   const size_t budget = std::min<size_t>(kMaxLdsPerWorkgroup - 2048 - rows_bytes, 112 * 1024);
-  const bool pyramid_fits = L >= 3 && (size_t)N * head_bytes * 8 / 100 + 64 <= budget;
+  const bool pyramid_fits = L >= 3 && (size_t)N * head_bytes * 13 / 200 + fda_staged_zero_bytes((int)head_bytes) <= budget;
   // The workgroups of a launch - one per CU, 1024 lanes and most of the LDS each - should pass over the chip in two
   // even rounds: measured on 128x128.. and 100x151.. pyramids (4 images, 8 heads of 32 fp16 channels), two rounds
   // take 0.158 / 0.135 ms against 0.180 / 0.165 ms without staging, while counts that leave a partial last round
@@ -476,8 +477,6 @@ void fda_choose_order(FdaLaunch *F, const FdaProblem &pr, int N, int G, int D, i
   if (g_opt.fda_stage != kOptTiled && !(pyramid_fits && pays)) return;
   F->stage_budget = (int)(budget & ~size_t(15));
   F->stage_blocks = std::max(1, std::min(blocks, (F->Q + sub_q - 1) / sub_q));
-  F->stage_nq = ((F->Q + F->stage_blocks - 1) / F->stage_blocks + sub_q - 1) / sub_q * sub_q;
-  F->stage_blocks = (F->Q + F->stage_nq - 1) / F->stage_nq;
 }
 
 int images_per_launch(const FdaProblem &pr, bool backward) {

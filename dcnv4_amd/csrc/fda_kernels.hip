@@ -14,6 +14,8 @@
 #include "common.hpp"
 #include "launch.hpp"
 
+#include <utility>
+
 namespace dcn {
 namespace {
 
@@ -114,8 +116,89 @@ __device__ __forceinline__ void fda_unstage_grads(const float *lds, const FdaLau
   }
 }
 
+// ------------------------------------------------------------------------------- forward, shared set-up inside a quad
+// When four or more lanes share a (query, head) - aligned quads of the wave - and K is a multiple of four, the lanes of
+// a quad split the per-point work that does not depend on the channel: lane j of the quad takes every fourth logit for
+// the softmax statistics and prepares sampling point k0 + j of each group of four (position, probability, the four
+// corner weights times the probability, the four corner offsets); the other three read what it prepared with DPP
+// quad broadcasts and add their own channel offset.  Per point and lane that leaves the gathers and the multiply-adds.
+template <int J> __device__ __forceinline__ int quad_pick(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, J * 0x55, 0xf, 0xf, true);
+}
+template <int... Js, typename F>
+__device__ __forceinline__ void static_for(std::integer_sequence<int, Js...>, F &&f) {
+  (f(std::integral_constant<int, Js>{}), ...);
+}
+
+__device__ __forceinline__ void quad_softmax_stats(const float *m, int n, int my_k, float &mx, float &inv) {
+  mx = m[my_k];
+  for (int k = my_k + 4; k < n; k += 4) mx = fmaxf(mx, m[k]);
+  mx = fmaxf(mx, dpp_quad_xor1(mx));
+  mx = fmaxf(mx, dpp_quad_xor2(mx));
+  float sum = 0.f;
+  for (int k = my_k; k < n; k += 4) sum += __expf(m[k] - mx);
+  sum += dpp_quad_xor1(sum);
+  sum += dpp_quad_xor2(sum);
+  inv = 1.f / sum;
+}
+
+// The K points of level l for one lane.  base: byte offset of the level's pixel 0 for this (image, head), without
+// the lane's channels; staged: the level lies in LDS at s_stage + base, with one head's width of zero bytes at s_stage
+// for corners outside the level (a lane's channel offset stays inside them).
+template <typename Tag, int CPT>
+__device__ __forceinline__ void fda_quad_level(float (&acc)[CPT], const float *s, int LK, int K, int l, const Level &lv,
+                                               float mx, float inv, uint32_t base, uint32_t step, uint32_t lane_off,
+                                               int my_k, bool staged, const char *s_stage,
+                                               const __amdgpu_buffer_rsrc_t &value) {
+  typedef Pack<Tag, CPT> pack;
+  typedef typename pack::raw_t raw_t;
+  for (int k0 = 0; k0 < K; k0 += 4) {
+    const int t = l * K + k0 + my_k;
+    const float x = sub_rn(mul_rn(s[2 * t], (float)lv.W), 0.5f);       // flash_deform_im2col_cuda.cuh:188-189
+    const float y = sub_rn(mul_rn(s[2 * t + 1], (float)lv.H), 0.5f);
+    const float pr = __expf(s[2 * LK + t] - mx) * inv;
+    const Tap tp = make_tap(y, x, lv.H, lv.W, base, step);
+    int wq[4], oq[4];
+#pragma unroll
+    for (int cn = 0; cn < 4; ++cn) {
+      wq[cn] = __builtin_bit_cast(int, pr * tp.w[cn]);
+      oq[cn] = (int)((staged && !((tp.valid >> cn) & 1u)) ? 0u : tp.off[cn]);
+    }
+    raw_t raw[4][4];
+    float w[4][4];
+    if (staged) {
+      static_for(std::make_integer_sequence<int, 4>{}, [&](auto j) {
+        constexpr int J = decltype(j)::value;
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn) {
+          w[J][cn] = __builtin_bit_cast(float, quad_pick<J>(wq[cn]));
+          raw[J][cn] = *reinterpret_cast<const raw_t *>(s_stage + ((uint32_t)quad_pick<J>(oq[cn]) + lane_off));
+        }
+      });
+    } else {
+      static_for(std::make_integer_sequence<int, 4>{}, [&](auto j) {
+        constexpr int J = decltype(j)::value;
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn) {
+          w[J][cn] = __builtin_bit_cast(float, quad_pick<J>(wq[cn]));
+          raw[J][cn] = buffer_load<pack::kBytes>(value, (uint32_t)quad_pick<J>(oq[cn]) + lane_off);
+        }
+      });
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int cn = 0; cn < 4; ++cn) {
+        float v[CPT];
+        pack::decode(raw[j][cn], v);
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) acc[c] = fmaf(w[j][cn], v[c], acc[c]);
+      }
+  }
+}
+
 // ------------------------------------------------------------------------------- forward
-template <typename Tag, int CPT, int KT>
+template <typename Tag, int CPT, int KT, bool QUAD>
 __global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLaunch p) {
   extern __shared__ float lds[];
   typedef Pack<Tag, CPT> pack;
@@ -154,14 +237,22 @@ __global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLau
     const int lr = rg / heads_here, g = g_fixed + rg - lr * heads_here;
     const int b = (row0 + lr) / p.Q;
     const float *s = lds + rg * row_len;
-    float mx, inv;
-    softmax_stats(s + 2 * LK, LK, mx, inv);
-    const uint32_t lane_base = (uint32_t)(g * p.D + chunk * CPT) * Tag::kBytes;
-
     float acc[CPT];
 #pragma unroll
     for (int c = 0; c < CPT; ++c) acc[c] = 0.f;
-
+    float mx, inv;
+    if constexpr (QUAD) {
+      const int my_k = chunk & 3;
+      quad_softmax_stats(s + 2 * LK, LK, my_k, mx, inv);
+      const uint32_t lane_off = (uint32_t)(chunk * CPT) * Tag::kBytes;
+      for (int l = 0; l < p.L; ++l) {
+        const Level lv = load_level(p, l);
+        const uint32_t base = (uint32_t)(b * p.N + lv.start) * pix_bytes + (uint32_t)(g * p.D) * Tag::kBytes;
+        fda_quad_level<Tag, CPT>(acc, s, LK, K, l, lv, mx, inv, base, pix_bytes, lane_off, my_k, false, nullptr, value);
+      }
+    } else {
+    softmax_stats(s + 2 * LK, LK, mx, inv);
+    const uint32_t lane_base = (uint32_t)(g * p.D + chunk * CPT) * Tag::kBytes;
     for (int l = 0; l < p.L; ++l) {
       const Level lv = load_level(p, l);
       const uint32_t base = (uint32_t)(b * p.N + lv.start) * pix_bytes + lane_base;
@@ -185,6 +276,7 @@ __global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLau
         }
       }
     }
+    }
     char *dst = (char *)p.out + ((size_t)(row0 + lr) * (p.G * p.D) + g * p.D + chunk * CPT) * Tag::kBytes;
     *reinterpret_cast<typename pack::raw_t *>(dst) = pack::encode(acc);
   }
@@ -198,7 +290,7 @@ __global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLau
 // own 64 lanes' queries (no workgroup barriers); sampling points on a staged level are served from LDS, the others from
 // memory as in fda_forward_kernel.  Same arithmetic in the same order per
 // (query, head): identical results.  Which levels fit is decided on the device from spatial_shapes.
-template <typename Tag, int CPT, int KT>
+template <typename Tag, int CPT, int KT, bool QUAD>
 __global__ void __launch_bounds__(kFdaStagedThreads) fda_forward_staged_kernel(const FdaLaunch p) {
   extern __shared__ float lds[];
   __shared__ int s_level_off[kMaxLevels];       // byte offset of a staged level in the stage area, -1: not staged
@@ -209,13 +301,18 @@ __global__ void __launch_bounds__(kFdaStagedThreads) fda_forward_staged_kernel(c
   const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
   const int rb = (int)(blk % (uint32_t)p.stage_blocks), bg = (int)(blk / (uint32_t)p.stage_blocks);
   const int b = bg / p.G, g = bg - b * p.G;
-  const int q_begin = rb * p.stage_nq, q_end = min(p.Q, q_begin + p.stage_nq);
+  // The queries of an (image, head) in passes of sub_q; its workgroups take whole passes, the first ones one more
+  // than the others when the passes do not divide evenly.
+  const int passes = (p.Q + sub_q - 1) / sub_q, base_passes = passes / p.stage_blocks, extra = passes - base_passes * p.stage_blocks;
+  const int q_begin = (rb * base_passes + min(rb, extra)) * sub_q;
+  const int q_end = min(p.Q, q_begin + (base_passes + (rb < extra ? 1 : 0)) * sub_q);
   const uint32_t head_bytes = (uint32_t)p.D * Tag::kBytes, pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
-  char *s_stage = reinterpret_cast<char *>(lds + (size_t)sub_q * row_len);      // 64 zero bytes, then the staged levels
+  char *s_stage = reinterpret_cast<char *>(lds + (size_t)sub_q * row_len);      // zero bytes, then the staged levels
+  const int zero_bytes = fda_staged_zero_bytes((int)head_bytes);
   const __amdgpu_buffer_rsrc_t value = make_rsrc(p.value, p.value_bytes);
 
   if (threadIdx.x == 0) {
-    int used = 64;
+    int used = zero_bytes;
     bool open = true;
     for (int l = p.L - 1; l >= 0; --l) {
       const Level lv = load_level(p, l);
@@ -225,7 +322,7 @@ __global__ void __launch_bounds__(kFdaStagedThreads) fda_forward_staged_kernel(c
       if (open) used += (int)bytes;
     }
   }
-  if (threadIdx.x < 4) reinterpret_cast<u32x4 *>(s_stage)[threadIdx.x] = u32x4{0u, 0u, 0u, 0u};
+  if ((int)threadIdx.x < zero_bytes / 16) reinterpret_cast<u32x4 *>(s_stage)[threadIdx.x] = u32x4{0u, 0u, 0u, 0u};
   __syncthreads();
   for (int l = 0; l < p.L; ++l) {
     const int off = s_level_off[l];
@@ -289,10 +386,22 @@ __global__ void __launch_bounds__(kFdaStagedThreads) fda_forward_staged_kernel(c
     if (lr >= nrow || chunk >= p.lanes.tpg) continue;
     const float *s = rows + lr * row_len;
     float mx, inv;
-    softmax_stats(s + 2 * LK, LK, mx, inv);
     float acc[CPT];
 #pragma unroll
     for (int c = 0; c < CPT; ++c) acc[c] = 0.f;
+    if constexpr (QUAD) {
+      const int my_k = chunk & 3;
+      quad_softmax_stats(s + 2 * LK, LK, my_k, mx, inv);
+      for (int l = 0; l < p.L; ++l) {
+        const Level lv = load_level(p, l);
+        const int off = s_level_off[l];
+        const bool staged = off >= 0;
+        const uint32_t base = staged ? (uint32_t)off : (uint32_t)(b * p.N + lv.start) * pix_bytes + (uint32_t)g * head_bytes;
+        fda_quad_level<Tag, CPT>(acc, s, LK, K, l, lv, mx, inv, base, staged ? head_bytes : pix_bytes, lane_off, my_k, staged,
+                                 s_stage, value);
+      }
+    } else {
+    softmax_stats(s + 2 * LK, LK, mx, inv);
     for (int l = 0; l < p.L; ++l) {
       const Level lv = load_level(p, l);
       const int off = s_level_off[l];
@@ -325,6 +434,7 @@ __global__ void __launch_bounds__(kFdaStagedThreads) fda_forward_staged_kernel(c
           for (int c = 0; c < CPT; ++c) acc[c] = fmaf(w, v[c], acc[c]);
         }
       }
+    }
     }
     char *dst = (char *)p.out + ((size_t)(row0 + lr) * (p.G * p.D) + g * p.D + chunk * CPT) * Tag::kBytes;
     *reinterpret_cast<typename pack::raw_t *>(dst) = pack::encode(acc);
@@ -502,6 +612,11 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
   fda_unstage_grads<Tag>(s_grad, p, row0, nrow, g_fixed, heads_here);
 }
 
+// Lanes of a (query, head) fill whole quads and the points come in fours: the forward kernels share the set-up.
+bool fda_quad_setup(const FdaLaunch &p) {
+  return (p.K % 4) == 0 && p.lanes.tpg >= 4 && p.lanes.tpg == (1 << p.lanes.tpgp_log2);
+}
+
 template <typename Tag, int CPT>
 hipError_t launch_staged(const FdaLaunch &p, hipStream_t stream) {
   const dim3 grid((unsigned)((p.n_row / p.Q) * p.G * p.stage_blocks)), block(kFdaStagedThreads);
@@ -511,8 +626,9 @@ hipError_t launch_staged(const FdaLaunch &p, hipStream_t stream) {
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
     return hipGetLastError();
   };
-  if (p.K == 4) return go(fda_forward_staged_kernel<Tag, CPT, 4>);
-  return go(fda_forward_staged_kernel<Tag, CPT, 0>);      // (unrolled for 8 points the kernel spills a hundred registers)
+  if (fda_quad_setup(p)) return go(fda_forward_staged_kernel<Tag, CPT, 0, true>);
+  if (p.K == 4) return go(fda_forward_staged_kernel<Tag, CPT, 4, false>);
+  return go(fda_forward_staged_kernel<Tag, CPT, 0, false>);      // (unrolled for 8 points the kernel spills a hundred registers)
 }
 
 template <typename Tag, int CPT, int MODE>      // MODE -1: forward
@@ -523,8 +639,14 @@ hipError_t launch_k(const FdaLaunch &p, hipStream_t stream, dim3 grid, dim3 bloc
 #define FDA_LAUNCH(KT)                                                                                     \
   do {                                                                                                     \
     if constexpr (MODE >= 0) hipLaunchKernelGGL((fda_backward_kernel<Tag, CPT, KT, MODE>), grid, block, lds, stream, p); \
-    else hipLaunchKernelGGL((fda_forward_kernel<Tag, CPT, KT>), grid, block, lds, stream, p);              \
+    else hipLaunchKernelGGL((fda_forward_kernel<Tag, CPT, KT, false>), grid, block, lds, stream, p);       \
   } while (0)
+  if constexpr (MODE < 0) {
+    if (fda_quad_setup(p)) {
+      hipLaunchKernelGGL((fda_forward_kernel<Tag, CPT, 0, true>), grid, block, lds, stream, p);
+      return hipGetLastError();
+    }
+  }
   if (p.K == 4) FDA_LAUNCH(4);
   else if (p.K == 8) FDA_LAUNCH(8);
   else FDA_LAUNCH(0);

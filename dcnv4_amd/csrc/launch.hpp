@@ -120,8 +120,8 @@ struct FdaLaunch {
   int head_major;           // forward: a workgroup takes nq_block queries of ONE head, workgroups ordered [image][head][block]
   // forward with the smallest levels of one head's value slice staged in LDS (stage_budget > 0; implies head_major)
   int stage_budget;         // bytes of LDS for staged levels, behind the rows; the kernel stages the last levels that fit
-  int stage_nq;             // queries one workgroup walks (in passes of as many queries as its lanes hold)
-  int stage_blocks;         // workgroups per (image, head)
+  int stage_blocks;         // workgroups per (image, head); each walks its share of the queries in passes of as many
+                            // queries as its lanes hold
   LaneMap lanes;
   // tiled grad_value path
   void *grad_value;         // [n_img, N, G, D] in the tensor dtype
@@ -231,5 +231,8 @@ size_t dcnv4_forward_lds_bytes(const DcnLaunch &p);
 size_t dcnv4_backward_lds_bytes(const DcnLaunch &p);
 size_t fda_forward_lds_bytes(const FdaLaunch &p);
 size_t fda_backward_lds_bytes(const FdaLaunch &p);
+// Zero bytes at the start of the staged forward's level area, read by corners that fall outside their level: one
+// head's width, so that any lane's channel offset stays inside them.
+__host__ __device__ inline int fda_staged_zero_bytes(int head_bytes) { return head_bytes < 64 ? 64 : (head_bytes + 15) & ~15; }
 
 }  // namespace dcn
