@@ -52,6 +52,19 @@ __device__ __forceinline__ void fda_stage_rows(float *lds, const FdaLaunch &p, i
     if (heads_here == p.G) {
       const bool vec16 = ((size_t)p.G * row_len * Tag::kBytes) % 16 == 0;
       stage_rows_to_lds<Tag>(lds, (const char *)p.sla + (size_t)row0 * p.G * row_len * Tag::kBytes, pairs * row_len, vec16);
+    } else if (constexpr int EPV = 16 / Tag::kBytes; row_len % EPV == 0) {      // rows of some heads: 16-byte pieces of a row
+      const int vpr = row_len / EPV;
+      const float inv_vpr = 1.f / (float)vpr;
+      const u32x4 *src = reinterpret_cast<const u32x4 *>(p.sla);
+      for (int i = threadIdx.x; i < pairs * vpr; i += blockDim.x) {
+        const int j = fdiv20(i, inv_vpr), v = i - j * vpr;
+        const int r = fdiv20(j, inv_h), gh = j - r * heads_here;
+        float f[EPV];
+        Pack<Tag, EPV>::decode(src[((size_t)(row0 + r) * p.G + g0 + gh) * vpr + v], f);
+#pragma unroll
+        for (int e = 0; e < EPV; e += 4)
+          *reinterpret_cast<f32x4 *>(lds + i * EPV + e) = f32x4{f[e], f[e + 1], f[e + 2], f[e + 3]};
+      }
     } else {
       const float inv_len = 1.f / (float)row_len;
       for (int i = threadIdx.x; i < pairs * row_len; i += blockDim.x) {
@@ -88,6 +101,21 @@ __device__ __forceinline__ void fda_unstage_grads(const float *lds, const FdaLau
     if (heads_here == p.G) {
       const bool vec16 = ((size_t)p.G * row_len * Tag::kBytes) % 16 == 0;
       unstage_rows_from_lds<Tag>((char *)p.grad_sla + (size_t)row0 * p.G * row_len * Tag::kBytes, lds, pairs * row_len, vec16);
+    } else if (constexpr int EPV = 16 / Tag::kBytes; row_len % EPV == 0) {
+      const int vpr = row_len / EPV;
+      const float inv_vpr = 1.f / (float)vpr;
+      u32x4 *dst = reinterpret_cast<u32x4 *>(p.grad_sla);
+      for (int i = threadIdx.x; i < pairs * vpr; i += blockDim.x) {
+        const int j = fdiv20(i, inv_vpr), v = i - j * vpr;
+        const int r = fdiv20(j, inv_h), gh = j - r * heads_here;
+        float f[EPV];
+#pragma unroll
+        for (int e = 0; e < EPV; e += 4) {
+          const f32x4 q = *reinterpret_cast<const f32x4 *>(lds + i * EPV + e);
+          f[e] = q.x; f[e + 1] = q.y; f[e + 2] = q.z; f[e + 3] = q.w;
+        }
+        dst[((size_t)(row0 + r) * p.G + g0 + gh) * vpr + v] = Pack<Tag, EPV>::encode(f);
+      }
     } else {
       const float inv_len = 1.f / (float)row_len;
       for (int i = threadIdx.x; i < pairs * row_len; i += blockDim.x) {
@@ -195,6 +223,81 @@ __device__ __forceinline__ void fda_quad_level(float (&acc)[CPT], const float *s
         for (int c = 0; c < CPT; ++c) acc[c] = fmaf(w[j][cn], v[c], acc[c]);
       }
   }
+}
+
+// Backward counterpart: the lanes of a quad gather the corners of four points prepared one by each of them, form their
+// channels' share of the sixteen corner dot products, and add them up across the quad so that each sum ends in the
+// lane that prepared its point (a transpose-reduce: after the exchange with the lane one away a lane holds the points
+// of its own parity, after the exchange with the lane two away its own point).  That lane applies the bilinear
+// derivatives and writes the point's three gradient slots, and its key and record (keys, recs: those of the query's
+// first point of this level).  Returns the lane's sum of probability x d(out)/d(prob).
+template <typename Tag, int CPT>
+__device__ __forceinline__ float fda_quad_level_backward(const float (&go)[CPT], const float *s, float *gs, int LK, int K, int l,
+                                                        const Level &lv, float mx, float inv, uint32_t base, uint32_t step,
+                                                        uint32_t lane_off, int my_k, int width, bool writer,
+                                                        const __amdgpu_buffer_rsrc_t &value, uint16_t *keys, f32x4_t *recs) {
+  typedef Pack<Tag, CPT> pack;
+  typedef typename pack::raw_t raw_t;
+  const bool odd = (my_k & 1) != 0, high = (my_k & 2) != 0;
+  float dot_mine = 0.f;
+  for (int k0 = 0; k0 < K; k0 += 4) {
+    const int t = l * K + k0 + my_k;
+    const float x = sub_rn(mul_rn(s[2 * t], (float)lv.W), 0.5f);
+    const float y = sub_rn(mul_rn(s[2 * t + 1], (float)lv.H), 0.5f);
+    const float pr = __expf(s[2 * LK + t] - mx) * inv;
+    const Tap tp = make_tap(y, x, lv.H, lv.W, base, step);
+    raw_t raw[4][4];
+    static_for(std::make_integer_sequence<int, 4>{}, [&](auto j) {
+      constexpr int J = decltype(j)::value;
+#pragma unroll
+      for (int cn = 0; cn < 4; ++cn)
+        raw[J][cn] = buffer_load<pack::kBytes>(value, (uint32_t)quad_pick<J>((int)tp.off[cn]) + lane_off);
+    });
+    float d[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int cn = 0; cn < 4; ++cn) {
+        float v[CPT];
+        pack::decode(raw[j][cn], v);
+        float a = 0.f;
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) a = fmaf(v[c], go[c], a);
+        d[j][cn] = a;
+      }
+    float r[4];
+#pragma unroll
+    for (int cn = 0; cn < 4; ++cn) {
+      float pair[2];
+#pragma unroll
+      for (int jh = 0; jh < 2; ++jh) {
+        const float give = odd ? d[2 * jh][cn] : d[2 * jh + 1][cn], keep = odd ? d[2 * jh + 1][cn] : d[2 * jh][cn];
+        pair[jh] = keep + dpp_quad_xor1(give);
+      }
+      const float give = high ? pair[0] : pair[1], keep = high ? pair[1] : pair[0];
+      r[cn] = keep + dpp_quad_xor2(give);
+      for (int o = 4; o < width; o <<= 1) r[cn] += __shfl_xor(r[cn], o, kWave);      // the other quads' channels
+    }
+    const float hy = 1.f - tp.ly, hx = 1.f - tp.lx;
+    const float gx = hy * (r[1] - r[0]) + tp.ly * (r[3] - r[2]);
+    const float gy = hx * (r[2] - r[0]) + tp.lx * (r[3] - r[1]);
+    const float gz = tp.w[0] * r[0] + tp.w[1] * r[1] + tp.w[2] * r[2] + tp.w[3] * r[3];
+    if (writer) {
+      gs[2 * t] = gx * (float)lv.W * pr;          // flash_deform_col2im_cuda.cuh:273-276
+      gs[2 * t + 1] = gy * (float)lv.H * pr;
+      gs[2 * LK + t] = gz;
+      // key and record of the point for the tiled grad_value kernel: the writers of a wave hold consecutive points
+      // of consecutive queries, whole 16-byte records side by side
+      uint32_t key = kFdaKeyOutside;
+      if (tp.valid != 0)
+        key = (tp.y0 + 1 >= kFdaKeyFieldMax || tp.x0 + 1 >= kFdaKeyFieldMax) ? kFdaKeySaturated
+                                                                            : ((uint32_t)(tp.y0 + 1) << 8) | (uint32_t)(tp.x0 + 1);
+      keys[k0 + my_k] = (uint16_t)key;
+      recs[k0 + my_k] = f32x4_t{x, y, pr, 0.f};
+    }
+    dot_mine = fmaf(pr, gz, dot_mine);
+  }
+  return dot_mine;
 }
 
 // ------------------------------------------------------------------------------- forward
@@ -449,7 +552,7 @@ __global__ void __launch_bounds__(kFdaStagedThreads) fda_forward_staged_kernel(c
 //                  and a (position, softmax probability) record, and grad_out regrouped by head
 //   kFdaFallback   exits at once unless the binning kernel flagged a level it cannot hold; then it scatters
 //                  with fp32 atomics into an fp32 image (grad_value itself for fp32 tensors, left zeroed by the tiled kernel)
-template <typename Tag, int CPT, int KT, int MODE>
+template <typename Tag, int CPT, int KT, int MODE, bool QUAD>      // QUAD: only with kFdaNoScatter
 __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLaunch p) {
   extern __shared__ float lds[];
   typedef Pack<Tag, CPT> pack;
@@ -482,6 +585,7 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
   const int items = (nrow * heads_here) << tpgp_log2;
   const uint32_t pix_bytes = (uint32_t)(p.G * p.D) * Tag::kBytes;
   const int K = KT > 0 ? KT : p.K;
+  const size_t key_stride = fda_key_stride(p.Q, K);
 
   for (int it = threadIdx.x; it < items; it += blockDim.x) {
     const int chunk = it & (width - 1);
@@ -492,7 +596,8 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
     const float *s = s_in + rg * row_len;
     float *gs = s_grad + rg * row_len;
     float mx, inv;
-    softmax_stats(s + 2 * LK, LK, mx, inv);
+    if constexpr (QUAD) quad_softmax_stats(s + 2 * LK, LK, chunk & 3, mx, inv);
+    else softmax_stats(s + 2 * LK, LK, mx, inv);
     const uint32_t lane_base = (uint32_t)(g * p.D + (active ? chunk : 0) * CPT) * Tag::kBytes;
 
     float go[CPT];
@@ -513,6 +618,26 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
       }
     }
 
+    if constexpr (QUAD) {      // every lane of the cluster is active; the first quad writes the gradient slots
+      const int my_k = chunk & 3;
+      const uint32_t lane_off = (uint32_t)(chunk * CPT) * Tag::kBytes;
+      for (int l = 0; l < p.L; ++l) {
+        const Level lv = load_level(p, l);
+        const uint32_t base = (uint32_t)(b * p.N + lv.start) * pix_bytes + (uint32_t)(g * p.D) * Tag::kBytes;
+        const size_t slot = (((size_t)b_local * p.G + g) * p.L + l) * key_stride + (size_t)q * K;
+        dot_rg += fda_quad_level_backward<Tag, CPT>(go, s, gs, LK, K, l, lv, mx, inv, base, pix_bytes, lane_off, my_k, width,
+                                                    chunk < 4, value, p.keys + slot, p.recs + slot);
+      }
+      dot_rg += dpp_quad_xor1(dot_rg);
+      dot_rg += dpp_quad_xor2(dot_rg);
+      if (chunk < 4) {
+        for (int t = my_k; t < LK; t += 4) {      // the lane's own points
+          const float pr = __expf(s[2 * LK + t] - mx) * inv;
+          gs[2 * LK + t] = pr * (gs[2 * LK + t] - dot_rg);
+        }
+      }
+      continue;
+    }
     for (int l = 0; l < p.L; ++l) {
       const Level lv = load_level(p, l);
       const uint32_t base = (uint32_t)(b * p.N + lv.start) * pix_bytes + lane_base;
@@ -585,10 +710,9 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
   }
   if constexpr (MODE == kFdaFallback) return;
   __syncthreads();
-  if constexpr (MODE == kFdaNoScatter) {
+  if constexpr (MODE == kFdaNoScatter && !QUAD) {
     // Keys and records of the workgroup's sampling points, one lane per point in the order they lie in memory
     // ([head][level][query][point]: whole 16-byte records side by side), from the staged rows.
-    const size_t stride = fda_key_stride(p.Q, K);
     for (int hl = 0; hl < heads_here * p.L; ++hl) {
       const int gh = hl / p.L, l = hl - gh * p.L, g = g_fixed + gh;
       const Level lv = load_level(p, l);
@@ -603,7 +727,7 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
           key = (tp.y0 + 1 >= kFdaKeyFieldMax || tp.x0 + 1 >= kFdaKeyFieldMax) ? kFdaKeySaturated
                                                                               : ((uint32_t)(tp.y0 + 1) << 8) | (uint32_t)(tp.x0 + 1);
         const int b_local = (row0 + lr) / p.Q, q = (row0 + lr) - b_local * p.Q;
-        const size_t slot = (((size_t)b_local * p.G + g) * p.L + l) * stride + (size_t)q * K + k;
+        const size_t slot = (((size_t)b_local * p.G + g) * p.L + l) * key_stride + (size_t)q * K + k;
         p.keys[slot] = (uint16_t)key;
         p.recs[slot] = f32x4_t{x, y, s[2 * LK + t], 0.f};
       }
@@ -612,7 +736,7 @@ __global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLa
   fda_unstage_grads<Tag>(s_grad, p, row0, nrow, g_fixed, heads_here);
 }
 
-// Lanes of a (query, head) fill whole quads and the points come in fours: the forward kernels share the set-up.
+// Lanes of a (query, head) fill whole quads and the points come in fours: the lanes of a quad share the set-up.
 bool fda_quad_setup(const FdaLaunch &p) {
   return (p.K % 4) == 0 && p.lanes.tpg >= 4 && p.lanes.tpg == (1 << p.lanes.tpgp_log2);
 }
@@ -638,12 +762,18 @@ hipError_t launch_k(const FdaLaunch &p, hipStream_t stream, dim3 grid, dim3 bloc
   }
 #define FDA_LAUNCH(KT)                                                                                     \
   do {                                                                                                     \
-    if constexpr (MODE >= 0) hipLaunchKernelGGL((fda_backward_kernel<Tag, CPT, KT, MODE>), grid, block, lds, stream, p); \
+    if constexpr (MODE >= 0) hipLaunchKernelGGL((fda_backward_kernel<Tag, CPT, KT, MODE, false>), grid, block, lds, stream, p); \
     else hipLaunchKernelGGL((fda_forward_kernel<Tag, CPT, KT, false>), grid, block, lds, stream, p);       \
   } while (0)
   if constexpr (MODE < 0) {
     if (fda_quad_setup(p)) {
       hipLaunchKernelGGL((fda_forward_kernel<Tag, CPT, 0, true>), grid, block, lds, stream, p);
+      return hipGetLastError();
+    }
+  }
+  if constexpr (MODE == kFdaNoScatter) {
+    if (fda_quad_setup(p)) {
+      hipLaunchKernelGGL((fda_backward_kernel<Tag, CPT, 0, MODE, true>), grid, block, lds, stream, p);
       return hipGetLastError();
     }
   }
