@@ -40,6 +40,7 @@ namespace {
 
 constexpr int kBinThreads = 1024;
 constexpr int kBinWordsPerLane = kFdaChunkPoints / 2 / kBinThreads;      // dwords of two keys per lane: 4
+constexpr int kBinSortedCap = 2 * kFdaChunkPoints;                       // list entries of a chunk put together in LDS
 constexpr int kBatch = 256;                  // listed points per batch: one per lane of the first four waves
 constexpr int kListCap = 1024;               // listed point ids held in LDS at a time
 constexpr int kTabCap = 256;                 // chunk table entries held in LDS at a time
@@ -84,6 +85,7 @@ template <typename Tag>
 __global__ void __launch_bounds__(kBinThreads) fda_bin_points_kernel(const FdaLaunch p) {
   __shared__ uint32_t s_hist[kFdaMaxTilesPerLevel];       // counts, then running cursors
   __shared__ uint32_t s_wave_sum[kBinThreads / kWave];
+  __shared__ __align__(16) uint16_t s_sorted[kBinSortedCap];      // the sorted list's first entries, as point numbers inside the chunk
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int QK = p.Q * p.K;
   const int chunk = blockIdx.x % p.n_chunks, seg = blockIdx.x / p.n_chunks;       // seg = (image * G + head) * L + level
@@ -172,20 +174,36 @@ __global__ void __launch_bounds__(kBinThreads) fda_bin_points_kernel(const FdaLa
   }
   __syncthreads();
 
-  // ---- pass 2: place
+  // ---- pass 2: place.  The list is put together in LDS and leaves in whole 16-byte pieces (scattered 4-byte stores
+  // cost the L2 a request each); entries beyond what the LDS array holds - a chunk whose points mostly straddle
+  // tiles - go to memory directly.
+  uint32_t total = 0;
+  for (int w = 0; w < kBinThreads / kWave; ++w) total += s_wave_sum[w];
   uint32_t *region = p.regions + (size_t)blockIdx.x * (4 * kFdaChunkPoints);
+  const uint32_t pt0 = (uint32_t)chunk * kFdaChunkPoints;
+  auto place = [&](uint32_t tile, uint32_t local) {
+    const uint32_t at = atomicAdd(&s_hist[tile], 1u);
+    if (at < (uint32_t)kBinSortedCap) s_sorted[at] = (uint16_t)local;
+    else region[at] = pt0 + local;
+  };
 #pragma unroll
   for (int u = 0; u < kBinWordsPerLane; ++u) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const Touch t = touch[2 * u + h];
       if (t.t00 == 0xffffffffu) continue;
-      const uint32_t pt = 2u * (uint32_t)(chunk * (kFdaChunkPoints / 2) + u * kBinThreads + tid) + h;
-      region[atomicAdd(&s_hist[t.t00], 1u)] = pt;
-      if (t.dx) region[atomicAdd(&s_hist[t.t00 + 1], 1u)] = pt;
-      if (t.dy) region[atomicAdd(&s_hist[t.t00 + lp.ntx], 1u)] = pt;
-      if (t.dx && t.dy) region[atomicAdd(&s_hist[t.t00 + lp.ntx + 1], 1u)] = pt;
+      const uint32_t local = 2u * (uint32_t)(u * kBinThreads + tid) + h;
+      place(t.t00, local);
+      if (t.dx) place(t.t00 + 1, local);
+      if (t.dy) place(t.t00 + lp.ntx, local);
+      if (t.dx && t.dy) place(t.t00 + lp.ntx + 1, local);
     }
+  }
+  __syncthreads();
+  const uint32_t n_lds = min(total, (uint32_t)kBinSortedCap);
+  for (uint32_t i = 4u * tid; i < n_lds; i += 4u * kBinThreads) {      // the last piece may run past the list, inside the region
+    const u32x2 w = *reinterpret_cast<const u32x2 *>(s_sorted + i);
+    *reinterpret_cast<u32x4 *>(region + i) = u32x4{pt0 + (w.x & 0xffffu), pt0 + (w.x >> 16), pt0 + (w.y & 0xffffu), pt0 + (w.y >> 16)};
   }
 }
 
