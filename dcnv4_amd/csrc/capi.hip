@@ -454,7 +454,7 @@ void fda_choose_order(FdaLaunch *F, const FdaProblem &pr, int N, int G, int D, i
   F->head_major = 1;
   const int width = 1 << F->lanes.tpgp_log2;
   const size_t lds_per_row = (size_t)3 * L * K * sizeof(float) * (backward ? 2 : 1);
-  F->nq_block = std::max(1, std::min(kBlockThreads / width, (int)(kMaxDynamicLds / lds_per_row)));
+  F->nq_block = std::max(1, std::min((backward ? kFdaBackwardThreads : kFdaForwardThreads) / width, (int)(kMaxDynamicLds / lds_per_row)));
   // Forward: the smallest levels of the head's value slice in LDS.  The level shapes live in device memory, so the
   // choice goes by what a pyramid with a factor of two between levels would need: its last two levels hold about
   // 5.9 % of the pixels (6.5 % asked for).  The kernel stages whatever really fits; with nothing staged it only runs

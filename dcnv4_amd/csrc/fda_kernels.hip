@@ -302,7 +302,7 @@ __device__ __forceinline__ float fda_quad_level_backward(const float (&go)[CPT],
 
 // ------------------------------------------------------------------------------- forward
 template <typename Tag, int CPT, int KT, bool QUAD>
-__global__ void __launch_bounds__(kBlockThreads) fda_forward_kernel(const FdaLaunch p) {
+__global__ void __launch_bounds__(kFdaForwardThreads) fda_forward_kernel(const FdaLaunch p) {
   extern __shared__ float lds[];
   typedef Pack<Tag, CPT> pack;
   const int LK = p.L * p.K, row_len = 3 * LK;
@@ -553,7 +553,7 @@ __global__ void __launch_bounds__(kFdaStagedThreads) fda_forward_staged_kernel(c
 //   kFdaFallback   exits at once unless the binning kernel flagged a level it cannot hold; then it scatters
 //                  with fp32 atomics into an fp32 image (grad_value itself for fp32 tensors, left zeroed by the tiled kernel)
 template <typename Tag, int CPT, int KT, int MODE, bool QUAD>      // QUAD: only with kFdaNoScatter
-__global__ void __launch_bounds__(kBlockThreads) fda_backward_kernel(const FdaLaunch p) {
+__global__ void __launch_bounds__(kFdaBackwardThreads) fda_backward_kernel(const FdaLaunch p) {
   extern __shared__ float lds[];
   typedef Pack<Tag, CPT> pack;
   if constexpr (MODE == kFdaFallback) {
@@ -789,7 +789,7 @@ hipError_t launch_by_cpt(const FdaLaunch &p, hipStream_t stream) {
   const bool head_major = p.head_major != 0;
   const dim3 grid(head_major ? (unsigned)((p.n_row / p.Q) * p.G * ((p.Q + p.nq_block - 1) / p.nq_block))
                              : (unsigned)((p.n_row + p.nq_block - 1) / p.nq_block)),
-      block(kBlockThreads);
+      block(MODE == kFdaNoScatter && head_major ? kFdaBackwardThreads : (MODE < 0 && head_major ? kFdaForwardThreads : kBlockThreads));
   const size_t lds = MODE >= 0 ? fda_backward_lds_bytes(p) : fda_forward_lds_bytes(p);
 #define FDA_CASE(N)                                                                       \
   case N:                                                                                 \
