@@ -354,31 +354,31 @@ __global__ void __launch_bounds__(kFdaForwardThreads) fda_forward_kernel(const F
         fda_quad_level<Tag, CPT>(acc, s, LK, K, l, lv, mx, inv, base, pix_bytes, lane_off, my_k, false, nullptr, value);
       }
     } else {
-    softmax_stats(s + 2 * LK, LK, mx, inv);
-    const uint32_t lane_base = (uint32_t)(g * p.D + chunk * CPT) * Tag::kBytes;
-    for (int l = 0; l < p.L; ++l) {
-      const Level lv = load_level(p, l);
-      const uint32_t base = (uint32_t)(b * p.N + lv.start) * pix_bytes + lane_base;
+      softmax_stats(s + 2 * LK, LK, mx, inv);
+      const uint32_t lane_base = (uint32_t)(g * p.D + chunk * CPT) * Tag::kBytes;
+      for (int l = 0; l < p.L; ++l) {
+        const Level lv = load_level(p, l);
+        const uint32_t base = (uint32_t)(b * p.N + lv.start) * pix_bytes + lane_base;
 #pragma unroll
-      for (int k = 0; k < K; ++k) {
-        const int t = l * K + k;
-        const float x = sub_rn(mul_rn(s[2 * t], (float)lv.W), 0.5f);       // flash_deform_im2col_cuda.cuh:188-189
-        const float y = sub_rn(mul_rn(s[2 * t + 1], (float)lv.H), 0.5f);
-        const float pr = __expf(s[2 * LK + t] - mx) * inv;
-        const Tap tp = make_tap(y, x, lv.H, lv.W, base, pix_bytes);
-        typename pack::raw_t raw[4];
+        for (int k = 0; k < K; ++k) {
+          const int t = l * K + k;
+          const float x = sub_rn(mul_rn(s[2 * t], (float)lv.W), 0.5f);       // flash_deform_im2col_cuda.cuh:188-189
+          const float y = sub_rn(mul_rn(s[2 * t + 1], (float)lv.H), 0.5f);
+          const float pr = __expf(s[2 * LK + t] - mx) * inv;
+          const Tap tp = make_tap(y, x, lv.H, lv.W, base, pix_bytes);
+          typename pack::raw_t raw[4];
 #pragma unroll
-        for (int cn = 0; cn < 4; ++cn) raw[cn] = buffer_load<pack::kBytes>(value, tp.off[cn]);
+          for (int cn = 0; cn < 4; ++cn) raw[cn] = buffer_load<pack::kBytes>(value, tp.off[cn]);
 #pragma unroll
-        for (int cn = 0; cn < 4; ++cn) {
-          float v[CPT];
-          pack::decode(raw[cn], v);
-          const float w = pr * tp.w[cn];
+          for (int cn = 0; cn < 4; ++cn) {
+            float v[CPT];
+            pack::decode(raw[cn], v);
+            const float w = pr * tp.w[cn];
 #pragma unroll
-          for (int c = 0; c < CPT; ++c) acc[c] = fmaf(w, v[c], acc[c]);
+            for (int c = 0; c < CPT; ++c) acc[c] = fmaf(w, v[c], acc[c]);
+          }
         }
       }
-    }
     }
     char *dst = (char *)p.out + ((size_t)(row0 + lr) * (p.G * p.D) + g * p.D + chunk * CPT) * Tag::kBytes;
     *reinterpret_cast<typename pack::raw_t *>(dst) = pack::encode(acc);
@@ -504,40 +504,41 @@ __global__ void __launch_bounds__(kFdaStagedThreads) fda_forward_staged_kernel(c
                                  s_stage, value);
       }
     } else {
-    softmax_stats(s + 2 * LK, LK, mx, inv);
-    for (int l = 0; l < p.L; ++l) {
-      const Level lv = load_level(p, l);
-      const int off = s_level_off[l];
-      const bool staged = off >= 0;
-      // staged: byte offsets into the stage area, a corner outside the level reads the zero bytes at its start
-      const uint32_t base = staged ? (uint32_t)off + lane_off : (uint32_t)(b * p.N + lv.start) * pix_bytes + (uint32_t)g * head_bytes + lane_off;
-      const uint32_t step = staged ? head_bytes : pix_bytes;
+      softmax_stats(s + 2 * LK, LK, mx, inv);
+      for (int l = 0; l < p.L; ++l) {
+        const Level lv = load_level(p, l);
+        const int off = s_level_off[l];
+        const bool staged = off >= 0;
+        // staged: byte offsets into the stage area, a corner outside the level reads the zero bytes at its start
+        const uint32_t base =
+            (staged ? (uint32_t)off : (uint32_t)(b * p.N + lv.start) * pix_bytes + (uint32_t)g * head_bytes) + lane_off;
+        const uint32_t step = staged ? head_bytes : pix_bytes;
 #pragma unroll
-      for (int k = 0; k < K; ++k) {
-        const int t = l * K + k;
-        const float x = sub_rn(mul_rn(s[2 * t], (float)lv.W), 0.5f);       // flash_deform_im2col_cuda.cuh:188-189
-        const float y = sub_rn(mul_rn(s[2 * t + 1], (float)lv.H), 0.5f);
-        const float pr = __expf(s[2 * LK + t] - mx) * inv;
-        const Tap tp = make_tap(y, x, lv.H, lv.W, base, step);
-        typename pack::raw_t raw[4];
-        if (staged) {
+        for (int k = 0; k < K; ++k) {
+          const int t = l * K + k;
+          const float x = sub_rn(mul_rn(s[2 * t], (float)lv.W), 0.5f);       // flash_deform_im2col_cuda.cuh:188-189
+          const float y = sub_rn(mul_rn(s[2 * t + 1], (float)lv.H), 0.5f);
+          const float pr = __expf(s[2 * LK + t] - mx) * inv;
+          const Tap tp = make_tap(y, x, lv.H, lv.W, base, step);
+          typename pack::raw_t raw[4];
+          if (staged) {
 #pragma unroll
-          for (int cn = 0; cn < 4; ++cn)
-            raw[cn] = *reinterpret_cast<const typename pack::raw_t *>(s_stage + ((tp.valid >> cn) & 1u ? tp.off[cn] : 0u));
-        } else {
+            for (int cn = 0; cn < 4; ++cn)
+              raw[cn] = *reinterpret_cast<const typename pack::raw_t *>(s_stage + ((tp.valid >> cn) & 1u ? tp.off[cn] : 0u));
+          } else {
 #pragma unroll
-          for (int cn = 0; cn < 4; ++cn) raw[cn] = buffer_load<pack::kBytes>(value, tp.off[cn]);
-        }
+            for (int cn = 0; cn < 4; ++cn) raw[cn] = buffer_load<pack::kBytes>(value, tp.off[cn]);
+          }
 #pragma unroll
-        for (int cn = 0; cn < 4; ++cn) {
-          float v[CPT];
-          pack::decode(raw[cn], v);
-          const float w = pr * tp.w[cn];
+          for (int cn = 0; cn < 4; ++cn) {
+            float v[CPT];
+            pack::decode(raw[cn], v);
+            const float w = pr * tp.w[cn];
 #pragma unroll
-          for (int c = 0; c < CPT; ++c) acc[c] = fmaf(w, v[c], acc[c]);
+            for (int c = 0; c < CPT; ++c) acc[c] = fmaf(w, v[c], acc[c]);
+          }
         }
       }
-    }
     }
     char *dst = (char *)p.out + ((size_t)(row0 + lr) * (p.G * p.D) + g * p.D + chunk * CPT) * Tag::kBytes;
     *reinterpret_cast<typename pack::raw_t *>(dst) = pack::encode(acc);
