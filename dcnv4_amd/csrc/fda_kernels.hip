@@ -14,6 +14,7 @@
 #include "common.hpp"
 #include "launch.hpp"
 
+#include <algorithm>
 #include <utility>
 
 namespace dcn {
@@ -790,7 +791,11 @@ hipError_t launch_by_cpt(const FdaLaunch &p, hipStream_t stream) {
   const bool head_major = p.head_major != 0;
   const dim3 grid(head_major ? (unsigned)((p.n_row / p.Q) * p.G * ((p.Q + p.nq_block - 1) / p.nq_block))
                              : (unsigned)((p.n_row + p.nq_block - 1) / p.nq_block)),
-      block(MODE == kFdaNoScatter && head_major ? kFdaBackwardThreads : (MODE < 0 && head_major ? kFdaForwardThreads : kBlockThreads));
+      // one head per workgroup: as many lanes as its queries fill (long rows leave the LDS room for fewer queries)
+      block(head_major && (MODE == kFdaNoScatter || MODE < 0)
+                ? (unsigned)std::min(MODE < 0 ? kFdaForwardThreads : kFdaBackwardThreads,
+                                     ((p.nq_block << p.lanes.tpgp_log2) + kWave - 1) / kWave * kWave)
+                : (unsigned)kBlockThreads);
   const size_t lds = MODE >= 0 ? fda_backward_lds_bytes(p) : fda_forward_lds_bytes(p);
 #define FDA_CASE(N)                                                                       \
   case N:                                                                                 \
