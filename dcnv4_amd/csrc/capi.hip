@@ -206,13 +206,13 @@ static bool plan_grad_value_for(DcnLaunch *L, int threads, int park_bytes) {
   L->tile_h_log2 = ceil_log2(L->tile_h);
   L->tile_w_log2 = ceil_log2(L->tile_w);
   const int anchors = (L->tile_h + 1) * (L->tile_w + 1);
-  const int max_items = kGradValueRounds * threads;
-  for (int ng = std::min({L->G, max_lists / anchors, 63, max_items / L->Kp}); ng >= 1; --ng) {
+  const int max_items = dcnv4_grad_value_max_slots(*L, threads), slots = dcnv4_grad_value_slots(*L);
+  for (int ng = std::min({L->G, max_lists / anchors, 63, max_items / slots}); ng >= 1; --ng) {
     L->ng_chunk = ng;
     int units = (ng * (L->gv_cw << L->gv_lps_log2) * park_bytes + 15) / 16;
     units |= 1;                                     // an odd number of 16-byte units spreads the rows over the LDS banks
     L->gv_go_stride = units * 16;
-    for (int s = std::min(1023, max_items / (L->Kp * ng)); s >= 1; s = s > 64 ? s - 16 : s - 1) {
+    for (int s = std::min(1023, max_items / (slots * ng)); s >= 1; s = s > 64 ? s - 16 : s - 1) {
       L->strip_pix = s;
       if (dcnv4_grad_value_lds_bytes(*L) <= budget) return true;
     }

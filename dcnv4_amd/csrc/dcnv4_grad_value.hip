@@ -82,7 +82,12 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
   u32x4 *s_entry = reinterpret_cast<u32x4 *>(s_go + (size_t)p.strip_pix * go_stride);
   // an entry's last word: parked grad_out address / 16 (14 bits) | index of the next entry << 14; the list ends at
   // the dummy entry behind the strip's items, which points at itself
-  const uint32_t end_idx = (uint32_t)(p.strip_pix * Kp * p.ng_chunk);
+  // Phase A's work items: for a 3x3 kernel a column of the kernel - three sampling points of one (pixel, group), with
+  // consecutive offsets in memory - so that what they share (the item's decode, the pixel's address and reference
+  // point) is done once; otherwise one sampling point.  Every item has kTaps entry slots.
+  constexpr int kTaps = KP > 0 ? 3 : 1;
+  const int upp = KP > 0 ? 3 : Kp;                            // items per (pixel, group)
+  const uint32_t end_idx = (uint32_t)(p.strip_pix * upp * kTaps * p.ng_chunk);
 
   // output pixels this tile visits: reference point (centre tap at zero offset) within `reach` of the tile
   const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
@@ -131,12 +136,12 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
     const int rows_cap = max(1, p.strip_pix / nwx);
     const int n_strips = (n_rows + rows_cap - 1) / rows_cap;
     const int rows_full = (n_rows + n_strips - 1) / n_strips;           // rows of the first strips (the last ones may have one fewer)
-    const int per_group = rows_full * nwx * Kp;                         // items of a group in a full strip
+    const int per_group = rows_full * nwx * upp;                        // items of a group in a full strip
     const int n_items = ng * per_group;
-    const float inv_per_group = 1.f / (float)per_group, inv_nwx = 1.f / (float)nwx, inv_kp = 1.f / (float)Kp;
+    const float inv_per_group = 1.f / (float)per_group, inv_nwx = 1.f / (float)nwx, inv_upp = 1.f / (float)upp;
 
-    // Phase A work items of this lane, one per round: row of the strip | column << 10 | group << 20 | tap << 26,
-    // all ones for a lane without an item.  The decode does not depend on the strip.
+    // Phase A work items of this lane, one per round: row of the strip | column << 10 | group << 20 | item of the
+    // (pixel, group) << 26, all ones for a lane without an item.  The decode does not depend on the strip.
     uint32_t item[ROUNDS];
 #pragma unroll
     for (int v = 0; v < ROUNDS; ++v) {
@@ -144,11 +149,29 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
       const bool in_range = j < n_items;
       const int gl = in_range ? fdiv_small(j, inv_per_group) : 0;
       const int rem = in_range ? j - gl * per_group : 0;
-      const int px = KP > 0 ? rem / (KP > 0 ? KP : 1) : fdiv_small(rem, inv_kp);
-      const int t = rem - px * Kp;
+      const int px = KP > 0 ? rem / 3 : fdiv_small(rem, inv_upp);
+      const int t = rem - px * upp;
       const int r = fdiv_small(px, inv_nwx), col = px - r * nwx;
       item[v] = in_range ? (uint32_t)r | ((uint32_t)col << 10) | ((uint32_t)gl << 20) | ((uint32_t)t << 26) : ~0u;
     }
+    // sampling point tj of item u: its index k among the group's points and its kernel position (x index outer,
+    // y index inner, dcnv4_im2col_cuda.cuh:216-236); false for the removed centre
+    auto tap_of = [&](int u, int tj, int &k, int &ti, int &tjj) -> bool {
+      if constexpr (KP == 9) {
+        k = 3 * u + tj; ti = u; tjj = tj;
+        return true;
+      } else if constexpr (KP == 8) {
+        const int kk = 3 * u + tj;
+        k = kk > 4 ? kk - 1 : kk; ti = u; tjj = tj;
+        return kk != 4;
+      } else {
+        k = u;
+        int tt = u;
+        if (p.remove_center && tt >= (p.kw / 2) * p.kh + p.kh / 2) ++tt;
+        ti = tt / p.kh; tjj = tt - ti * p.kh;
+        return true;
+      }
+    };
 
     // parking: 16-byte vectors when a group's channels are whole vectors and fill their parked width
     constexpr int kVec = 16 / Tag::kBytes;
@@ -159,19 +182,25 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
 
     // a lane's offsets of a strip, requested one strip ahead (before the previous strip's phase B) so that their
     // latency hides there; the modulation scalar lies in the same row and is read when it is needed
-    elem_t pf_x[ROUNDS], pf_y[ROUNDS];
+    elem_t pf_x[ROUNDS][kTaps], pf_y[ROUNDS][kTaps];
     auto prefetch = [&](int s) {
       const int rows_s = (n_rows - s + n_strips - 1) / n_strips;
 #pragma unroll
       for (int v = 0; v < ROUNDS; ++v) {
-        pf_x[v] = pf_y[v] = elem_t(0);
+#pragma unroll
+        for (int tj = 0; tj < kTaps; ++tj) pf_x[v][tj] = pf_y[v][tj] = elem_t(0);
         uint32_t it = item[v];
         asm volatile("" : "+v"(it));        // decoded afresh every strip: hoisted out of the loop, the fields of all rounds stay in registers
-        const int r = (int)(it & 0x3ffu), col = (int)((it >> 10) & 0x3ffu), gl = (int)((it >> 20) & 0x3fu), t = (int)(it >> 26);
+        const int r = (int)(it & 0x3ffu), col = (int)((it >> 10) & 0x3ffu), gl = (int)((it >> 20) & 0x3fu), u = (int)(it >> 26);
         if (it == ~0u || r >= rows_s) continue;
         const int ho = ho_lo + s + r * n_strips, wo = wo_lo + col;
         const elem_t *om = om_img + ((uint32_t)(ho * p.Wo + wo) * (uint32_t)p.P_pad + (uint32_t)((g0 + gl) * 3 * Kp));
-        pf_x[v] = om[2 * t]; pf_y[v] = om[2 * t + 1];
+#pragma unroll
+        for (int tj = 0; tj < kTaps; ++tj) {
+          int k, ti, tjj;
+          if (!tap_of(u, tj, k, ti, tjj)) continue;
+          pf_x[v][tj] = om[2 * k]; pf_y[v][tj] = om[2 * k + 1];
+        }
       }
     };
     prefetch(0);
@@ -209,7 +238,7 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
         }
       }
 
-      // ---- phase A: one lane per (group, pixel, tap).  A sampling point whose 2x2 corner block touches the tile is
+      // ---- phase A: one lane per item.  A sampling point whose 2x2 corner block touches the tile is
       // linked into the list of its ANCHOR - the block's first corner, which may lie one row above or one column left
       // of the tile: the lane swaps its entry's index into the list head and stores the old head as its successor.
 #pragma unroll
@@ -217,44 +246,49 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
         if (v * kValThreads >= n_items) continue;               // uniform
         uint32_t it = item[v];
         asm volatile("" : "+v"(it));
-        const int r = (int)(it & 0x3ffu), col = (int)((it >> 10) & 0x3ffu), gl = (int)((it >> 20) & 0x3fu), t = (int)(it >> 26);
+        const int r = (int)(it & 0x3ffu), col = (int)((it >> 10) & 0x3ffu), gl = (int)((it >> 20) & 0x3fu), u = (int)(it >> 26);
         if (it == ~0u || r >= rows_s) continue;
-        int ti, tj;
-        if constexpr (KP > 0) {
-          tap_ij_3x3(KP, t, ti, tj);
-        } else {      // x index outer, y index inner, centre skipped when remove_center
-          int tt = t;
-          if (p.remove_center && tt >= (p.kw / 2) * p.kh + p.kh / 2) ++tt;
-          ti = tt / p.kh; tj = tt - ti * p.kh;
-        }
         const int ho = ho_lo + s + r * n_strips, wo = wo_lo + col;
         const elem_t *om = om_img + ((uint32_t)(ho * p.Wo + wo) * (uint32_t)p.P_pad + (uint32_t)((g0 + gl) * 3 * Kp));
-        const elem_t m_raw = om[2 * Kp + t];      // requested before the position is formed: its latency hides behind that arithmetic
-        const float off_x = to_f(pf_x[v]), off_y = to_f(pf_y[v]);
         const float x_base = sub_rn((float)(cx0 + wo * p.sw), x_sub), y_base = sub_rn((float)(cy0 + ho * p.sh), y_sub);
-        const float x = add_rn(x_base, mul_rn(add_rn((float)(ti * p.dw), off_x), p.offset_scale));
-        const float y = add_rn(y_base, mul_rn(add_rn((float)(tj * p.dh), off_y), p.offset_scale));
-        // the reference's range test (dcnv4_col2im_cuda.cuh:317); NaN and huge coordinates fail it
-        if (!((y > -1.f) && (x > -1.f) && (y < Hf) && (x < Wf))) continue;
-        const float fy = floorf(y), fx = floorf(x);
-        // anchor relative to the anchor grid, whose first row and column lie one cell outside the tile
-        const int ay = (int)fy - ty0 + 1, ax = (int)fx - tx0 + 1;
-        if ((unsigned)ay > (unsigned)th || (unsigned)ax > (unsigned)tw) continue;
-        float m = to_f(m_raw);
-        if (p.softmax) {          // rare: normalise over this group's taps
-          float mx = load_f(om + 2 * Kp), sum = 0.f;
-          for (int k = 1; k < Kp; ++k) mx = fmaxf(mx, load_f(om + 2 * Kp + k));
-          for (int k = 0; k < Kp; ++k) sum += __expf(load_f(om + 2 * Kp + k) - mx);
-          m = __expf(m - mx) / sum;
-        }
-        const float ly = y - fy, lx = x - fx;
-        const int list = (ay * p.ng_chunk + gl) * aw + ax;
-        const uint32_t mine = (uint32_t)(v * kValThreads + tid);
-        const uint32_t succ = __hip_atomic_exchange(&head[list], mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         const int px = r * nwx + col;
         const uint32_t go_addr16 = (uint32_t)(px * go_stride + gl * Dp * kParkBytes) >> 4;
-        s_entry[mine] = u32x4{__builtin_bit_cast(uint32_t, m * (1.f - ly)), __builtin_bit_cast(uint32_t, m * ly),
-                              __builtin_bit_cast(uint32_t, lx), go_addr16 | (succ << 14)};
+        const int list_row = gl * aw;
+        // the item's modulation scalars, requested together before any position is formed: one latency per item
+        elem_t m_raws[kTaps];
+#pragma unroll
+        for (int tj = 0; tj < kTaps; ++tj) {
+          int k, ti, tjj;
+          m_raws[tj] = tap_of(u, tj, k, ti, tjj) ? om[2 * Kp + k] : elem_t(0);
+        }
+#pragma unroll
+        for (int tj = 0; tj < kTaps; ++tj) {
+          int k, ti, tjj;
+          if (!tap_of(u, tj, k, ti, tjj)) continue;
+          const elem_t m_raw = m_raws[tj];
+          const float off_x = to_f(pf_x[v][tj]), off_y = to_f(pf_y[v][tj]);
+          const float x = add_rn(x_base, mul_rn(add_rn((float)(ti * p.dw), off_x), p.offset_scale));
+          const float y = add_rn(y_base, mul_rn(add_rn((float)(tjj * p.dh), off_y), p.offset_scale));
+          // the reference's range test (dcnv4_col2im_cuda.cuh:317); NaN and huge coordinates fail it
+          if (!((y > -1.f) && (x > -1.f) && (y < Hf) && (x < Wf))) continue;
+          const float fy = floorf(y), fx = floorf(x);
+          // anchor relative to the anchor grid, whose first row and column lie one cell outside the tile
+          const int ay = (int)fy - ty0 + 1, ax = (int)fx - tx0 + 1;
+          if ((unsigned)ay > (unsigned)th || (unsigned)ax > (unsigned)tw) continue;
+          float m = to_f(m_raw);
+          if (p.softmax) {          // rare: normalise over this group's taps
+            float mx = load_f(om + 2 * Kp), sum = 0.f;
+            for (int kk = 1; kk < Kp; ++kk) mx = fmaxf(mx, load_f(om + 2 * Kp + kk));
+            for (int kk = 0; kk < Kp; ++kk) sum += __expf(load_f(om + 2 * Kp + kk) - mx);
+            m = __expf(m - mx) / sum;
+          }
+          const float ly = y - fy, lx = x - fx;
+          const int list = ay * (p.ng_chunk * aw) + list_row + ax;
+          const uint32_t mine = (uint32_t)((v * kValThreads + tid) * kTaps + tj);
+          const uint32_t succ = __hip_atomic_exchange(&head[list], mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          s_entry[mine] = u32x4{__builtin_bit_cast(uint32_t, m * (1.f - ly)), __builtin_bit_cast(uint32_t, m * ly),
+                                __builtin_bit_cast(uint32_t, lx), go_addr16 | (succ << 14)};
+        }
         __builtin_amdgcn_sched_barrier(0);      // one round at a time: interleaved, the rounds' temporaries spill
       }
       if (s + 1 < n_strips) prefetch(s + 1);
@@ -354,6 +388,8 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
   }
 }
 
+constexpr int gv_rounds(int kp) { return kp > 0 ? kGradValueColumnRounds : kGradValueRounds; }
+
 template <typename Tag>
 hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
   const int n_chunks = (p.G + p.ng_chunk - 1) / p.ng_chunk;
@@ -369,11 +405,11 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
 #define GV_CASE(KPV)                                                                \
   do {                                                                              \
     if (p.gv_threads == 512) {                                                      \
-      if (p.gv_cw == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, kGradValueRounds, 512>);      \
-      return go(dcnv4_grad_value_kernel<Tag, KPV, 16, kGradValueRounds, 512>);      \
+      if (p.gv_cw == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, gv_rounds(KPV), 512>);      \
+      return go(dcnv4_grad_value_kernel<Tag, KPV, 16, gv_rounds(KPV), 512>);      \
     }                                                                               \
-    if (p.gv_cw == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, kGradValueRounds, 1024>);       \
-    return go(dcnv4_grad_value_kernel<Tag, KPV, 16, kGradValueRounds, 1024>);       \
+    if (p.gv_cw == 8) return go(dcnv4_grad_value_kernel<Tag, KPV, 8, gv_rounds(KPV), 1024>);       \
+    return go(dcnv4_grad_value_kernel<Tag, KPV, 16, gv_rounds(KPV), 1024>);       \
   } while (0)
   if (k3 && !p.remove_center) GV_CASE(9);
   if (k3 && p.remove_center) GV_CASE(8);
@@ -384,7 +420,7 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
 }  // namespace
 
 size_t dcnv4_grad_value_lds_bytes(const DcnLaunch &p) {
-  const size_t items = (size_t)p.strip_pix * p.Kp * p.ng_chunk;
+  const size_t items = (size_t)p.strip_pix * dcnv4_grad_value_slots(p) * p.ng_chunk;
   // list heads (two sets), parked grad_out, entries + the dummy entry that ends every list; at the end the fp32 image
   // of the tile takes the place of all of it
   const size_t strip = 2 * (size_t)p.gv_threads * sizeof(uint32_t) + (size_t)p.strip_pix * p.gv_go_stride + (items + 1) * sizeof(u32x4);

@@ -88,9 +88,10 @@ struct DcnLaunch {
   int gt_reach;             // input pixels around an output pixel's reference point that the window covers
 };
 
-// Sampling points a lane of the tiled grad_value kernel handles per strip, at most: a strip holds at most
-// gv_threads * kGradValueRounds of them.
-constexpr int kGradValueRounds = 5;
+// Work items a lane of the tiled grad_value kernel handles per strip, at most.  An item is one sampling point, or -
+// for a 3x3 kernel - a column of the kernel: three points of one (pixel, group), the removed centre included.
+constexpr int kGradValueRounds = 5;            // items of one point
+constexpr int kGradValueColumnRounds = 2;      // items of three points
 // floats between the cells of the fp32 tile image in which the corner sums meet: the cell's channels rounded up to an odd
 // number of 16-byte units, so that the lanes of one LDS instruction (consecutive cells) fall into different banks
 __host__ __device__ inline int dcnv4_grad_value_image_stride(int channels) { return ((((channels + 3) / 4) | 1) * 4); }
@@ -217,6 +218,13 @@ hipError_t launch_depthwise_grad_weight_reduce(int dtype, const DwLaunch &p, hip
 hipError_t launch_dcnv4_forward(int dtype, const DcnLaunch &p, hipStream_t stream);
 hipError_t launch_dcnv4_offset_mask_grad(int dtype, const DcnLaunch &p, hipStream_t stream);
 hipError_t launch_dcnv4_grad_value(int dtype, const DcnLaunch &p, hipStream_t stream);
+// Entry slots of the tiled grad_value kernel per (pixel, group) of a strip, and at most per strip: three-point items
+// for a 3x3 kernel (nine slots, also when the centre is removed), else an item per sampling point.
+inline bool dcnv4_grad_value_columns(const DcnLaunch &p) { return p.kh == 3 && p.kw == 3; }
+inline int dcnv4_grad_value_slots(const DcnLaunch &p) { return dcnv4_grad_value_columns(p) ? 9 : p.Kp; }
+inline int dcnv4_grad_value_max_slots(const DcnLaunch &p, int threads) {
+  return dcnv4_grad_value_columns(p) ? kGradValueColumnRounds * threads * 3 : kGradValueRounds * threads;
+}
 size_t dcnv4_grad_value_lds_bytes(const DcnLaunch &p);
 hipError_t launch_dcnv4_forward_tiled(int dtype, const DcnLaunch &p, hipStream_t stream);
 hipError_t launch_dcnv4_offset_mask_grad_tiled(int dtype, const DcnLaunch &p, hipStream_t stream);
