@@ -253,6 +253,16 @@ __device__ __forceinline__ void unstage_tile_grads(const DcnLaunch &p, const Til
   }
 }
 
+// Two adjacent lanes that share a (pixel, group) - each with half of its channels - also share the work per sampling
+// point that does not depend on the channel: of every two points the even lane prepares the first and the odd lane
+// the second, and both read what the other prepared with a DPP move (J = 0: the even lane's value, 1: the odd lane's).
+template <int J> __device__ __forceinline__ int pair_pick(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, J == 0 ? 0xA0 : 0xF5, 0xf, 0xf, true);      // quad_perm [J, J, 2 + J, 2 + J]
+}
+template <int J> __device__ __forceinline__ float pair_pick(float v) {
+  return __builtin_bit_cast(float, pair_pick<J>(__builtin_bit_cast(int, v)));
+}
+
 // One sampling point against the staged window.
 struct WinTap {
   float w[4];          // bilinear weights of the four corners (without the modulation)
@@ -280,7 +290,7 @@ __device__ __forceinline__ WinTap window_tap(float y, float x, int H, int W, con
   return r;
 }
 
-template <typename Tag, int NV, int KP>
+template <typename Tag, int NV, int KP, bool PAIR>      // PAIR: gt_lpg == 2 and KP > 0
 __global__ void __launch_bounds__(kTiledThreads) dcnv4_forward_tiled_kernel(const DcnLaunch p) {
   extern __shared__ u32x4 lds128[];
   typedef typename RawWord<Tag::kBytes>::type elem_t;
@@ -375,8 +385,41 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_forward_tiled_kernel(cons
     // A real loop, one sampling point at a time: unrolled, the compiler front-loads all 72 LDS reads
     // and spills, and keeping two points in flight by hand costs more in registers (occupancy) than
     // the overlap returns; other waves cover the LDS latency.
+    int k_first = 0;
+    if constexpr (PAIR) {
+      const int common_bytes = lane_bytes - part * NV * 16, part_bytes = part * NV * 16;
 #pragma unroll 1
-    for (int k = 0; k < KP; ++k) {
+      for (int k0 = 0; k0 + 1 < KP; k0 += 2) {
+        int i, j;
+        tap_ij_3x3(KP, k0 + part, i, j);
+        float y, x, m;
+        position(k0 + part, i, j, y, x, m);
+        const WinTap wt = window_tap(y, x, p.H, p.W, t, cell_stride, common_bytes, zero_base);
+        const int far_own = wt.inside && !wt.ok;
+        float wq[4];
+#pragma unroll
+        for (int cn = 0; cn < 4; ++cn) wq[cn] = m * wt.w[cn];
+        auto one = [&](auto jj) {
+          constexpr int J = decltype(jj)::value;
+          far_mask |= (mask_t)pair_pick<J>(far_own) << (k0 + J);
+          const int addr = pair_pick<J>(wt.addr) + part_bytes;
+          Flight fl;
+#pragma unroll
+          for (int cn = 0; cn < 4; ++cn) {
+            fl.w[cn] = pair_pick<J>(wq[cn]);
+            const char *src = s_win + addr + (cn & 1) * cell_stride + (cn >> 1) * row_bytes;
+#pragma unroll
+            for (int v = 0; v < NV; ++v) fl.raw[cn][v] = *reinterpret_cast<const u32x4 *>(src + 16 * v);
+          }
+          retire(fl);
+        };
+        one(std::integral_constant<int, 0>{});
+        one(std::integral_constant<int, 1>{});
+      }
+      k_first = KP & ~1;      // an odd last point: both lanes prepare it
+    }
+#pragma unroll 1
+    for (int k = k_first; k < KP; ++k) {
       int i, j;
       tap_ij_3x3(KP, k, i, j);
       Flight fl;
@@ -423,7 +466,7 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_forward_tiled_kernel(cons
 // LDS (each slot is read before it is overwritten) and the slices go back to memory as rows;
 // the workgroup that owns the last groups also clears the padding tail of its rows.  The kernel
 // also folds the reach the grad_value kernel has to cover into GradState.
-template <typename Tag, int NV, int KP>
+template <typename Tag, int NV, int KP, bool PAIR>      // PAIR: gt_lpg == 2 and KP > 0
 __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_kernel(const DcnLaunch p) {
   extern __shared__ u32x4 lds128[];
   typedef typename RawWord<Tag::kBytes>::type elem_t;
@@ -471,19 +514,19 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
     const bool pair = p.gt_lpg == 2;       // the two lanes of a (pixel, group) add their halves of each dot product
     typedef typename std::conditional<(KP > 0), uint32_t, uint64_t>::type mask_t;
     mask_t far_mask = 0;
-    auto put = [&](int k, float gx, float gy, float gz, float m) {
-      if (part != 0) return;
+    auto put = [&](int k, float gx, float gy, float gz, float m, bool writer) {
+      if (!writer) return;
       const float f0[1] = {gx * p.offset_scale * m}, f1[1] = {gy * p.offset_scale * m}, f2[1] = {gz};
       om[2 * k] = Pack<Tag, 1>::encode(f0);
       om[2 * k + 1] = Pack<Tag, 1>::encode(f1);
       om[2 * Kp + k] = Pack<Tag, 1>::encode(f2);
     };
-    auto combine = [&](int k, const float (&d)[4], float ly, float lx, const float (&w)[4], float m) {
+    auto combine = [&](int k, const float (&d)[4], float ly, float lx, const float (&w)[4], float m, bool writer) {
       const float hy = 1.f - ly, hx = 1.f - lx;
       const float gx = hy * (d[1] - d[0]) + ly * (d[3] - d[2]);      // common.h:188-201
       const float gy = hx * (d[2] - d[0]) + lx * (d[3] - d[1]);
       const float gz = w[0] * d[0] + w[1] * d[1] + w[2] * d[2] + w[3] * d[3];
-      put(k, gx, gy, gz, m);
+      put(k, gx, gy, gz, m, writer);
     };
     auto one_tap = [&](int k, int i, int j) {
       const float x = add_rn(x_base, mul_rn(add_rn((float)(i * p.dw), lds_elem<Tag>(om, 2 * k)), p.offset_scale));
@@ -530,7 +573,64 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
         }
         d[cn] = pair ? acc + dpp_quad_xor1(acc) : acc;
       }
-      combine(k, d, wt.ly, wt.lx, wt.w, m);      // all zeros for a point outside the image or the window
+      combine(k, d, wt.ly, wt.lx, wt.w, m, part == 0);      // all zeros for a point outside the image or the window
+    };
+    // The corner . grad_out sums of one point from the window, over all channels of the group.
+    auto window_dots = [&](int addr, float (&d)[4]) {
+      u32x4 raw[4][NV];
+#pragma unroll
+      for (int cn = 0; cn < 4; ++cn) {
+        const char *src = s_win + addr + (cn & 1) * cell_stride + (cn >> 1) * row_bytes;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) raw[cn][v] = *reinterpret_cast<const u32x4 *>(src + 16 * v);
+      }
+#pragma unroll
+      for (int cn = 0; cn < 4; ++cn) {
+        float acc = 0.f;
+        if constexpr (Tag::kBytes == 2) {
+          float acc1 = 0.f;
+#pragma unroll
+          for (int v = 0; v < NV; ++v) {
+            const u32x4 a = raw[cn][v], g = go_raw[v];
+            const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, gw[4] = {g.x, g.y, g.z, g.w};
+            acc = dot2_pair<Tag>(aw[0], gw[0], acc);
+            acc1 = dot2_pair<Tag>(aw[1], gw[1], acc1);
+            acc = dot2_pair<Tag>(aw[2], gw[2], acc);
+            acc1 = dot2_pair<Tag>(aw[3], gw[3], acc1);
+          }
+          acc += acc1;
+        } else {
+#pragma unroll
+          for (int v = 0; v < NV; ++v) {
+            float f[EPV];
+            pack::decode(raw[cn][v], f);
+#pragma unroll
+            for (int c = 0; c < EPV; ++c) acc = fmaf(f[c], go[v][c], acc);
+          }
+        }
+        d[cn] = acc + dpp_quad_xor1(acc);
+      }
+    };
+    // Two points at a time for a pair of lanes: each prepares one of them, both gather and multiply for both, and
+    // the lane that prepared a point forms its gradients and writes them.
+    auto two_taps = [&](int k0) {
+      const int k = k0 + part;
+      int i, j;
+      tap_ij_3x3(KP, k, i, j);
+      const float x = add_rn(x_base, mul_rn(add_rn((float)(i * p.dw), lds_elem<Tag>(om, 2 * k)), p.offset_scale));
+      const float y = add_rn(y_base, mul_rn(add_rn((float)(j * p.dh), lds_elem<Tag>(om, 2 * k + 1)), p.offset_scale));
+      const float m = lds_elem<Tag>(om, 2 * Kp + k);
+      const int part_bytes = part * NV * 16;
+      const WinTap wt = window_tap(y, x, p.H, p.W, t, cell_stride, lane_bytes - part_bytes, zero_base);
+      const int far_own = wt.inside && !wt.ok;
+      if (wt.inside) reach_f = fmaxf(reach_f, fmaxf(fabsf(x - p0xf), fabsf(y - p0yf)));
+      far_mask |= ((mask_t)pair_pick<0>(far_own) << k0) | ((mask_t)pair_pick<1>(far_own) << (k0 + 1));
+      float d0[4], d1[4], d[4];
+      window_dots(pair_pick<0>(wt.addr) + part_bytes, d0);
+      window_dots(pair_pick<1>(wt.addr) + part_bytes, d1);
+#pragma unroll
+      for (int cn = 0; cn < 4; ++cn) d[cn] = part ? d1[cn] : d0[cn];
+      combine(k, d, wt.ly, wt.lx, wt.w, m, true);
     };
     // a sampling point whose corners lie outside the staged window: gather from memory; its
     // offsets are re-read from memory because the LDS slots already hold gradients
@@ -557,12 +657,18 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
         }
         d[cn] = pair ? acc + dpp_quad_xor1(acc) : acc;
       }
-      combine(k, d, tp.ly, tp.lx, tp.w, m);
+      combine(k, d, tp.ly, tp.lx, tp.w, m, part == 0);
     };
 
     if constexpr (KP > 0) {
+      int k_first = 0;
+      if constexpr (PAIR) {
 #pragma unroll 1
-      for (int k = 0; k < KP; ++k) {
+        for (int k0 = 0; k0 + 1 < KP; k0 += 2) two_taps(k0);
+        k_first = KP & ~1;      // an odd last point: both lanes prepare it, the even one writes
+      }
+#pragma unroll 1
+      for (int k = k_first; k < KP; ++k) {
         int i, j;
         tap_ij_3x3(KP, k, i, j);
         one_tap(k, i, j);
@@ -603,7 +709,7 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
   unstage_tile_grads<Tag>(p, t, s_om);
 }
 
-template <typename Tag, int NV, bool BWD>
+template <typename Tag, int NV, bool BWD, bool PAIR>
 hipError_t launch_nv(const DcnLaunch &p, hipStream_t stream, dim3 grid, dim3 block, size_t lds) {
   const bool k3 = p.kh == 3 && p.kw == 3;
   auto go = [&](auto kernel) -> hipError_t {
@@ -613,13 +719,13 @@ hipError_t launch_nv(const DcnLaunch &p, hipStream_t stream, dim3 grid, dim3 blo
     return hipGetLastError();
   };
   if constexpr (BWD) {
-    if (k3 && !p.remove_center) return go(dcnv4_offset_mask_grad_tiled_kernel<Tag, NV, 9>);
-    if (k3 && p.remove_center) return go(dcnv4_offset_mask_grad_tiled_kernel<Tag, NV, 8>);
-    return go(dcnv4_offset_mask_grad_tiled_kernel<Tag, NV, 0>);
+    if (k3 && !p.remove_center) return go(dcnv4_offset_mask_grad_tiled_kernel<Tag, NV, 9, PAIR>);
+    if (k3 && p.remove_center) return go(dcnv4_offset_mask_grad_tiled_kernel<Tag, NV, 8, PAIR>);
+    return go(dcnv4_offset_mask_grad_tiled_kernel<Tag, NV, 0, false>);
   } else {
-    if (k3 && !p.remove_center) return go(dcnv4_forward_tiled_kernel<Tag, NV, 9>);
-    if (k3 && p.remove_center) return go(dcnv4_forward_tiled_kernel<Tag, NV, 8>);
-    return go(dcnv4_forward_tiled_kernel<Tag, NV, 0>);
+    if (k3 && !p.remove_center) return go(dcnv4_forward_tiled_kernel<Tag, NV, 9, PAIR>);
+    if (k3 && p.remove_center) return go(dcnv4_forward_tiled_kernel<Tag, NV, 8, PAIR>);
+    return go(dcnv4_forward_tiled_kernel<Tag, NV, 0, false>);
   }
 }
 
@@ -632,11 +738,12 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
   const dim3 grid((unsigned)(n_img * nty * ntx * n_chunks));
   const dim3 block((unsigned)((p.gt_h * p.gt_w * p.gt_ng * p.gt_lpg + kWave - 1) / kWave * kWave));
   const size_t lds = dcnv4_tiled_gather_lds_bytes(p, Tag::kBytes);
+  const bool pair = p.gt_lpg == 2;      // two lanes per (pixel, group): they share the set-up of the sampling points
   switch (p.D * Tag::kBytes / 16 / p.gt_lpg) {      // 16-byte vectors per lane
-    case 1: return launch_nv<Tag, 1, BWD>(p, stream, grid, block, lds);
-    case 2: return launch_nv<Tag, 2, BWD>(p, stream, grid, block, lds);
-    case 4: return launch_nv<Tag, 4, BWD>(p, stream, grid, block, lds);
-    case 8: return launch_nv<Tag, 8, BWD>(p, stream, grid, block, lds);
+    case 1: return launch_nv<Tag, 1, BWD, false>(p, stream, grid, block, lds);
+    case 2: return pair ? launch_nv<Tag, 2, BWD, true>(p, stream, grid, block, lds) : launch_nv<Tag, 2, BWD, false>(p, stream, grid, block, lds);
+    case 4: return pair ? launch_nv<Tag, 4, BWD, true>(p, stream, grid, block, lds) : launch_nv<Tag, 4, BWD, false>(p, stream, grid, block, lds);
+    case 8: return launch_nv<Tag, 8, BWD, false>(p, stream, grid, block, lds);
   }
   return hipErrorInvalidValue;
 }
