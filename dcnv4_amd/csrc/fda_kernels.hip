@@ -61,7 +61,7 @@ __device__ __forceinline__ void fda_stage_rows(float *lds, const FdaLaunch &p, i
         const int j = fdiv20(i, inv_vpr), v = i - j * vpr;
         const int r = fdiv20(j, inv_h), gh = j - r * heads_here;
         float f[EPV];
-        Pack<Tag, EPV>::decode(src[((size_t)(row0 + r) * p.G + g0 + gh) * vpr + v], f);
+        Pack<Tag, EPV>::decode(__builtin_nontemporal_load(src + ((size_t)(row0 + r) * p.G + g0 + gh) * vpr + v), f);
 #pragma unroll
         for (int e = 0; e < EPV; e += 4)
           *reinterpret_cast<f32x4 *>(lds + i * EPV + e) = f32x4{f[e], f[e + 1], f[e + 2], f[e + 3]};
@@ -115,7 +115,7 @@ __device__ __forceinline__ void fda_unstage_grads(const float *lds, const FdaLau
           const f32x4 q = *reinterpret_cast<const f32x4 *>(lds + i * EPV + e);
           f[e] = q.x; f[e + 1] = q.y; f[e + 2] = q.z; f[e + 3] = q.w;
         }
-        dst[((size_t)(row0 + r) * p.G + g0 + gh) * vpr + v] = Pack<Tag, EPV>::encode(f);
+        __builtin_nontemporal_store(Pack<Tag, EPV>::encode(f), dst + ((size_t)(row0 + r) * p.G + g0 + gh) * vpr + v);
       }
     } else {
       const float inv_len = 1.f / (float)row_len;
@@ -293,8 +293,8 @@ __device__ __forceinline__ float fda_quad_level_backward(const float (&go)[CPT],
       if (tp.valid != 0)
         key = (tp.y0 + 1 >= kFdaKeyFieldMax || tp.x0 + 1 >= kFdaKeyFieldMax) ? kFdaKeySaturated
                                                                             : ((uint32_t)(tp.y0 + 1) << 8) | (uint32_t)(tp.x0 + 1);
-      keys[k0 + my_k] = (uint16_t)key;
-      recs[k0 + my_k] = f32x4_t{x, y, pr, 0.f};
+      __builtin_nontemporal_store((uint16_t)key, keys + k0 + my_k);
+      __builtin_nontemporal_store(f32x4_t{x, y, pr, 0.f}, recs + k0 + my_k);
     }
     dot_mine = fmaf(pr, gz, dot_mine);
   }
@@ -605,7 +605,7 @@ __global__ void __launch_bounds__(kFdaBackwardThreads) fda_backward_kernel(const
     float go[CPT];
     {
       const char *src = (const char *)p.grad_out + ((size_t)(row0 + lr) * (p.G * p.D)) * Tag::kBytes + lane_base;
-      pack::decode(*reinterpret_cast<const typename pack::raw_t *>(src), go);
+      pack::decode(__builtin_nontemporal_load(reinterpret_cast<const typename pack::raw_t *>(src)), go);
       if (!active) {
 #pragma unroll
         for (int c = 0; c < CPT; ++c) go[c] = 0.f;
@@ -616,7 +616,7 @@ __global__ void __launch_bounds__(kFdaBackwardThreads) fda_backward_kernel(const
     if constexpr (MODE == kFdaNoScatter) {      // grad_out regrouped by head: the grad_value kernel gathers rows of one head at a time
       if (active) {
         char *dst = (char *)p.go_rows + ((((size_t)b_local * p.G + g) * p.Q + q) * p.D + chunk * CPT) * Tag::kBytes;
-        *reinterpret_cast<typename pack::raw_t *>(dst) = pack::encode(go);
+        __builtin_nontemporal_store(pack::encode(go), reinterpret_cast<typename pack::raw_t *>(dst));
       }
     }
 
