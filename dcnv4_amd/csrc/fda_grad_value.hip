@@ -129,7 +129,7 @@ __global__ void __launch_bounds__(kBinThreads) fda_bin_points_kernel(const FdaLa
 #pragma unroll
   for (int u = 0; u < kBinWordsPerLane; ++u) {
     const int w = chunk * (kFdaChunkPoints / 2) + u * kBinThreads + tid;
-    const uint32_t word = keys[min(w, n_words - 1)];
+    const uint32_t word = __builtin_nontemporal_load(keys + min(w, n_words - 1));
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const Touch t = touch_of((word >> (16 * h)) & 0xffffu, w < n_words ? 2u * (uint32_t)w + h : 0xffffffffu);
@@ -203,7 +203,8 @@ __global__ void __launch_bounds__(kBinThreads) fda_bin_points_kernel(const FdaLa
   const uint32_t n_lds = min(total, (uint32_t)kBinSortedCap);
   for (uint32_t i = 4u * tid; i < n_lds; i += 4u * kBinThreads) {      // the last piece may run past the list, inside the region
     const u32x2 w = *reinterpret_cast<const u32x2 *>(s_sorted + i);
-    *reinterpret_cast<u32x4 *>(region + i) = u32x4{pt0 + (w.x & 0xffffu), pt0 + (w.x >> 16), pt0 + (w.y & 0xffffu), pt0 + (w.y >> 16)};
+    __builtin_nontemporal_store(u32x4{pt0 + (w.x & 0xffffu), pt0 + (w.x >> 16), pt0 + (w.y & 0xffffu), pt0 + (w.y >> 16)},
+                                reinterpret_cast<u32x4 *>(region + i));
   }
 }
 
@@ -485,7 +486,7 @@ __global__ void __launch_bounds__(kTileCells * LPC * SUBS) fda_grad_value_kernel
               if (s_pre[mid] <= e) lo = mid; else hi = mid;
             }
             const uint32_t *region = p.regions + ((size_t)seg * p.n_chunks + c0 + lo) * (4 * kFdaChunkPoints);
-            s_list[i] = region[(s_tab[lo] & 0xffffu) + (e - s_pre[lo])];
+            s_list[i] = __builtin_nontemporal_load(region + (s_tab[lo] & 0xffffu) + (e - s_pre[lo]));      // read once
           }
           __syncthreads();
           apply_list(ne);
@@ -517,7 +518,7 @@ __global__ void __launch_bounds__(kTileCells * LPC * SUBS) fda_grad_value_kernel
       if (n >= 0 && n < p.N) {
         elem_t *dst = reinterpret_cast<elem_t *>(p.grad_value) + (((size_t)b * p.N + (size_t)n) * p.G + g) * D + my_part * CW;
         if ((D % CW) == 0 && (CW * Tag::kBytes) % 4 == 0) {
-          if (my_part * CW < D) *reinterpret_cast<goN_t *>(dst) = Pack<Tag, CW>::encode(acc);
+          if (my_part * CW < D) __builtin_nontemporal_store(Pack<Tag, CW>::encode(acc), reinterpret_cast<goN_t *>(dst));
         } else {
 #pragma unroll
           for (int c = 0; c < CW; ++c)

@@ -382,7 +382,7 @@ __global__ void __launch_bounds__(kFdaForwardThreads) fda_forward_kernel(const F
       }
     }
     char *dst = (char *)p.out + ((size_t)(row0 + lr) * (p.G * p.D) + g * p.D + chunk * CPT) * Tag::kBytes;
-    *reinterpret_cast<typename pack::raw_t *>(dst) = pack::encode(acc);
+    __builtin_nontemporal_store(pack::encode(acc), reinterpret_cast<typename pack::raw_t *>(dst));
   }
 }
 
