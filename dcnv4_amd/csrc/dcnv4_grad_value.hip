@@ -36,6 +36,7 @@
 #include "common.hpp"
 #include "launch.hpp"
 
+
 namespace dcn {
 namespace {
 
@@ -373,7 +374,10 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
         const f32x4 v = *reinterpret_cast<const f32x4 *>(src + i);
         f[i] = v.x; f[i + 1] = v.y; f[i + 2] = v.z; f[i + 3] = v.w;
       }
-      *reinterpret_cast<u32x4 *>(gv_img + ((size_t)((ty0 + cy) * p.W + tx0 + cx) * C + (g0 + gl) * D + ch)) = Pack<Tag, kVecOut>::encode(f);
+      u32x4 *dst = reinterpret_cast<u32x4 *>(gv_img + ((size_t)((ty0 + cy) * p.W + tx0 + cx) * C + (g0 + gl) * D + ch));
+      // fp32 tensors: with the nontemporal hint (T stage 1 backward 0.187 -> 0.180 ms); 16-bit ones lose 1-3 % to it
+      if constexpr (Tag::kBytes == 4) __builtin_nontemporal_store(Pack<Tag, kVecOut>::encode(f), dst);
+      else *dst = Pack<Tag, kVecOut>::encode(f);
     }
   } else {
     const int epc = ng * D;                                      // elements per cell

@@ -24,6 +24,7 @@
 #include "common.hpp"
 #include "launch.hpp"
 
+
 namespace dcn {
 namespace {
 
@@ -221,6 +222,9 @@ __device__ __forceinline__ void unstage_tile_grads(const DcnLaunch &p, const Til
     const uint32_t row_bytes = (uint32_t)p.Wo * p.P_pad * Tag::kBytes;
     const __amdgpu_buffer_rsrc_t rows = make_rsrc(gom, (uint32_t)(t.th - 1) * row_bytes + (uint32_t)((t.tw - 1) * p.P_pad + run) * Tag::kBytes);
     const uint32_t *s_om_w = reinterpret_cast<const uint32_t *>(s_om);
+    // fp32 gradients leave with the nontemporal hint (T stage 1 backward 0.187 -> 0.181 ms); with 16-bit tensors the
+    // same hint costs 1-3 %
+    constexpr int kStorePolicy = Tag::kBytes == 4 ? 2 : 0;
     const int ppp = bd >> team_log2;
     const int pl = tid >> team_log2, j = tid & ((1 << team_log2) - 1);
     for (int px0 = 0; px0 < t.tw; px0 += ppp) {
@@ -230,7 +234,7 @@ __device__ __forceinline__ void unstage_tile_grads(const DcnLaunch &p, const Til
         const int l_lane = px * (lds_row / EPW) + j;
         for (int py = 0; py < t.th; ++py)
           __builtin_amdgcn_raw_buffer_store_b32(s_om_w[l_lane + py * (p.gt_w * (lds_row / EPW))], rows,
-                                                g_lane + (uint32_t)py * row_bytes, 0, 0);
+                                                g_lane + (uint32_t)py * row_bytes, 0, kStorePolicy);
       }
     }
   } else {
