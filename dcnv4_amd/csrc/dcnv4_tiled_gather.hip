@@ -80,6 +80,17 @@ __device__ __forceinline__ TileGeom tile_geometry(const DcnLaunch &p) {
   return t;
 }
 
+// offset_mask / grad_offset_mask slices of a tile move in whole dwords when a pixel's run starts on a dword boundary
+// in memory and in LDS and either ends on one or has room for one element more: behind the last group the row is
+// padded, and a chunk with fewer groups than gt_ng leaves its LDS slice partly unused.
+template <typename Tag>
+__device__ __forceinline__ bool tile_runs_in_dwords(const DcnLaunch &p, const TileGeom &t) {
+  if constexpr (Tag::kBytes == 4) return true;
+  const int run = t.ng * 3 * p.Kp, lds_row = p.gt_ng * 3 * p.Kp;
+  if (((p.P_pad | (t.g0 * 3 * p.Kp) | lds_row) & 1) != 0) return false;
+  return (run & 1) == 0 || (run + 1 <= lds_row && t.g0 * 3 * p.Kp + run + 1 <= p.P_pad);
+}
+
 // Fills the workgroup's LDS: the input window and this chunk's slice of offset_mask.
 //
 // Window: [wy0, wy0+wh) x [wx0, wx0+ww) of this chunk's channels, cell-major (cell = all channels
@@ -107,15 +118,17 @@ __device__ __forceinline__ void stage_tile(const DcnLaunch &p, const TileGeom &t
   const int run = t.ng * 3 * p.Kp, lds_row = p.gt_ng * 3 * p.Kp;          // elements per pixel: copied / LDS stride
   const elem_t *om = reinterpret_cast<const elem_t *>(p.offset_mask) + ((size_t)t.b * p.Q + (size_t)t.oy0 * p.Wo + t.ox0) * p.P_pad +
                      t.g0 * 3 * p.Kp;                                      // first element of the tile's slice
-  // whole dwords when every run starts and ends on a dword boundary (always for fp32)
-  const bool dwords = Tag::kBytes == 4 || (((p.P_pad | (t.g0 * 3 * p.Kp) | run | lds_row) & 1) == 0);
-  const int rw = run / EPW;                                               // dwords per pixel
+  // whole dwords when every run starts on a dword boundary (always for fp32); a run of an odd number of 16-bit
+  // elements - the last chunk of an odd number of groups - takes the element behind it along, which lies in the row's
+  // padding and has room in the LDS slice
+  const bool dwords = tile_runs_in_dwords<Tag>(p, t);
+  const int rw = (run + EPW - 1) / EPW;                                   // dwords per pixel
   int team_log2 = 0;
   while ((1 << team_log2) < rw) ++team_log2;
   const bool teams = dwords && (1 << team_log2) <= bd;
   // a power-of-two team of lanes per tile pixel; the tile's rows are row_bytes apart in memory
   const uint32_t om_row_bytes = (uint32_t)p.Wo * p.P_pad * Tag::kBytes;
-  const __amdgpu_buffer_rsrc_t om_rows = make_rsrc(om, teams ? (uint32_t)(t.th - 1) * om_row_bytes + (uint32_t)((t.tw - 1) * p.P_pad + run) * Tag::kBytes : 0u);
+  const __amdgpu_buffer_rsrc_t om_rows = make_rsrc(om, teams ? (uint32_t)(t.th - 1) * om_row_bytes + (uint32_t)((t.tw - 1) * p.P_pad + rw * EPW) * Tag::kBytes : 0u);
   uint32_t *s_om_w = reinterpret_cast<uint32_t *>(s_om);
   const int ppp = max(bd >> team_log2, 1);                                // pixels per pass
   const int pl = tid >> team_log2, j = tid & ((1 << team_log2) - 1);
@@ -214,13 +227,14 @@ __device__ __forceinline__ void unstage_tile_grads(const DcnLaunch &p, const Til
   const int run = t.ng * 3 * p.Kp, lds_row = p.gt_ng * 3 * p.Kp;
   elem_t *gom = reinterpret_cast<elem_t *>(p.grad_offset_mask) + ((size_t)t.b * p.Q + (size_t)t.oy0 * p.Wo + t.ox0) * p.P_pad +
                 t.g0 * 3 * p.Kp;
-  const bool dwords = Tag::kBytes == 4 || (((p.P_pad | (t.g0 * 3 * p.Kp) | run | lds_row) & 1) == 0);
-  const int rw = run / EPW;
+  const bool dwords = tile_runs_in_dwords<Tag>(p, t);
+  const int rw = (run + EPW - 1) / EPW;
+  const bool odd_run = (run % EPW) != 0;      // the last dword's upper half lies in the padding: its gradient is zero
   int team_log2 = 0;
   while ((1 << team_log2) < rw) ++team_log2;
   if (dwords && (1 << team_log2) <= bd) {
     const uint32_t row_bytes = (uint32_t)p.Wo * p.P_pad * Tag::kBytes;
-    const __amdgpu_buffer_rsrc_t rows = make_rsrc(gom, (uint32_t)(t.th - 1) * row_bytes + (uint32_t)((t.tw - 1) * p.P_pad + run) * Tag::kBytes);
+    const __amdgpu_buffer_rsrc_t rows = make_rsrc(gom, (uint32_t)(t.th - 1) * row_bytes + (uint32_t)((t.tw - 1) * p.P_pad + rw * EPW) * Tag::kBytes);
     const uint32_t *s_om_w = reinterpret_cast<const uint32_t *>(s_om);
     // fp32 gradients leave with the nontemporal hint (T stage 1 backward 0.187 -> 0.181 ms); with 16-bit tensors the
     // same hint costs 1-3 %
@@ -232,8 +246,9 @@ __device__ __forceinline__ void unstage_tile_grads(const DcnLaunch &p, const Til
       if (px < t.tw && j < rw) {
         const uint32_t g_lane = (uint32_t)(px * p.P_pad) * Tag::kBytes + 4u * j;
         const int l_lane = px * (lds_row / EPW) + j;
+        const uint32_t keep = (odd_run && j == rw - 1) ? 0xffffu : 0xffffffffu;
         for (int py = 0; py < t.th; ++py)
-          __builtin_amdgcn_raw_buffer_store_b32(s_om_w[l_lane + py * (p.gt_w * (lds_row / EPW))], rows,
+          __builtin_amdgcn_raw_buffer_store_b32(s_om_w[l_lane + py * (p.gt_w * (lds_row / EPW))] & keep, rows,
                                                 g_lane + (uint32_t)py * row_bytes, 0, kStorePolicy);
       }
     }
