@@ -80,6 +80,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-detail", action="store_true", help="skip per-operator timings other than the step's own")
     ap.add_argument("--no-model", action="store_true", help="skip the FlashInternImage-B end-to-end forward")
+    ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the step (step_graph_ms)")
     ap.add_argument("--only-op", default=None, metavar="OP:SHAPE:DTYPE",
                     help="profiling aid: run just one operator of the step --steps times and exit, e.g. "
                          "dcnv4_bwd:T-stage1:float32 (prints its HIP-event time); also copy:MB for a plain device copy")
@@ -277,6 +278,29 @@ def main():
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
+    # The same step captured once in a HIP graph and replayed: what remains of a step when the host only submits one
+    # graph instead of making 16 operator calls (reported beside ms_per_step, never in place of it).
+    step_graph_ms = None
+    if not args.no_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        step_graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        del graph
+
     # ------------------------------------------------------------------ per-operator detail
     detail = []
 
@@ -460,11 +484,12 @@ def main():
     line = {
         "metric": "DCNv4 fwd+bwd achieved HBM GB/s (algorithmic bytes / time)", "value": round(value, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "step_graph_ms": None if step_graph_ms is None else round(step_graph_ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "DCNv4 forward+backward, FlashInternImage-T stages (56x56 C64 G4, 28x28 C128 G8, "
                                "14x14 C256 G16, 7x7 C512 G32), batch 64, 3x3 s1 p1, fp16 and fp32 tensors, fp32 arithmetic",
                    "step_algorithmic_MB": round(step_bytes / 1e6, 1), "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2)},
-        "roofline": roofline, "cpu_baseline": cpu, "flash_intern_image_b": model_line, "detail": detail,
+        "roofline": roofline, "cpu_baseline": cpu, "detail": detail, "flash_intern_image_b": model_line,
     }
     print(json.dumps(line))
 

@@ -494,6 +494,15 @@ int check_ptrs(std::initializer_list<const void *> ptrs) {
   return DCNV4_OK;
 }
 
+// A small parameter vector that the kernels read element by element (a view into a flat parameter buffer need not
+// start on a 16-byte boundary).
+int check_elem_ptr(const void *p, int elem_bytes_of_ptr) {
+  if (p == nullptr) return fail(DCNV4_ERR_RUNTIME, "null tensor pointer");
+  if ((reinterpret_cast<uintptr_t>(p) & (uintptr_t)(elem_bytes_of_ptr - 1)) != 0)
+    return fail(DCNV4_ERR_RUNTIME, "tensor pointer %p is not aligned to its %d-byte elements", p, elem_bytes_of_ptr);
+  return DCNV4_OK;
+}
+
 int hip_fail(const char *what, hipError_t e) {
   return fail(DCNV4_ERR_RUNTIME, "%s: %s", what, hipGetErrorString(e));
 }
@@ -1183,7 +1192,8 @@ int dcnv4_gfx950_center_feature_blend_forward(const void *sampled, const void *p
                                               int channels, int groups, void *stream) {
   CfLaunch L;
   if (int rc = cf_prepare(&L, dtype, rows, channels, groups)) return rc;
-  if (int rc = check_ptrs({sampled, projected, weight, bias, output})) return rc;
+  if (int rc = check_ptrs({sampled, projected, weight, output})) return rc;
+  if (int rc = check_elem_ptr(bias, elem_bytes(dtype))) return rc;      // read with scalar loads
   L.y = sampled; L.x = projected; L.weight = weight; L.bias = bias; L.out = output;
   if (hipError_t e = launch_center_feature_blend(dtype, L, false, static_cast<hipStream_t>(stream)))
     return hip_fail("centre-feature blend launch", e);
@@ -1196,7 +1206,8 @@ int dcnv4_gfx950_center_feature_blend_backward(const void *grad_output, const vo
                                                long long rows, int channels, int groups, void *stream) {
   CfLaunch L;
   if (int rc = cf_prepare(&L, dtype, rows, channels, groups)) return rc;
-  if (int rc = check_ptrs({grad_output, sampled, projected, weight, bias, grad_sampled, grad_projected, grad_gate_logits})) return rc;
+  if (int rc = check_ptrs({grad_output, sampled, projected, weight, grad_sampled, grad_projected, grad_gate_logits})) return rc;
+  if (int rc = check_elem_ptr(bias, elem_bytes(dtype))) return rc;
   L.grad_out = grad_output; L.y = sampled; L.x = projected; L.weight = weight; L.bias = bias;
   L.grad_y = grad_sampled; L.grad_x = grad_projected; L.grad_logits = grad_gate_logits;
   if (hipError_t e = launch_center_feature_blend(dtype, L, true, static_cast<hipStream_t>(stream)))

@@ -91,8 +91,10 @@ __device__ __forceinline__ void fda_stage_rows(float *lds, const FdaLaunch &p, i
   }
 }
 
-// The gradient rows back to memory, same layouts; the gradient of a location passes through the fp16 rounding
-// unchanged (the derivative of a cast) and is written in the locations' dtype.
+// The gradient rows back to memory, same layouts.  The gradient of a location is written in the locations' dtype;
+// for fp32 locations it is rounded through fp16 first (values beyond the fp16 range become infinities), as autograd
+// does in the reference's module: the gradient of `sampling_locations.half()` arrives as an fp16 tensor and is then
+// widened (DCNv4_op/DCNv4/modules/flash_deform_attn.py:132-133).
 template <typename Tag>
 __device__ __forceinline__ void fda_unstage_grads(const float *lds, const FdaLaunch &p, int row0, int nrow, int g0, int heads_here) {
   typedef typename RawWord<Tag::kBytes>::type elem_t;
@@ -134,7 +136,7 @@ __device__ __forceinline__ void fda_unstage_grads(const float *lds, const FdaLau
     const int r = fdiv20(j, inv_h), gh = j - r * heads_here;
     const size_t dst = ((size_t)(row0 + r) * p.G + g0 + gh) * (2 * LK) + e;
     const float f[1] = {lds[j * row_len + e]};
-    if (p.loc_f32) reinterpret_cast<float *>(p.grad_loc)[dst] = f[0];
+    if (p.loc_f32) reinterpret_cast<float *>(p.grad_loc)[dst] = (float)(_Float16)f[0];
     else reinterpret_cast<elem_t *>(p.grad_loc)[dst] = Pack<Tag, 1>::encode(f);
   }
   for (int i = threadIdx.x; i < pairs * LK; i += blockDim.x) {

@@ -315,6 +315,12 @@ def layer_norm_residual_backward(grad_output, input, weight, bias, gamma, eps, n
     return [grad_input, grad_weight, grad_bias, grad_gamma]
 
 
+def _aligned16(t):
+    """`t`, or a copy of it when its storage does not start on a 16-byte boundary (a view into a flat parameter
+    buffer): the kernels read this tensor in 16-byte vectors."""
+    return t if t.data_ptr() % 16 == 0 else t.clone(memory_format=torch.contiguous_format)
+
+
 def _blend_common(sampled, projected, weight, bias):
     _check(sampled, "sampled")
     _check(projected, "projected", sampled.dtype)
@@ -331,6 +337,7 @@ def center_feature_blend_forward(sampled, projected, weight, bias):
     """``sampled * (1 - gate) + projected * gate`` with ``gate = sigmoid(sampled @ weight.T + bias)`` per (pixel,
     group), every channel using its group's gate (DCNv4_op/DCNv4/modules/dcnv4.py:142-147) in one kernel."""
     code, rows, channels, groups = _blend_common(sampled, projected, weight, bias)
+    weight = _aligned16(weight)
     with torch.cuda.device(sampled.device):
         output = torch.empty_like(sampled)
         if sampled.numel():
@@ -344,6 +351,7 @@ def center_feature_blend_backward(grad_output, sampled, projected, weight, bias)
     """``[grad_sampled, grad_projected, grad_gate_logits]``; the last is fp32 (rows, groups): ``grad_weight`` is
     ``grad_gate_logits.T @ sampled`` and ``grad_bias`` its column sums."""
     code, rows, channels, groups = _blend_common(sampled, projected, weight, bias)
+    weight = _aligned16(weight)
     _check(grad_output, "grad_output", sampled.dtype)
     if grad_output.shape != sampled.shape:
         raise RuntimeError("grad_output must have the shape of sampled")

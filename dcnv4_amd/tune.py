@@ -43,7 +43,7 @@ def candidates(G, D, elem_bytes, direction):
     """(label, options, d_stride, n_thread) for a DCNv4 call; the first one is the library's own choice.  Every launch
     parameter the kernels have is swept, as the reference's search scripts sweep theirs
     (DCNv4_op/scripts/search_dcnv4.py:100-115): kernel family, hints of the direct family, the staged reach and the
-    output-tile cap of the LDS-tiled gathers, the input-tile cap of the grad_value kernel."""
+    output-tile cap of the LDS-tiled gathers, the input-tile cap and the workgroup size of the grad_value kernel."""
     out = [("library", {}, 0, 0)]
     for reach in (2, 3, 4, 6):
         out.append((f"reach {reach}", {"reach": reach}, 0, 0))
@@ -60,6 +60,9 @@ def candidates(G, D, elem_bytes, direction):
         for tile in (16, 8):
             out.append((f"grad_value tile {tile}", {"tile": tile}, 0, 0))
             out.append((f"grad_value tile {tile} reach 3", {"tile": tile, "reach": 3}, 0, 0))
+        for threads in (512, 1024):
+            out.append((f"grad_value {threads} lanes", {"gv_threads": threads}, 0, 0))
+            out.append((f"grad_value {threads} lanes tile 16", {"gv_threads": threads, "tile": 16}, 0, 0))
     return out
 
 

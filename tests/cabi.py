@@ -125,12 +125,12 @@ def layer_norm_residual(y, residual, weight, bias, gamma, eps):
     return out
 
 
-def dcnv4_backward_static_scratch(value, om, go, geom, G, D, scale, rc=0, softmax=0, im2col_step=256):
-    """The allocation-free entry point: no workspace argument, scratch inside the library."""
+def dcnv4_backward_static_scratch(value, om, go, geom, G, D, scale, rc=0, softmax=0, im2col_step=256, out=None):
+    """The allocation-free entry point: no workspace argument, scratch inside the library.  `out` = (grad_value,
+    grad_offset_mask) tensors that exist already; without it they are created here."""
     L = _lib.load()
     B, H, W, _ = value.shape
-    gv = torch.full_like(value, float("nan"))
-    gom = torch.full_like(om, float("nan"))
+    gv, gom = out if out is not None else (torch.full_like(value, float("nan")), torch.full_like(om, float("nan")))
     rc_ = L.dcnv4_gfx950_backward_static_scratch(value.data_ptr(), om.data_ptr(), go.data_ptr(), gv.data_ptr(), gom.data_ptr(),
                                                  CODES[value.dtype], B, H, W, G, D, *geom, float(scale), im2col_step, rc,
                                                  om.shape[-1], softmax, 0, 0, _stream())

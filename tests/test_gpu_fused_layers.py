@@ -123,6 +123,20 @@ def test_center_feature_function_gradients_match_autograd_of_the_reference_expre
         assert torch.allclose(a, e, rtol=1e-4, atol=1e-4 * max(1.0, float(e.abs().max())))
 
 
+def test_center_feature_function_takes_parameters_that_are_views_into_a_flat_buffer():
+    """Flattened / fused parameter storage: weight and bias start 8 bytes into a 16-byte unit, where the
+    reference's F.linear works (DCNv4_op/DCNv4/modules/dcnv4.py:17-26)."""
+    from dcnv4_amd.functions import CenterFeatureBlendFunction
+    torch.manual_seed(6)
+    flat = torch.randn(2 + 4 * 64 + 4, device="cuda")
+    w, b = flat[2:2 + 256].view(4, 64), flat[258:262]
+    assert w.data_ptr() % 16 == 8 and b.data_ptr() % 16 == 8
+    y, x = torch.randn(3, 5, 64, device="cuda"), torch.randn(3, 5, 64, device="cuda")
+    got = CenterFeatureBlendFunction.apply(y, x, w, b)
+    s = torch.nn.functional.linear(y, w, b).sigmoid()[..., None].repeat(1, 1, 1, 16).flatten(-2)
+    assert torch.allclose(got, y * (1 - s) + x * s, rtol=1e-5, atol=1e-5)
+
+
 # ---------------------------------------------------------------- attention on un-packed rows
 @pytest.mark.parametrize("loc_fp32", [True, False], ids=["loc_fp32", "loc_like_value"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
@@ -173,6 +187,31 @@ def test_flash_deform_attn_split_head_major_order(oracle):
     cabi.assert_close(gv, wgv, *GRAD_TOL[torch.float16], what="grad_value")
     cabi.assert_close(gloc, wgs[..., : 2 * LK], 1e-2, 1e-2 * float(np.abs(wgs[..., : 2 * LK]).max()), what="grad_sampling_locations")
     cabi.assert_close(glog, wgs[..., 2 * LK:], *GRAD_TOL[torch.float16], what="grad_attention_logits")
+
+
+def test_flash_deform_attn_split_function_equals_the_reference_modules_half_and_cat_graph():
+    """fp32 locations through the split Function against the graph the reference's module builds with torch ops -
+    `.half()`, `cat`, the packed Function (DCNv4_op/DCNv4/modules/flash_deform_attn.py:132-133): autograd hands the
+    locations' gradient back through an fp16 tensor, so it is an fp16-rounded value in an fp32 tensor, bit for bit.
+    Gradients beyond the fp16 range (they would be infinities on both sides) are not covered: parity unpinned there."""
+    from dcnv4_amd.functions import FlashDeformAttnFunction, FlashDeformAttnSplitFunction
+    B, shapes, G, D, K = 2, [(20, 24), (10, 12), (5, 6)], 4, 32, 4
+    v, shp, st, sla, go = make_fda_inputs(B, shapes, G, D, K, 150, seed=21, dtype=torch.float32)
+    LK = len(shapes) * K
+    v, go = v.cuda().half(), (300.0 * go).cuda().half()
+    shp, st = shp.cuda(), st.cuda()
+    loc = sla[..., : 2 * LK].contiguous().cuda().requires_grad_(True)              # fp32
+    logits = sla[..., 2 * LK:].contiguous().cuda().half().requires_grad_(True)
+    out = FlashDeformAttnSplitFunction.apply(v, shp, st, loc, logits, 64, K)
+    g_loc, g_logits = torch.autograd.grad(out, [loc, logits], go)
+    loc2, logits2 = loc.detach().clone().requires_grad_(True), logits.detach().clone().requires_grad_(True)
+    out2 = FlashDeformAttnFunction.apply(v, shp, st, torch.cat([loc2.half(), logits2], -1), 64, K)
+    w_loc, w_logits = torch.autograd.grad(out2, [loc2, logits2], go)
+    assert g_loc.dtype == torch.float32 and w_loc.dtype == torch.float32
+    assert torch.equal(out, out2)
+    assert torch.equal(g_loc, w_loc), f"largest difference {(g_loc - w_loc).abs().max().item()}"
+    assert torch.equal(g_logits, w_logits)
+    assert torch.equal(g_loc, g_loc.half().float())          # every value is fp16-representable
 
 
 def test_flash_deform_attn_split_rejects_mismatched_location_dtype():

@@ -94,6 +94,10 @@ KERNEL_PATHS = {
     "tile8_reach1": dict(tile=8, reach=1),
     "gv512": dict(gv_threads=512),                             # grad_value workgroups of 512 / 1024 lanes
     "gv1024": dict(gv_threads=1024),
+    "gather_tile4": dict(gather_tile=4),                       # smaller output tiles of the LDS-tiled gathers (more groups each)
+    "gather_tile8": dict(gather_tile=8),
+    "gather_tile8_reach2": dict(gather_tile=8, reach=2),
+    "gather_tile4_gv512": dict(gather_tile=4, gv_threads=512),
 }
 
 

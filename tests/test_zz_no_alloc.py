@@ -21,16 +21,22 @@ def test_static_scratch_backward_matches_workspace_backward_twice_in_a_row(oracl
         print(f"static scratch call {n}: {B}x{H}x{W} G{G} D{D} {dtype}", flush=True)
         vd, omd, god = v.cuda(), om.cuda(), go.cuda()
         gv_ws, gom_ws = cabi.dcnv4_backward(vd, omd, god, GEOM, G, D, 1.0)
-        before = torch.cuda.memory_allocated()
-        gv, gom = cabi.dcnv4_backward_static_scratch(vd, omd, god, GEOM, G, D, 1.0)
+        # outputs exist before the call; around the call itself neither torch's allocator nor the device's free
+        # memory may move (the entry point's own first-call set-up - the scratch address, a kernel attribute - allocates
+        # nothing either)
+        gv, gom = torch.full_like(vd, float("nan")), torch.full_like(omd, float("nan"))
         torch.cuda.synchronize()
+        before = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.mem_get_info()[0])
+        cabi.dcnv4_backward_static_scratch(vd, omd, god, GEOM, G, D, 1.0, out=(gv, gom))
+        torch.cuda.synchronize()
+        after = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.mem_get_info()[0])
+        assert after == before, f"the allocation-free entry point moved device memory: {before} -> {after}"
         rtol, atol = GRAD_TOL[dtype]
         cabi.assert_close(gv, cabi.f64(gv_ws), rtol, atol, what=f"grad_value, call {n}")
         cabi.assert_close(gom, cabi.f64(gom_ws), rtol, atol, what=f"grad_offset_mask, call {n}")
         wgv, wgom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *GEOM, G, D, 1.0, 0, coord_f32=True)
         cabi.assert_close(gv, wgv, rtol, atol, what=f"grad_value vs oracle, call {n}")
         cabi.assert_close(gom, wgom, rtol, atol, what=f"grad_offset_mask vs oracle, call {n}")
-        del before
 
 
 def test_static_scratch_backward_reports_errors_like_the_workspace_entry_point():
