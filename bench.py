@@ -41,6 +41,8 @@ CFG5 = [("B-stage1", 128, 56, 56, 112, 7), ("B-stage2", 128, 28, 28, 224, 14),
 CFG4_SHAPES = [(128, 128), (64, 64), (32, 32), (16, 16)]
 # the shape of the reference's only timing note (DCNv4_op/scripts/test_dcnv4_bwd.py:94-106: 64 x 56 x 56 x 128, 4 groups of 32)
 DEVNOTE = [("ref-note-56x56-C128-G4", 64, 56, 56, 128, 4)]
+# groups of 64 channels: two of the reference's tuned keys (DCNv4_op/DCNv4/functions/table.py:452-461, "64x56x56x4x64", "64x28x28x4x64")
+WIDE = [("ref-key-56x56-G4-D64", 64, 56, 56, 256, 4), ("ref-key-28x28-G4-D64", 64, 28, 28, 256, 4)]
 
 
 def p_pad(G, K=9):
@@ -243,7 +245,7 @@ def main():
                                   "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)}))
                 return
             sys.exit(f"--only-op {args.only_op}: no such shape")
-        for table, off in ((CFG2, 3.0), (CFG3, 4.0), (CFG5, 3.0), (DEVNOTE, 3.0)):
+        for table, off in ((CFG2, 3.0), (CFG3, 4.0), (CFG5, 3.0), (DEVNOTE, 3.0), (WIDE, 3.0)):
             for name, B, H, W, C, G in table:
                 if name != shape_name:
                     continue
@@ -322,8 +324,13 @@ def main():
             fb, bb = dcn_bytes(2, B, H, W, C, G)
             add("dcnv4_fwd", name, torch.float16, time_op(lambda: dcn_fwd(t, G, C), args.op_iters), fb)
             add("dcnv4_bwd", name, torch.float16, time_op(lambda: dcn_bwd(t, G, C), args.op_iters), bb)
+            if name == "L-dense1":
+                # robustness row: the same call with ONE sampling point of one pixel sent 200 pixels away (the backward
+                # keeps the common reach for all workgroups but the one that point lands in)
+                t[1][0, 10, 10, 0] = 200.0
+                add("dcnv4_bwd", name + " + one offset of 200 px", torch.float16, time_op(lambda: dcn_bwd(t, G, C), max(10, args.op_iters // 5)), bb)
             del t
-        for name, B, H, W, C, G in DEVNOTE:
+        for name, B, H, W, C, G in DEVNOTE + WIDE:
             t = dcn_inputs(B, H, W, C, G, torch.float16, 3.0)
             fb, bb = dcn_bytes(2, B, H, W, C, G)
             add("dcnv4_fwd", name, torch.float16, time_op(lambda: dcn_fwd(t, G, C), args.op_iters), fb)

@@ -17,8 +17,9 @@
 //     rounded to fp32, summed in fp32, the result rounded once to the tensor dtype;
 //   * the workgroup visits every output pixel whose reference point lies within the reach the
 //     data needs (GradState::reach_needed, written by the grad_offset_mask kernel that runs
-//     first; any value up to the whole image), in strips of interleaved rows, so that every
-//     strip spreads its points evenly over the tile.  Per strip:
+//     first: what the sampling points within the reach cap need; a tile that points beyond the
+//     cap land in reads its own, larger number from GradState::far_reach), in strips of
+//     interleaved rows, so that every strip spreads its points evenly over the tile.  Per strip:
 //       park   the strip's grad_out rows are copied to LDS;
 //       A      one lane per (group, pixel, kernel tap) recomputes the sampling position and links
 //              a 16-byte entry (m * hy, m * ly, lx, address of the pixel's parked grad_out | next)
@@ -93,7 +94,10 @@ __global__ void __launch_bounds__(NT) dcnv4_grad_value_kernel(const DcnLaunch p)
   // output pixels this tile visits: reference point (centre tap at zero offset) within `reach` of the tile
   const int half_w = (p.dw * (p.kw - 1)) >> 1, half_h = (p.dh * (p.kh - 1)) >> 1;
   const int cy0 = half_h - p.ph, cx0 = half_w - p.pw, Ho = p.Q / p.Wo;
-  const int reach = p.gv_whole ? (1 << 20) : (int)min(p.state->reach_needed, 1u << 20);
+  // the reach that the bulk of the sampling points needs, or - for a tile that points beyond the reach cap land in -
+  // how far away the output pixels of those points lie (GradState::far_reach): only such tiles pay for outliers
+  const int reach = p.gv_whole ? (1 << 20)
+                               : (int)min(max(p.state->reach_needed, p.state->far_reach[dcnv4_far_slot(b, ty, tx, nty, ntx, chunk, n_chunks)]), 1u << 20);
   const int ho_lo = max(0, ceil_div_signed(ty0 - reach - cy0, p.sh));
   const int ho_hi = min(Ho, ceil_div_signed(ty0 + eh + reach - cy0, p.sh));
   const int wo_lo_all = max(0, ceil_div_signed(tx0 - reach - cx0, p.sw));

@@ -181,7 +181,8 @@ __global__ void __launch_bounds__(kBlockThreads) dcnv4_offset_mask_grad_kernel(c
           const int y1 = t.y0 + (t.ly > 0.f ? 1 : 0), x1 = t.x0 + (t.lx > 0.f ? 1 : 0);
           const int d = max(max(p0y - max(t.y0, 0), min(y1, p.H - 1) - p0y),
                             max(p0x - max(t.x0, 0), min(x1, p.W - 1) - p0x));
-          reach_needed = max(reach_needed, (uint32_t)max(d, 0));
+          if ((float)d > p.gv_reach_cap) { if (chunk == 0) dcnv4_fold_far_point(p, pix / p.Q, g, t.y0, t.x0, p0y, p0x); }
+          else reach_needed = max(reach_needed, (uint32_t)max(d, 0));
         }
       }
       typename pack::raw_t raw[4];

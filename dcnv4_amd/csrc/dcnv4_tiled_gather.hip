@@ -555,7 +555,9 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
       far_mask |= (mask_t)(wt.inside && !wt.ok) << k;
       // Chebyshev distance of the point from the reference point; its ceiling is how far the weighted corners of
       // the 2x2 block lie from it at most (a point at an integer distance k has its far corners at weight 0)
-      if (wt.inside) reach_f = fmaxf(reach_f, fmaxf(fabsf(x - p0xf), fabsf(y - p0yf)));
+      // (points beyond the cap are not `ok` - the cap exceeds what any window covers - and are folded where they are served)
+      const float dist = fmaxf(fabsf(x - p0xf), fabsf(y - p0yf));
+      if (wt.inside && dist <= p.gv_reach_cap) reach_f = fmaxf(reach_f, dist);
       u32x4 raw[4][NV];
 #pragma unroll
       for (int cn = 0; cn < 4; ++cn) {
@@ -642,7 +644,8 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
       const int part_bytes = part * NV * 16;
       const WinTap wt = window_tap(y, x, p.H, p.W, t, cell_stride, lane_bytes - part_bytes, zero_base);
       const int far_own = wt.inside && !wt.ok;
-      if (wt.inside) reach_f = fmaxf(reach_f, fmaxf(fabsf(x - p0xf), fabsf(y - p0yf)));
+      const float dist = fmaxf(fabsf(x - p0xf), fabsf(y - p0yf));
+      if (wt.inside && dist <= p.gv_reach_cap) reach_f = fmaxf(reach_f, dist);
       far_mask |= ((mask_t)pair_pick<0>(far_own) << k0) | ((mask_t)pair_pick<1>(far_own) << (k0 + 1));
       float d0[4], d1[4], d[4];
       window_dots(pair_pick<0>(wt.addr) + part_bytes, d0);
@@ -663,6 +666,8 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
       const float y = add_rn(y_base, mul_rn(add_rn((float)(j * p.dh), lds_elem<Tag>(om_g, 2 * k + 1)), p.offset_scale));
       const float m = lds_elem<Tag>(om_g, 2 * Kp + k);
       const Tap tp = make_tap(y, x, p.H, p.W, img_base, pix_bytes);
+      // beyond the reach cap: left out of the reach statistic above, folded per destination tile instead
+      if (tp.valid != 0 && fmaxf(fabsf(x - p0xf), fabsf(y - p0yf)) > p.gv_reach_cap) dcnv4_fold_far_point(p, t.b, t.g0 + gl, tp.y0, tp.x0, p0y, p0x);
       float d[4];
 #pragma unroll
       for (int cn = 0; cn < 4; ++cn) {

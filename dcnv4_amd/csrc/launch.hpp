@@ -18,13 +18,20 @@ constexpr int kBlockThreads = 256;
 constexpr size_t kMaxDynamicLds = 64 * 1024;      // without raising the per-kernel limit
 constexpr size_t kMaxLdsPerWorkgroup = 160 * 1024;  // gfx950
 
-// Device-side scratch word block shared by the kernels of one backward call (16 bytes).
+// Device-side scratch word block shared by the kernels of one backward call (256 bytes).
+constexpr int kFarSlots = 56;
 struct GradState {
   uint32_t unused0;
   uint32_t unused1;
-  uint32_t reach_needed;   // DCNv4: ceiling of the largest Chebyshev distance (pixels) of an in-range sampling point from its output pixel's reference point
+  uint32_t reach_needed;   // DCNv4: ceiling of the largest Chebyshev distance (pixels) of an in-range sampling point from its output pixel's reference point, over the points within the reach cap
   uint32_t reserved;       // attention backward: set when a level has more tiles than the binning kernel can count
+  uint32_t pad[4];
+  // DCNv4: for the sampling points beyond the reach cap, per workgroup of the grad_value kernel (tile and chunk of
+  // groups; they share the slots round-robin): how far from the tile the output pixels lie whose points land in it; 0: none.
+  // Only the workgroups an outlier lands in pay for it.
+  uint32_t far_reach[kFarSlots];
 };
+static_assert(sizeof(GradState) == 256, "GradState fills the state block");
 
 // Dynamic LDS above 64 KB needs hipFuncAttributeMaxDynamicSharedMemorySize on the kernel, on every device that runs
 // it (the reference sets it on every launch, DCNv4_op/src/cuda/dcnv4_col2im_cuda.cuh:454).  Set once per (kernel,
@@ -86,7 +93,34 @@ struct DcnLaunch {
   int gt_pad;               // bytes between the cells of the staged window (16: fewer LDS bank conflicts; 0: a larger window fits)
   int gt_wh, gt_ww;         // largest input window (rows, columns of cells) a tile stages
   int gt_reach;             // input pixels around an output pixel's reference point that the window covers
+  float gv_reach_cap;       // sampling points farther than this from their reference point stay out of reach_needed and are folded into GradState::far_reach
 };
+
+// Slot of GradState::far_reach that the workgroup of the grad_value kernel for (image within its launch, tile, chunk of
+// groups) uses.
+__host__ __device__ inline uint32_t dcnv4_far_slot(int img, int ty, int tx, int nty, int ntx, int chunk, int n_chunks) {
+  return (uint32_t)(((img * nty + ty) * ntx + tx) * n_chunks + chunk) % (uint32_t)kFarSlots;
+}
+// A sampling point beyond the reach cap, of group g, with first corner (y0, x0), of an output pixel of image `img` whose
+// reference point is (p0y, p0x): for every grad_value tile one of its in-image corners lands in, records how far outside
+// the tile the pixel lies (the condition under which the tile's workgroup for that group visits a pixel,
+// dcnv4_grad_value.hip).  Rare path: straight to memory.
+__device__ inline void dcnv4_fold_far_point(const DcnLaunch &p, int img, int g, int y0, int x0, int p0y, int p0x) {
+  const int nty = (p.H + p.tile_h - 1) / p.tile_h, ntx = (p.W + p.tile_w - 1) / p.tile_w;
+  const int n_chunks = (p.G + p.ng_chunk - 1) / p.ng_chunk, chunk = g / p.ng_chunk;
+  for (int c = 0; c < 4; ++c) {
+    const int cy = y0 + (c >> 1), cx = x0 + (c & 1);
+    if ((unsigned)cy >= (unsigned)p.H || (unsigned)cx >= (unsigned)p.W) continue;
+    const int ty = cy / p.tile_h, tx = cx / p.tile_w;
+    const int ty0 = ty * p.tile_h, tx0 = tx * p.tile_w;
+    const int b = max(max(ty0 - p0y, p0y - (ty0 + p.tile_h - 1)), max(tx0 - p0x, p0x - (tx0 + p.tile_w - 1)));
+    if (b > 0) atomicMax(&p.state->far_reach[dcnv4_far_slot(img, ty, tx, nty, ntx, chunk, n_chunks)], (uint32_t)min(b, 1 << 20));
+  }
+}
+
+// Lower bound of the reach cap: the statistic in reach_needed then stays at what the bulk of the sampling points needs
+// when a few offsets are outliers.
+constexpr int kReachCap = 16;
 
 // Work items a lane of the tiled grad_value kernel handles per strip, at most.  An item is one sampling point, or -
 // for a 3x3 kernel - a column of the kernel: three points of one (pixel, group), the removed centre included.

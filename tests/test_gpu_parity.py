@@ -35,6 +35,8 @@ DCN_CASES = {
     "d6_three_lane_cluster": (2, 6, 5, 3, 6, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
     "d48_six_lane_cluster": (1, 8, 8, 2, 48, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
     "d64": (1, 8, 9, 2, 64, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
+    # groups of 64 channels as in a third of the reference's tuned keys (DCNv4_op/DCNv4/functions/table.py:452-461), several tiles
+    "d64_g4_20x18": (2, 20, 18, 4, 64, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 3.0),
     # four lanes of 32 channels per (cell, group) in the tiled grad_value kernel, the last one partly idle
     "d104_four_lanes_per_slot": (1, 9, 7, 2, 104, (3, 3, 1, 1, 1, 1, 1, 1), 0, 1.0, 2.0),
     # the widest group the fp32 backward takes: 64 gather lanes, eight lanes of 32 channels per (cell, group)
@@ -104,7 +106,7 @@ KERNEL_PATHS = {
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
 @pytest.mark.parametrize("path", list(KERNEL_PATHS))
 @pytest.mark.parametrize("name", ["cfg1_56x56_c64_g4", "g7_c112_scale_half", "remove_center", "stride2", "dilation2_pad2",
-                                  "kernel_5x5", "far_offsets_mostly_outside", "wide_g80"])
+                                  "kernel_5x5", "far_offsets_mostly_outside", "wide_g80", "d64_g4_20x18"])
 def test_dcnv4_every_kernel_path_matches_oracle(oracle, name, path, dtype):
     from dcnv4_amd import ext
     v, om, go, (geom, G, D, scale, rc) = _dcn_inputs(DCN_CASES[name], dtype, seed=zlib.crc32((name + path).encode()) % 1000)

@@ -135,6 +135,14 @@ def _magnitude_sum_dcn(oracle, v, om, go, G, D, scale, K=9):
     return mag
 
 
+def _magnitude_sum_dcn_geom(oracle, v, om, go, geom, G, D, scale, K=9):
+    om_abs = cabi.f64(om).copy()
+    body = om_abs[..., : G * K * 3].reshape(*om_abs.shape[:3], G, K * 3)
+    body[..., 2 * K:] = np.abs(body[..., 2 * K:])
+    mag, _ = oracle.dcnv4_backward(cabi.f64(v), om_abs, np.abs(cabi.f64(go)), *geom, G, D, scale, 0, coord_f32=True)
+    return mag
+
+
 def _assert_accumulated_like_fp32(got, want, mag, dtype, what):
     """|got - want| <= one generous rounding of the result in the tensor dtype + 2^-14 of the sum of magnitudes."""
     eps = {torch.float32: 2.0 ** -20, torch.float16: 2.0 ** -9, torch.bfloat16: 2.0 ** -6}[dtype]
@@ -216,6 +224,35 @@ def test_dcnv4_far_offsets_at_image_scale_keep_the_stated_tolerance(oracle, dtyp
     gv, gom = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), GEOM3, G, D, 2.0)
     torch.cuda.synchronize()
     cabi.assert_close(out, want, *FWD_TOL[dtype], what="output")
+    _assert_accumulated_like_fp32(gv, wgv, mag, dtype, "grad_value")
+    cabi.assert_close(gom, wgom, *GRAD_TOL[dtype], what="grad_offset_mask")
+
+
+@pytest.mark.parametrize("gather", ["tiled", "direct"])
+@pytest.mark.parametrize("geom", [GEOM3, (3, 3, 2, 2, 1, 1, 1, 1)], ids=["stride1", "stride2"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32], ids=["fp16", "bf16", "fp32"])
+def test_dcnv4_backward_with_a_few_outlier_offsets(oracle, dtype, geom, gather):
+    """Offsets U(-2, 2) on a 72x40 image (six grad_value tiles) except for a handful of sampling points sent 20 to 70
+    pixels away - into other tiles, onto the image's far corner, outside the image: the backward keeps the reach of
+    the bulk for all tiles and lets only the tiles such a point lands in look further; every gradient must come out
+    as if nothing were special, summed in fp32."""
+    from dcnv4_amd import ext
+    B, H, W, G, D, K = 2, 72, 40, 2, 16, 9
+    v, om, go = make_dcnv4_inputs(B, H, W, G, D, *geom, offset_range=2.0, seed=31, dtype=torch.float32)
+    Ho, Wo = om.shape[1:3]
+    body = om[..., : G * K * 3].reshape(B, Ho, Wo, G, K * 3)
+    far = [  # image, output row, output column, group, tap, x offset, y offset
+        (0, 2, 1, 0, 4, 30.0, 50.0), (0, Ho - 1, Wo - 1, 1, 0, -35.0, -66.0), (1, Ho // 2, 2, 0, 8, 33.25, -0.5),
+        (1, 1, Wo // 2, 1, 3, 0.5, 60.75), (0, 3, 3, 1, 7, 300.0, 5.0), (1, Ho - 2, 1, 0, 2, 25.5, -40.5), (0, Ho // 2, Wo // 2, 0, 5, -17.5, 21.0)]
+    for b, r, c, g, k, dx, dy in far:
+        body[b, r, c, g, 2 * k], body[b, r, c, g, 2 * k + 1] = dx, dy
+    v, om, go = v.to(dtype), om.to(dtype), go.to(dtype)
+    print(f"outlier offsets {dtype} {geom} {gather}", flush=True)
+    wgv, wgom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *geom, G, D, 1.0, 0, coord_f32=True)
+    mag = _magnitude_sum_dcn_geom(oracle, v, om, go, geom, G, D, 1.0)
+    with ext.launch_options(gather=gather):
+        gv, gom = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), geom, G, D, 1.0)
+    torch.cuda.synchronize()
     _assert_accumulated_like_fp32(gv, wgv, mag, dtype, "grad_value")
     cabi.assert_close(gom, wgom, *GRAD_TOL[dtype], what="grad_offset_mask")
 
