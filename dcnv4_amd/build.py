@@ -13,9 +13,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "libdcnv4_gfx950.so")
-SOURCES = ["capi.hip", "dcnv4_kernels.hip", "dcnv4_tiled_gather.hip", "dcnv4_grad_value.hip", "fda_kernels.hip", "fda_grad_value.hip",
+SOURCES = ["capi.hip", "dcnv4_kernels.hip", "dcnv4_tiled_gather.hip", "dcnv4_grad_value.hip", "dcnv4_backward_dual.hip", "fda_kernels.hip", "fda_grad_value.hip",
            "depthwise_conv.hip", "layer_norm.hip", "center_feature.hip"]
-HEADERS = [os.path.join(CSRC, "common.hpp"), os.path.join(CSRC, "launch.hpp"),
+HEADERS = [os.path.join(CSRC, "common.hpp"), os.path.join(CSRC, "launch.hpp"), os.path.join(CSRC, "dcnv4_tiled_gather.hpp"), os.path.join(CSRC, "dcnv4_grad_value.hpp"),
            os.path.join(os.path.dirname(HERE), "include", "dcnv4_gfx950.h")]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -166,6 +166,7 @@ struct LaunchOptions {
   int tile = 0;                // largest side of a grad_value tile (8, 16, 32); 0: default
   int gather_tile = 0;         // largest side of an output tile of the tiled gathers (4, 8, 16); 0: default (16)
   int gv_threads = 0;          // lanes per workgroup of the grad_value kernel (512, 1024); 0: default
+  int dual = kOptAuto;         // DCNv4 backward whose grad_value tiles are whole images: 1 / auto one launch with two workgroup roles, 2 two launches
   int fda_order = kOptAuto;    // attention forward: 1 whole query rows per workgroup, 2 one head per workgroup
   int fda_stage = kOptAuto;    // attention forward: 1 stage the smallest levels of a head in LDS, 2 never
 };
@@ -618,6 +619,7 @@ static int *launch_option_slot(const char *name) {
   if (std::strcmp(name, "tile") == 0) return &g_opt.tile;
   if (std::strcmp(name, "gather_tile") == 0) return &g_opt.gather_tile;
   if (std::strcmp(name, "gv_threads") == 0) return &g_opt.gv_threads;
+  if (std::strcmp(name, "dual") == 0) return &g_opt.dual;
   if (std::strcmp(name, "fda_order") == 0) return &g_opt.fda_order;
   if (std::strcmp(name, "fda_stage") == 0) return &g_opt.fda_stage;
   return nullptr;
@@ -727,7 +729,9 @@ static int dcn_backward_impl(const void *value, const void *offset_mask, const v
     if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);
   }
   const int per = images_per_launch(pr, false);
-  for (int pass = 0; pass < 2; ++pass) {
+  // both kernels in one launch when they do not depend on each other and the shape suits the two-role kernel
+  const bool dual = g_opt.dual != kOptPlain && dcnv4_backward_dual_fits(base, pr.s, std::min(per, batch), g_opt.dual == kOptTiled ? (1 << 20) : kCusPerDevice);
+  for (int pass = 0; pass < (dual ? 1 : 2); ++pass) {
     for (int b0 = 0; b0 < batch; b0 += per) {
       const int nb = std::min(per, batch - b0);
       DcnLaunch L = base;
@@ -740,7 +744,8 @@ static int dcn_backward_impl(const void *value, const void *offset_mask, const v
       L.n_pix = nb * L.Q;
       L.n_img = nb;
       hipError_t e = hipSuccess;
-      if (pass == 0 && gather_tiled) e = launch_dcnv4_offset_mask_grad_tiled(dtype, L, st);
+      if (dual) e = launch_dcnv4_backward_dual(dtype, L, st);
+      else if (pass == 0 && gather_tiled) e = launch_dcnv4_offset_mask_grad_tiled(dtype, L, st);
       else if (pass == 0) e = launch_dcnv4_offset_mask_grad(dtype, L, st);
       else e = launch_dcnv4_grad_value(dtype, L, st);
       if (e) return hip_fail("dcnv4 backward launch", e);
@@ -941,9 +946,13 @@ static int fda_backward_impl(const void *value, const int64_t *spatial_shapes, c
     base.regions = reinterpret_cast<uint32_t *>(ws + sc.regions);
     base.n_chunks = sc.n_chunks;
     base.tile_stride = sc.tile_stride;
-    hipLaunchKernelGGL(init_state_kernel, dim3(1), dim3(64), 0, st, base.state);
-    if (hipError_t e = hipGetLastError()) return hip_fail("state init launch", e);
-    for (int pass = 0; pass < 3; ++pass) {
+    // The state block (the binning kernel's flag) is cleared by the first kernel itself, which runs to its end
+    // before the binning kernel starts.  The fallback - three launches that return at once without the flag - can
+    // only be needed when a level has more tiles than the binning kernel counts (kFdaMaxTilesPerLevel); tiles have
+    // at least 8 cells (a level of up to four rows is cut into 1 x 8 pieces), so a tensor of fewer cells than that
+    // many tiles' worth cannot raise the flag and the launches are left out.
+    const bool fallback_possible = (size_t)spatial_size / 8 + 64 > (size_t)kFdaMaxTilesPerLevel;
+    for (int pass = 0; pass < (fallback_possible ? 3 : 2); ++pass) {
       for (int b0 = 0; b0 < batch; b0 += per) {
         const int nb = std::min(per, batch - b0);
         FdaLaunch F = base;
@@ -961,6 +970,7 @@ static int fda_backward_impl(const void *value, const int64_t *spatial_shapes, c
         F.n_img = nb;
         hipError_t e = hipSuccess;
         if (pass == 0) fda_choose_order(&F, pr, spatial_size, num_heads, head_channels, num_levels, num_points, true);
+        F.clear_state = (pass == 0 && b0 == 0) ? 1 : 0;
         if (pass == 0) e = launch_fda_backward(dtype, F, kFdaNoScatter, st);
         else if (pass == 1) e = launch_fda_grad_value(dtype, F, st);
         else {

@@ -563,6 +563,12 @@ __global__ void __launch_bounds__(kFdaBackwardThreads) fda_backward_kernel(const
   if constexpr (MODE == kFdaFallback) {
     if (p.state->reserved == 0u) return;
   }
+  if constexpr (MODE == kFdaNoScatter) {
+    // the first kernel of the tiled backward clears the state block for the kernels behind it (nobody reads it before
+    // this kernel has ended); with several launches per call only the first one does
+    if (p.clear_state && blockIdx.x == 0 && threadIdx.x < sizeof(GradState) / sizeof(uint32_t))
+      reinterpret_cast<uint32_t *>(p.state)[threadIdx.x] = 0u;
+  }
   const int LK = p.L * p.K, row_len = 3 * LK;
   const uint32_t blk = xcd_contiguous_block(blockIdx.x, gridDim.x);
   int row0, nrow, heads_here = p.G, g_fixed = 0;

@@ -161,6 +161,7 @@ struct FdaLaunch {
   // tiled grad_value path
   void *grad_value;         // [n_img, N, G, D] in the tensor dtype
   GradState *state;         // `reserved` only
+  int clear_state;          // first kernel of the tiled backward: clear the state block
   uint16_t *keys;           // [n_img, G, L, QKp] one key per sampling point (QKp = Q*K rounded up to even)
   f32x4_t *recs;            // same layout: (x, y, softmax probability, 0) of the point, x and y in cells of its level
   void *go_rows;            // [n_img, G, Q, D] grad_out regrouped by head, tensor dtype: a head's rows lie densely
@@ -252,6 +253,10 @@ hipError_t launch_depthwise_grad_weight_reduce(int dtype, const DwLaunch &p, hip
 hipError_t launch_dcnv4_forward(int dtype, const DcnLaunch &p, hipStream_t stream);
 hipError_t launch_dcnv4_offset_mask_grad(int dtype, const DcnLaunch &p, hipStream_t stream);
 hipError_t launch_dcnv4_grad_value(int dtype, const DcnLaunch &p, hipStream_t stream);
+// Both kernels of the backward as one launch with two workgroup roles, for shapes whose grad_value tiles are whole images
+// (dcnv4_backward_dual.hip).
+bool dcnv4_backward_dual_fits(const DcnLaunch &p, int elem_bytes, int n_img, int n_cus);
+hipError_t launch_dcnv4_backward_dual(int dtype, const DcnLaunch &p, hipStream_t stream);
 // Entry slots of the tiled grad_value kernel per (pixel, group) of a strip, and at most per strip: three-point items
 // for a 3x3 kernel (nine slots, also when the centre is removed), else an item per sampling point.
 inline bool dcnv4_grad_value_columns(const DcnLaunch &p) { return p.kh == 3 && p.kw == 3; }

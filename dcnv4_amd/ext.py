@@ -31,8 +31,31 @@ def _check(t, name, dtype=None):
         raise RuntimeError(f"{name} has dtype {t.dtype}, expected {dtype}")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    # the raw handle of torch's current stream on the current device (the direct binding costs a tenth of a
+    # microsecond, going through the Stream object three: the small stages' calls are bound by host time)
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
+
+
+class _on_device:
+    """`with torch.cuda.device(d)` for the common case that d is the current device already: nothing to switch."""
+
+    def __init__(self, device):
+        self.ctx = None if device.index is None or device.index == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            return self.ctx.__exit__(*exc)
+        return False
 
 
 def _hint(v):
@@ -47,13 +70,13 @@ _ORDER = {"auto": 0, "rows": 1, "heads": 2}
 class launch_options:
     """Context manager over the calling thread's launch options (include/dcnv4_gfx950.h,
     ``dcnv4_gfx950_set_launch_option``): ``gather`` in auto / tiled / direct, ``scatter`` in auto / tiled / atomic,
-    ``reach`` an int or None, ``tile`` 8 / 16 / 32 or None, ``gather_tile`` 4 / 8 / 16 or None, ``gv_threads`` 512 / 1024 or None, ``fda_order`` in auto / rows / heads, ``fda_stage`` in auto / on / off.  Used by the tuner,
+    ``reach`` an int or None, ``tile`` 8 / 16 / 32 or None, ``gather_tile`` 4 / 8 / 16 or None, ``gv_threads`` 512 / 1024 or None, ``dual`` in auto / on / off, ``fda_order`` in auto / rows / heads, ``fda_stage`` in auto / on / off.  Used by the tuner,
     by dispatch-table entries that carry options and by tests that force a kernel family; on exit every option is
     back at the value it had on entry, so contexts nest.  Results do not depend on the options beyond the rounding
     of sums."""
 
     def __init__(self, gather=None, scatter=None, reach=None, tile=None, fda_order=None, gather_tile=None, gv_threads=None,
-                 fda_stage=None):
+                 fda_stage=None, dual=None):
         self.values = {}
         if gather is not None:
             self.values["gather"] = _FAMILY[gather]
@@ -67,6 +90,8 @@ class launch_options:
             self.values["gather_tile"] = int(gather_tile)
         if gv_threads is not None:
             self.values["gv_threads"] = int(gv_threads)
+        if dual is not None:
+            self.values["dual"] = {"auto": 0, "on": 1, "off": 2}[dual]
         if fda_order is not None:
             self.values["fda_order"] = _ORDER[fda_order]
         if fda_stage is not None:
@@ -108,7 +133,7 @@ def dcnv4_forward(value, p_offset, kernel_h, kernel_w, stride_h, stride_w, pad_h
     ho, wo = _out_hw(h, w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w)
     if tuple(p_offset.shape[:3]) != (batch, ho, wo):
         raise RuntimeError(f"offset_mask shape {tuple(p_offset.shape)} does not match output ({batch}, {ho}, {wo}, *)")
-    with torch.cuda.device(value.device):
+    with _on_device(value.device):
         output = torch.empty((batch, ho, wo, channels), dtype=value.dtype, device=value.device)
         _lib.check(_L.dcnv4_gfx950_forward(
             value.data_ptr(), p_offset.data_ptr(), output.data_ptr(), code, batch, h, w, group, group_channels,
@@ -133,7 +158,7 @@ def dcnv4_backward(value, p_offset, kernel_h, kernel_w, stride_h, stride_w, pad_
     ho, wo = _out_hw(h, w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w)
     if tuple(p_offset.shape[:3]) != (batch, ho, wo) or grad_output.numel() != batch * ho * wo * channels:
         raise RuntimeError("offset_mask / grad_output shapes do not match the output extent")
-    with torch.cuda.device(value.device):
+    with _on_device(value.device):
         grad_input = torch.empty_like(value)
         grad_offset = torch.empty_like(p_offset)
         ws_bytes = _L.dcnv4_gfx950_backward_workspace_bytes(code, batch, h, w, group, group_channels)
@@ -170,7 +195,7 @@ def flash_deform_attn_forward(value, spatial_shapes, level_start_index, sampling
     batch, spatial_size, num_heads, channels, num_levels, num_query = _fda_common(
         value, spatial_shapes, level_start_index, sampling_loc_attn, K)
     code = _dtype_code(value, "value")
-    with torch.cuda.device(value.device):
+    with _on_device(value.device):
         output = torch.empty((batch, num_query, num_heads * channels), dtype=value.dtype, device=value.device)
         _lib.check(_L.flash_deform_attn_gfx950_forward(
             value.data_ptr(), spatial_shapes.data_ptr(), level_start_index.data_ptr(), sampling_loc_attn.data_ptr(),
@@ -187,7 +212,7 @@ def flash_deform_attn_backward(value, spatial_shapes, level_start_index, samplin
     if grad_output.numel() != batch * num_query * num_heads * channels:
         raise RuntimeError("grad_output shape does not match the output")
     code = _dtype_code(value, "value")
-    with torch.cuda.device(value.device):
+    with _on_device(value.device):
         grad_value = torch.empty_like(value)
         grad_sla = torch.empty_like(sampling_loc_attn)
         ws_bytes = _L.flash_deform_attn_gfx950_backward_workspace_bytes(code, batch, spatial_size, num_heads, channels,
@@ -219,7 +244,7 @@ def depthwise_conv_forward(input, weight, bias, pad):
     if bias is not None and bias.numel() != channels:
         raise RuntimeError(f"bias has {bias.numel()} elements for {channels} channels")
     ho, wo = h + 2 * pad - k + 1, w + 2 * pad - k + 1
-    with torch.cuda.device(input.device):
+    with _on_device(input.device):
         output = torch.empty((batch, max(ho, 0), max(wo, 0), channels), dtype=input.dtype, device=input.device)
         _lib.check(_L.dcnv4_gfx950_depthwise_conv_forward(
             input.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None, output.data_ptr(),
@@ -240,7 +265,7 @@ def depthwise_conv_backward(input, weight, grad_output, pad, has_bias=True, need
     ho, wo = h + 2 * pad - k + 1, w + 2 * pad - k + 1
     if tuple(grad_output.shape) != (batch, ho, wo, channels):
         raise RuntimeError(f"grad_output shape {tuple(grad_output.shape)} does not match the output {(batch, ho, wo, channels)}")
-    with torch.cuda.device(input.device):
+    with _on_device(input.device):
         grad_input = torch.empty_like(input) if need_input_grad else None
         grad_weight = torch.empty_like(weight) if need_weight_grad else None
         grad_bias = torch.empty(channels, dtype=input.dtype, device=input.device) if (need_weight_grad and has_bias) else None
@@ -270,7 +295,7 @@ def layer_norm_residual_forward(input, residual, weight, bias, gamma, eps):
     channels = input.shape[-1]
     if weight.numel() != channels or bias.numel() != channels or (gamma is not None and gamma.numel() != channels):
         raise RuntimeError(f"weight, bias and gamma must have {channels} elements")
-    with torch.cuda.device(input.device):
+    with _on_device(input.device):
         output = torch.empty_like(input)
         if input.numel():
             _lib.check(_L.dcnv4_gfx950_layer_norm_residual_forward(
@@ -298,7 +323,7 @@ def layer_norm_residual_backward(grad_output, input, weight, bias, gamma, eps, n
     code = _dtype_code(input, "input")
     channels = input.shape[-1]
     rows = input.numel() // max(channels, 1)
-    with torch.cuda.device(input.device):
+    with _on_device(input.device):
         grad_input = torch.empty_like(input)
         new = lambda: torch.empty(channels, dtype=input.dtype, device=input.device)
         grad_weight = new() if need_param_grads else None
@@ -338,7 +363,7 @@ def center_feature_blend_forward(sampled, projected, weight, bias):
     group), every channel using its group's gate (DCNv4_op/DCNv4/modules/dcnv4.py:142-147) in one kernel."""
     code, rows, channels, groups = _blend_common(sampled, projected, weight, bias)
     weight = _aligned16(weight)
-    with torch.cuda.device(sampled.device):
+    with _on_device(sampled.device):
         output = torch.empty_like(sampled)
         if sampled.numel():
             _lib.check(_L.dcnv4_gfx950_center_feature_blend_forward(
@@ -355,7 +380,7 @@ def center_feature_blend_backward(grad_output, sampled, projected, weight, bias)
     _check(grad_output, "grad_output", sampled.dtype)
     if grad_output.shape != sampled.shape:
         raise RuntimeError("grad_output must have the shape of sampled")
-    with torch.cuda.device(sampled.device):
+    with _on_device(sampled.device):
         grad_sampled, grad_projected = torch.empty_like(sampled), torch.empty_like(sampled)
         grad_logits = torch.empty((rows, groups), dtype=torch.float32, device=sampled.device)
         if sampled.numel():
@@ -396,7 +421,7 @@ def flash_deform_attn_forward_split(value, spatial_shapes, level_start_index, sa
     batch, spatial_size, num_heads, channels, num_levels, num_query = _fda_split_common(
         value, spatial_shapes, level_start_index, sampling_locations, attention_logits, K)
     code = _dtype_code(value, "value")
-    with torch.cuda.device(value.device):
+    with _on_device(value.device):
         output = torch.empty((batch, num_query, num_heads * channels), dtype=value.dtype, device=value.device)
         _lib.check(_L.flash_deform_attn_gfx950_forward_split(
             value.data_ptr(), spatial_shapes.data_ptr(), level_start_index.data_ptr(), sampling_locations.data_ptr(),
@@ -415,7 +440,7 @@ def flash_deform_attn_backward_split(value, spatial_shapes, level_start_index, s
     if grad_output.numel() != batch * num_query * num_heads * channels:
         raise RuntimeError("grad_output shape does not match the output")
     code = _dtype_code(value, "value")
-    with torch.cuda.device(value.device):
+    with _on_device(value.device):
         grad_value = torch.empty_like(value)
         grad_loc = torch.empty_like(sampling_locations)
         grad_logits = torch.empty_like(attention_logits)
@@ -439,6 +464,6 @@ def stream_copy(src, dst):
     nbytes = src.numel() * src.element_size()
     if nbytes != dst.numel() * dst.element_size():
         raise RuntimeError("src and dst differ in size")
-    with torch.cuda.device(src.device):
+    with _on_device(src.device):
         _lib.check(_L.dcnv4_gfx950_stream_copy(src.data_ptr(), dst.data_ptr(), nbytes, _stream()))
     return dst

@@ -33,7 +33,7 @@ def _load_table(path=TABLE_PATH):
 
 
 # key -> {"d_stride": int, "n_thread": int, and optionally "gather": str, "tile": int, "reach": int}
-OPTION_KEYS = ("gather", "scatter", "tile", "reach", "gather_tile", "gv_threads", "fda_order", "fda_stage")
+OPTION_KEYS = ("gather", "scatter", "tile", "reach", "gather_tile", "gv_threads", "dual", "fda_order", "fda_stage")
 GFX950_TABLE = _load_table()
 
 

@@ -68,6 +68,8 @@ const char *dcnv4_gfx950_last_error(void);
  *   "fda_stage"  0 library's choice, 1 stage the smallest levels of one head's value slice in LDS whenever the
  *                one-head-per-workgroup order is used, 2 never (flash deformable attention forward)
  *   "gv_threads" 0 library's choice, else 512 or 1024: lanes per workgroup of the DCNv4 grad_value kernel
+ *   "dual"       DCNv4 backward on images small enough to be one grad_value tile: 0 / 1 both kernels as one launch with
+ *                two workgroup roles when the shape suits it, 2 always two launches
  * dcnv4_gfx950_get_launch_option reads a value back, so that a caller can restore what it found.
  */
 int dcnv4_gfx950_set_launch_option(const char *name, int value);

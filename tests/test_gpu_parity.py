@@ -100,13 +100,17 @@ KERNEL_PATHS = {
     "gather_tile8": dict(gather_tile=8),
     "gather_tile8_reach2": dict(gather_tile=8, reach=2),
     "gather_tile4_gv512": dict(gather_tile=4, gv_threads=512),
+    # images that are one grad_value tile: both backward kernels as one launch with two workgroup roles, or as two launches
+    "dual_on": dict(dual="on", gv_threads=512),
+    "dual_off": dict(dual="off"),
 }
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
 @pytest.mark.parametrize("path", list(KERNEL_PATHS))
 @pytest.mark.parametrize("name", ["cfg1_56x56_c64_g4", "g7_c112_scale_half", "remove_center", "stride2", "dilation2_pad2",
-                                  "kernel_5x5", "far_offsets_mostly_outside", "wide_g80", "d64_g4_20x18"])
+                                  "kernel_5x5", "far_offsets_mostly_outside", "wide_g80", "d64_g4_20x18", "stage_7x7_c512_g32",
+                                  "stage_28x28_c128_g8"])
 def test_dcnv4_every_kernel_path_matches_oracle(oracle, name, path, dtype):
     from dcnv4_amd import ext
     v, om, go, (geom, G, D, scale, rc) = _dcn_inputs(DCN_CASES[name], dtype, seed=zlib.crc32((name + path).encode()) % 1000)

@@ -213,6 +213,8 @@ def test_launch_options_are_validated_without_a_gpu():
     assert lib.dcnv4_gfx950_set_launch_option(b"gather_tile", 5) == _lib.ERR_INVALID_ARGUMENT
     assert lib.dcnv4_gfx950_set_launch_option(b"gv_threads", 512) == 0 and lib.dcnv4_gfx950_set_launch_option(b"gv_threads", 0) == 0
     assert lib.dcnv4_gfx950_set_launch_option(b"gv_threads", 256) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.dcnv4_gfx950_set_launch_option(b"dual", 2) == 0 and lib.dcnv4_gfx950_set_launch_option(b"dual", 0) == 0
+    assert lib.dcnv4_gfx950_set_launch_option(b"dual", 3) == _lib.ERR_INVALID_ARGUMENT
     assert lib.dcnv4_gfx950_set_launch_option(b"gather", 5) == _lib.ERR_INVALID_ARGUMENT
     assert lib.dcnv4_gfx950_set_launch_option(b"nonsense", 1) == _lib.ERR_INVALID_ARGUMENT
     assert b"nonsense" in lib.dcnv4_gfx950_last_error()
