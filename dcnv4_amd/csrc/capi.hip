@@ -730,7 +730,8 @@ static int dcn_backward_impl(const void *value, const void *offset_mask, const v
   }
   const int per = images_per_launch(pr, false);
   // both kernels in one launch when they do not depend on each other and the shape suits the two-role kernel
-  const bool dual = g_opt.dual != kOptPlain && dcnv4_backward_dual_fits(base, pr.s, std::min(per, batch), g_opt.dual == kOptTiled ? (1 << 20) : kCusPerDevice);
+  const bool dual = g_opt.dual != kOptPlain && dcnv4_backward_dual_fits(base, pr.s);
+  if (dual) base.dual_interleave = dcnv4_backward_dual_workgroups(base, std::min(per, batch)) <= 3u * kCusPerDevice ? 1 : 0;
   for (int pass = 0; pass < (dual ? 1 : 2); ++pass) {
     for (int b0 = 0; b0 < batch; b0 += per) {
       const int nb = std::min(per, batch - b0);

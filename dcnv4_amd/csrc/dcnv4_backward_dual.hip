@@ -5,9 +5,11 @@
 // other: the grad_value workgroups visit every output pixel whatever the reach the first kernel measures.  On the
 // small stages (14x14, 7x7 images: a few hundred workgroups, 15-20 us per kernel of which a quarter is the fixed cost
 // of a dispatch) the two launches run back to back with the chip half empty.  Here both kinds of workgroup share one
-// grid: every dispatch slot of 16 consecutive workgroup ids holds 8 workgroups of each role, so that both roles are
-// resident on every CU at once and a role's k-th workgroup still runs on XCD k % 8 (the order both bodies assume for
-// their L2 locality).  The bodies are the kernels' own, unchanged: identical bits.
+// grid: when it is small enough to be resident at once, every 16 consecutive workgroup ids hold 8 workgroups of each
+// role, so that both roles are on every CU together and a role's k-th workgroup still runs on XCD k % 8 (the order
+// both bodies assume for their L2 locality); a larger grid holds one role after the other, which still saves a
+// dispatch and lets the second role start while the first one's last workgroups finish.  The bodies are the kernels'
+// own, unchanged: identical bits.
 // Reference for the two roles: DCNv4_op/src/cuda/dcnv4_col2im_cuda.cuh:196-366 (one kernel there, with atomics).
 #include "dcnv4_grad_value.hpp"
 #include "dcnv4_tiled_gather.hpp"
@@ -18,8 +20,8 @@ namespace {
 constexpr int kDualThreads = 512;
 
 // Role and number within its role of workgroup `bid`: n1 workgroups of the first role, n2 of the second.
-__device__ __forceinline__ bool dual_first_role(uint32_t bid, uint32_t n1, uint32_t n2, uint32_t &local) {
-  const uint32_t m = min(n1, n2) & ~7u;           // interleaved in eights while both roles last
+__device__ __forceinline__ bool dual_first_role(uint32_t bid, uint32_t n1, uint32_t n2, uint32_t &local, bool interleave) {
+  const uint32_t m = interleave ? min(n1, n2) & ~7u : 0u;           // interleaved in eights while both roles last
   if (bid < 2u * m) {
     const uint32_t r = bid & 15u;
     local = (bid >> 4) * 8u + (r & 7u);
@@ -32,9 +34,9 @@ __device__ __forceinline__ bool dual_first_role(uint32_t bid, uint32_t n1, uint3
 }
 
 template <typename Tag, int NV, bool PAIR>
-__global__ void __launch_bounds__(kDualThreads, 4) dcnv4_backward_dual_kernel(const DcnLaunch p, uint32_t n1, uint32_t n2) {
+__global__ void __launch_bounds__(kDualThreads, 4) dcnv4_backward_dual_kernel(const DcnLaunch p, uint32_t n1, uint32_t n2, int interleave) {
   uint32_t local;
-  if (dual_first_role(blockIdx.x, n1, n2, local)) dcnv4_offset_mask_grad_tiled_body<Tag, NV, 9, PAIR>(p, local, n1);
+  if (dual_first_role(blockIdx.x, n1, n2, local, interleave != 0)) dcnv4_offset_mask_grad_tiled_body<Tag, NV, 9, PAIR>(p, local, n1);
   else dcnv4_grad_value_body<Tag, 9, 16, kGradValueColumnRounds, kDualThreads>(p, local, n2);
 }
 
@@ -52,7 +54,7 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
   const size_t lds = std::max(dcnv4_tiled_gather_lds_bytes(p, Tag::kBytes), dcnv4_grad_value_lds_bytes(p));
   auto go = [&](auto kernel) -> hipError_t {
     if (hipError_t e = ensure_dynamic_lds_limit(reinterpret_cast<const void *>(kernel), kMaxLdsPerWorkgroup - 1024)) return e;
-    hipLaunchKernelGGL(kernel, dim3(n1 + n2), dim3(kDualThreads), lds, stream, p, n1, n2);
+    hipLaunchKernelGGL(kernel, dim3(n1 + n2), dim3(kDualThreads), lds, stream, p, n1, n2, p.dual_interleave);
     return hipGetLastError();
   };
   const bool pair = p.gt_lpg == 2;
@@ -67,20 +69,25 @@ hipError_t launch_t(const DcnLaunch &p, hipStream_t stream) {
 }  // namespace
 
 // The launch plans (tiled gather and grad_value, both in p) suit the two-role kernel: a 3x3 kernel with its centre, whole
-// images as grad_value tiles in 512-lane workgroups, at most 64 channels a lane pair in the first role, 512 lanes there too
-// - and few enough workgroups to be resident (nearly) all at once, two per CU: that is when the roles overlap.  Measured
-// at batch 64: 7x7 images of 32 groups, 512 + 256 or 704 workgroups in all, 30.8 -> 21.7 us (fp16), 32.3 -> 27.9 us (fp32);
-// 14x14 images of 16 groups, 1024 / 1536 workgroups, 41.4 -> 41.9 us and 46.2 -> 50.0 us: left as two launches.
-bool dcnv4_backward_dual_fits(const DcnLaunch &p, int elem_bytes, int n_img, int n_cus) {
+// images as grad_value tiles in 512-lane workgroups, at most 64 channels a lane pair in the first role, 512 lanes there too.
+bool dcnv4_backward_dual_fits(const DcnLaunch &p, int elem_bytes) {
   if (!p.gv_whole || p.gt_h == 0 || p.softmax || p.kh != 3 || p.kw != 3 || p.remove_center) return false;
   if (p.gv_threads != kDualThreads || p.gv_cw != 16) return false;
   if (p.gt_h * p.gt_w * p.gt_ng * p.gt_lpg > kDualThreads) return false;
-  uint32_t n1, n2;
-  role_counts(p, n_img, &n1, &n2);
-  if (n1 + n2 > 3u * (uint32_t)n_cus) return false;
   const int nv = p.D * elem_bytes / 16 / p.gt_lpg;
   if (p.D * elem_bytes % (16 * p.gt_lpg) != 0 || !(nv == 1 || nv == 2 || nv == 4)) return false;
   return std::max(dcnv4_tiled_gather_lds_bytes(p, elem_bytes), dcnv4_grad_value_lds_bytes(p)) <= kMaxLdsPerWorkgroup / 2 - 512;
+}
+
+// Workgroups of both roles together, for n_img images.  Few enough to be resident (nearly) all at once, two per CU, and
+// the roles are interleaved and overlap (batch 64, 7x7 images of 32 groups, 512 / 704 workgroups: 30.8 -> 21.7 us fp16,
+// 32.3 -> 27.5 us fp32); more, and interleaving only slows both roles down (14x14 images of 16 groups, 1024 / 1536
+// workgroups: 41.4 -> 41.4 us, 46.1 -> 50.0 us), while one role after the other in the same grid still saves a dispatch
+// and the first role's tail (38.2 us, 45.4 us).
+uint32_t dcnv4_backward_dual_workgroups(const DcnLaunch &p, int n_img) {
+  uint32_t n1, n2;
+  role_counts(p, n_img, &n1, &n2);
+  return n1 + n2;
 }
 
 hipError_t launch_dcnv4_backward_dual(int dtype, const DcnLaunch &p, hipStream_t stream) {

@@ -93,6 +93,7 @@ struct DcnLaunch {
   int gt_pad;               // bytes between the cells of the staged window (16: fewer LDS bank conflicts; 0: a larger window fits)
   int gt_wh, gt_ww;         // largest input window (rows, columns of cells) a tile stages
   int gt_reach;             // input pixels around an output pixel's reference point that the window covers
+  int dual_interleave;      // two-role backward: workgroups of the two roles alternate in eights (else one role after the other)
   float gv_reach_cap;       // sampling points farther than this from their reference point stay out of reach_needed and are folded into GradState::far_reach
 };
 
@@ -255,7 +256,8 @@ hipError_t launch_dcnv4_offset_mask_grad(int dtype, const DcnLaunch &p, hipStrea
 hipError_t launch_dcnv4_grad_value(int dtype, const DcnLaunch &p, hipStream_t stream);
 // Both kernels of the backward as one launch with two workgroup roles, for shapes whose grad_value tiles are whole images
 // (dcnv4_backward_dual.hip).
-bool dcnv4_backward_dual_fits(const DcnLaunch &p, int elem_bytes, int n_img, int n_cus);
+bool dcnv4_backward_dual_fits(const DcnLaunch &p, int elem_bytes);
+uint32_t dcnv4_backward_dual_workgroups(const DcnLaunch &p, int n_img);
 hipError_t launch_dcnv4_backward_dual(int dtype, const DcnLaunch &p, hipStream_t stream);
 // Entry slots of the tiled grad_value kernel per (pixel, group) of a strip, and at most per strip: three-point items
 // for a 3x3 kernel (nine slots, also when the centre is removed), else an item per sampling point.
