@@ -11,8 +11,11 @@ more than ``--margin`` (default 3 %) and by more than ``--min-gain-us`` (default
 kernel-family options costs a few microseconds of host time per call), so an empty table is a valid outcome.
 """
 import argparse
+import glob
+import hashlib
 import json
 import math
+import os
 import sys
 import time
 
@@ -21,8 +24,24 @@ SHAPES = {
     "t": [(64, 56, 56, 4, 16), (64, 28, 28, 8, 16), (64, 14, 14, 16, 16), (64, 7, 7, 32, 16)],
     "b": [(128, 56, 56, 7, 16), (128, 28, 28, 14, 16), (128, 14, 14, 28, 16), (128, 7, 7, 56, 16)],
     "dense": [(2, 256, 256, 10, 16), (2, 128, 128, 20, 16), (2, 64, 64, 40, 16), (2, 32, 32, 80, 16)],
+    # groups of 64 channels: keys of the reference's table (DCNv4_op/DCNv4/functions/table.py:452-461)
+    "wide": [(64, 56, 56, 4, 64), (64, 28, 28, 4, 64)],
 }
 GEOM = (3, 3, 1, 1, 1, 1, 1, 1)
+
+
+def library_sources_sha256():
+    """Hash of the library's sources (csrc/*.hip, *.hpp and the C header): a table records which kernels it was tuned on,
+    also where no git history travels with the tree."""
+    here = os.path.dirname(os.path.abspath(__file__))
+    files = sorted(glob.glob(os.path.join(here, "csrc", "*.hip")) + glob.glob(os.path.join(here, "csrc", "*.hpp")) +
+                   [os.path.join(os.path.dirname(here), "include", "dcnv4_gfx950.h")])
+    h = hashlib.sha256()
+    for f in files:
+        h.update(os.path.basename(f).encode() + b"\0")
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
 
 
 def _time(fn, iters, warm):
@@ -43,7 +62,7 @@ def candidates(G, D, elem_bytes, direction):
     """(label, options, d_stride, n_thread) for a DCNv4 call; the first one is the library's own choice.  Every launch
     parameter the kernels have is swept, as the reference's search scripts sweep theirs
     (DCNv4_op/scripts/search_dcnv4.py:100-115): kernel family, hints of the direct family, the staged reach and the
-    output-tile cap of the LDS-tiled gathers, the input-tile cap and the workgroup size of the grad_value kernel."""
+    output-tile cap of the LDS-tiled gathers, the input-tile cap and the workgroup size of the grad_value kernel, one launch or two for the backward of small images."""
     out = [("library", {}, 0, 0)]
     for reach in (2, 3, 4, 6):
         out.append((f"reach {reach}", {"reach": reach}, 0, 0))
@@ -60,6 +79,8 @@ def candidates(G, D, elem_bytes, direction):
         for tile in (16, 8):
             out.append((f"grad_value tile {tile}", {"tile": tile}, 0, 0))
             out.append((f"grad_value tile {tile} reach 3", {"tile": tile, "reach": 3}, 0, 0))
+        out.append(("two launches", {"dual": "off"}, 0, 0))
+        out.append(("one launch, two workgroup roles", {"dual": "on", "gv_threads": 512}, 0, 0))
         for threads in (512, 1024):
             out.append((f"grad_value {threads} lanes", {"gv_threads": threads}, 0, 0))
             out.append((f"grad_value {threads} lanes tile 16", {"gv_threads": threads, "tile": 16}, 0, 0))
@@ -165,7 +186,7 @@ def tune(shape_sets, dtypes, iters=50, warm=10, margin=0.03, min_gain_us=10.0, o
 
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
-    ap.add_argument("--shapes", default="t,b,dense,detr,detr_coco",
+    ap.add_argument("--shapes", default="t,b,dense,wide,detr,detr_coco",
                     help="comma-separated shape sets: " + ", ".join(list(SHAPES) + list(ATTN_SHAPES)))
     ap.add_argument("--dtypes", default="float16,float32")
     ap.add_argument("--iters", type=int, default=50)
@@ -173,6 +194,7 @@ def main(argv=None):
     ap.add_argument("--min-gain-us", type=float, default=10.0)
     ap.add_argument("--out", default=None, help="table file (default: dcnv4_amd/functions/gfx950_table.json)")
     ap.add_argument("--report", default=None, help="also write every timing to this JSON file")
+    ap.add_argument("--library-commit", default=None, help="git commit of the library the table is made on (recorded in the table)")
     args = ap.parse_args(argv)
     import torch
     if not torch.cuda.is_available():
@@ -182,7 +204,8 @@ def main(argv=None):
     entries, report = tune(args.shapes.split(","), args.dtypes.split(","), iters=args.iters, margin=args.margin,
                            min_gain_us=args.min_gain_us)
     table = {"device": torch.cuda.get_device_name(0), "made": time.strftime("%Y-%m-%d"), "abi_version": _lib.ABI_VERSION,
-             "margin": args.margin,
+             "library_commit": args.library_commit, "library_sources_sha256": library_sources_sha256(),
+             "cases": len(report), "margin": args.margin,
              "min_gain_us": args.min_gain_us, "entries": entries}
     out = args.out or launch_spec.TABLE_PATH
     with open(out, "w") as f:

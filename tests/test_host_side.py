@@ -299,7 +299,8 @@ def test_tuner_candidates_are_valid_hints_and_start_with_the_library_choice():
         assert {"reach": 3} in [c[1] for c in fwd] and {"gather_tile": 8} in [c[1] for c in fwd]
         bwd = tune.candidates(G, D, es, "bwd")
         assert bwd[0] == ("library", {}, 0, 0) and {"tile": 16} in [c[1] for c in bwd] and {"reach": 2} in [c[1] for c in bwd]
-    assert set(tune.SHAPES) == {"t", "b", "dense"} and all(len(v) == 4 for v in tune.SHAPES.values())
+    assert {"gv_threads": 512} in [c[1] for c in bwd] and {"dual": "off"} in [c[1] for c in bwd]
+    assert set(tune.SHAPES) == {"t", "b", "dense", "wide"} and all(len(v) in (2, 4) for v in tune.SHAPES.values())
     att = tune.attention_candidates("bwd")
     assert att[0] == ("library", {}) and {"scatter": "atomic"} in [c[1] for c in att] and {"fda_order": "heads"} in [c[1] for c in att]
     # every option the tuner may write is one the table loader passes on
@@ -341,3 +342,16 @@ def test_module_initial_values_follow_the_reference_recipe():
         d = d / d.abs().max()
         for k in range(4):
             assert torch.allclose(bias[h, :, k], (d * (k + 1)).expand(3, 2), atol=1e-6)
+
+
+def test_committed_table_records_the_library_it_was_tuned_on():
+    """The tuner stamps its table with the commit and a hash of the library's sources (DCNv4_op/scripts/find_best.py
+    pastes its winners into table.py by hand; here a reader can tell which kernels the numbers belong to)."""
+    import json
+    from dcnv4_amd import tune
+    from dcnv4_amd.functions import launch_spec as ls
+    table = json.load(open(ls.TABLE_PATH))
+    assert isinstance(table.get("entries"), dict) and table.get("cases", 0) >= 56
+    assert isinstance(table.get("library_commit"), str) and len(table["library_commit"]) >= 7
+    sha = table.get("library_sources_sha256")
+    assert isinstance(sha, str) and len(sha) == 64 and len(tune.library_sources_sha256()) == 64
