@@ -63,11 +63,25 @@ def fda_bytes(s, B, N, Q, G, D, L, K):
 # `bench.py --only-op <key>`, each counter scaled by its reading for a plain copy of known size
 # (`--only-op copy:256`: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0, KiB).  The summaries are in profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    # algorithmic 334.0e6: the grad_value kernel reads offset_mask and grad_out again (141.5e6), and the gradients'
-    # nontemporal stores are counted in the pieces in which the workgroups that share a line write it (215.7e6 for 141.4e6)
-    "dcnv4_bwd:T-stage1:float32": 550.0e6,
-    "dcnv4_bwd:T-stage1:float16": 238.0e6,     # algorithmic 167.0e6
+    # (profiles/dcnv4_step_operators_traffic.txt; the backward's excess over its algorithmic bytes: the grad_value kernel reads
+    # offset_mask and grad_out a second time, and the fp32 gradients' nontemporal stores are counted in the pieces in which
+    # the workgroups that share a line write it)
     "dcnv4_fwd:T-stage1:float16": 96.5e6,      # algorithmic 96.3e6
+    "dcnv4_bwd:T-stage1:float16": 238.0e6,     # algorithmic 167.0e6
+    "dcnv4_fwd:T-stage2:float16": 47.5e6,      # algorithmic 47.4e6
+    "dcnv4_bwd:T-stage2:float16": 116.8e6,     # algorithmic 81.9e6
+    "dcnv4_fwd:T-stage3:float16": 23.8e6,      # algorithmic 23.7e6
+    "dcnv4_bwd:T-stage3:float16": 51.3e6,      # algorithmic 40.9e6
+    "dcnv4_fwd:T-stage4:float16": 12.0e6,      # algorithmic 11.8e6
+    "dcnv4_bwd:T-stage4:float16": 23.0e6,      # algorithmic 20.5e6
+    "dcnv4_fwd:T-stage1:float32": 192.8e6,     # algorithmic 192.7e6
+    "dcnv4_bwd:T-stage1:float32": 551.1e6,     # algorithmic 334.0e6
+    "dcnv4_fwd:T-stage2:float32": 94.9e6,      # algorithmic 94.7e6
+    "dcnv4_bwd:T-stage2:float32": 262.8e6,     # algorithmic 163.8e6
+    "dcnv4_fwd:T-stage3:float32": 47.5e6,      # algorithmic 47.4e6
+    "dcnv4_bwd:T-stage3:float32": 121.0e6,     # algorithmic 81.9e6
+    "dcnv4_fwd:T-stage4:float32": 23.9e6,      # algorithmic 23.7e6
+    "dcnv4_bwd:T-stage4:float32": 45.1e6,      # algorithmic 40.9e6
 }
 
 
@@ -78,6 +92,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--offset-range", type=float, default=None,
                     help="with --only-op dcnv4_*: offsets uniform in +-this many pixels instead of the benchmark's +-3 (+-4 for the dense shapes)")
+    ap.add_argument("--far-offset", action="store_true",
+                    help="with --only-op dcnv4_*: one sampling point of one pixel is sent 200 pixels away (the robustness row of the detail table)")
     ap.add_argument("--op-iters", type=int, default=100, help="timed launches per operator in the detail table")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-detail", action="store_true", help="skip per-operator timings other than the step's own")
@@ -158,6 +174,16 @@ def main():
         src, dst = torch.randn(n, device=dev), torch.empty(n, device=dev)
         ms = time_op(lambda: ext.stream_copy(src, dst), iters, warm=warm)
         return ms, n * 4, 2 * n * 4 / (ms * 1e-3) / 1e9
+
+    if args.only_op == "lds_probe":
+        # LDS read patterns: ticks per wave-level 16-byte read, and each pattern against the best one
+        names = ["consecutive addresses (slot = lane, one cell per wave)", "random cells, slot = lane & 15 (16 lanes cover 256 B)",
+                 "random cells, slot = lane & 7 (8 lanes cover 128 B)", "random cells, random slots (a gather of rows)",
+                 "random cells, every lane on slot 0"]
+        ticks = [min(ext.lds_read_probe(pat, 4000) for _ in range(3)) for pat in range(5)]
+        print(json.dumps({"only_op": "lds_probe", "unit": "cycle-counter ticks per wave instruction (ds_read_b128, 16 waves, 8 reads in flight)",
+                          "patterns": [{"pattern": n, "ticks": round(t, 2), "vs_best": round(t / min(ticks), 2)} for n, t in zip(names, ticks)]}))
+        return
 
     if args.only_op and args.only_op.startswith("copy:"):
         # plain copy of known size: calibrates FETCH_SIZE / WRITE_SIZE counters and shows the HBM ceiling
@@ -250,6 +276,8 @@ def main():
                 if name != shape_name:
                     continue
                 t = dcn_inputs(B, H, W, C, G, dtype, off if args.offset_range is None else args.offset_range)
+                if args.far_offset:
+                    t[1][0, 10, 10, 0] = 200.0
                 fn = (lambda: dcn_fwd(t, G, C)) if op == "dcnv4_fwd" else (lambda: dcn_bwd(t, G, C))
                 ms = time_op(fn, args.steps, warm=args.warmup)
                 nbytes = dcn_bytes(t[0].element_size(), B, H, W, C, G)[0 if op == "dcnv4_fwd" else 1]

@@ -10,7 +10,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libdcnv4_gfx950.so")
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 OK, ERR_INVALID_ARGUMENT, ERR_RUNTIME = 0, 1, 2
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 
@@ -39,6 +39,7 @@ SIGNATURES = {
     "dcnv4_gfx950_layer_norm_residual_backward": (_i, [_vp] * 10 + [_sz, _i, ctypes.c_longlong, _i, _f, _vp]),
     "dcnv4_gfx950_center_feature_blend_forward": (_i, [_vp] * 5 + [_i, ctypes.c_longlong, _i, _i, _vp]),
     "dcnv4_gfx950_stream_copy": (_i, [_vp, _vp, _sz, _vp]),
+    "dcnv4_gfx950_lds_read_probe": (_i, [_i, _i, _vp, _vp]),
     "dcnv4_gfx950_center_feature_blend_backward": (_i, [_vp] * 8 + [_i, ctypes.c_longlong, _i, _i, _vp]),
 }
 

@@ -102,6 +102,42 @@ __global__ void __launch_bounds__(256) stream_copy_kernel(const u32x4 *src, u32x
     if (base + u * 256 < n16) __builtin_nontemporal_store(v[u], dst + base + u * 256);
 }
 
+// LDS read probe: a 1024-lane workgroup issues `iters` rounds of eight 16-byte LDS reads per lane whose addresses follow
+// one of a few patterns, and reports the cycle counter's ticks per wave instruction.  Every lane reads at
+// cell * 1024 + slot * 16 with a cell (of 64) that changes per read.
+//   0  all lanes of a wave in one cell, slot = lane (1 KB of consecutive addresses)
+//   1  a random cell per lane, slot = lane & 15: any 16 consecutive lanes cover 16 different slots of 256 bytes
+//   2  a random cell per lane, slot = lane & 7: 8 consecutive lanes cover the 8 slots of 128 bytes
+//   3  a random cell and a random slot per lane (what a gather from rows at data-dependent cells looks like)
+//   4  a random cell per lane, slot 0 for every lane (the worst case)
+__global__ void __launch_bounds__(1024) lds_read_probe_kernel(int pattern, int iters, uint32_t *ticks_per_1000) {
+  __shared__ u32x4 cells[4096];                   // 64 KB
+  for (int i = threadIdx.x; i < 4096; i += 1024) cells[i] = u32x4{(uint32_t)i, 0u, 0u, 0u};
+  __syncthreads();
+  const int lane = threadIdx.x & 63;
+  uint32_t seed = threadIdx.x * 131u + 7u;
+  u32x4 acc = {0u, 0u, 0u, 0u};
+  const int fixed_slot = pattern == 0 ? lane : (pattern == 1 ? (lane & 15) : (pattern == 2 ? (lane & 7) : 0));
+  __syncthreads();
+  const long long t0 = clock64();
+  for (int i = 0; i < iters; ++i) {
+    seed = seed * 1664525u + 1013904223u;
+    const uint32_t r = seed >> 8;
+    u32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int cell = pattern == 0 ? ((i + u) & 63) : (int)((r >> (3 * u)) & 63u);
+      const int slot = pattern == 3 ? (int)((r >> (2 * u + 1)) & 63u) : fixed_slot;
+      v[u] = cells[cell * 64 + slot];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc ^= v[u];
+  }
+  const long long t1 = clock64();
+  if (threadIdx.x == 0) *ticks_per_1000 = (uint32_t)((t1 - t0) * 1000 / ((long long)iters * 8 * 16));      // 16 waves, 8 reads a round
+  if (acc.x == 0xdeadbeefu) *ticks_per_1000 = acc.y;      // keeps the reads alive
+}
+
 int grid_for(size_t work_items) {
   const size_t blocks = (work_items + 255) / 256;
   return (int)std::min<size_t>(std::max<size_t>(blocks, 1), 256 * 32);
@@ -1239,6 +1275,15 @@ int dcnv4_gfx950_center_feature_blend_backward(const void *grad_output, const vo
   L.grad_y = grad_sampled; L.grad_x = grad_projected; L.grad_logits = grad_gate_logits;
   if (hipError_t e = launch_center_feature_blend(dtype, L, true, static_cast<hipStream_t>(stream)))
     return hip_fail("centre-feature blend backward launch", e);
+  return DCNV4_OK;
+}
+
+int dcnv4_gfx950_lds_read_probe(int pattern, int iters, unsigned int *ticks_per_1000_reads, void *stream) {
+  if (pattern < 0 || pattern > 4 || iters < 1 || iters > (1 << 20))
+    return fail(DCNV4_ERR_INVALID_ARGUMENT, "LDS read probe: pattern %d (0..4), %d rounds (1..2^20)", pattern, iters);
+  if (ticks_per_1000_reads == nullptr) return fail(DCNV4_ERR_RUNTIME, "null tensor pointer");
+  hipLaunchKernelGGL(lds_read_probe_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream), pattern, iters, ticks_per_1000_reads);
+  if (hipError_t e = hipGetLastError()) return hip_fail("LDS read probe launch", e);
   return DCNV4_OK;
 }
 

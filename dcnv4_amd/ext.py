@@ -467,3 +467,13 @@ def stream_copy(src, dst):
     with _on_device(src.device):
         _lib.check(_L.dcnv4_gfx950_stream_copy(src.data_ptr(), dst.data_ptr(), nbytes, _stream()))
     return dst
+
+
+def lds_read_probe(pattern, iters=4000, device=None):
+    """Ticks of the cycle counter per wave-level 16-byte LDS read for one of the probe's address patterns (0 consecutive,
+    1 random cells with slot = lane & 15, 2 slot = lane & 7, 3 random cells and slots, 4 all lanes on one slot)."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
+    with _on_device(device):
+        out = torch.zeros(1, dtype=torch.int32, device=device)
+        _lib.check(_L.dcnv4_gfx950_lds_read_probe(int(pattern), int(iters), out.data_ptr(), _stream()))
+        return out.item() / 1000.0

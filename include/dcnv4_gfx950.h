@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define DCNV4_GFX950_ABI_VERSION 5
+#define DCNV4_GFX950_ABI_VERSION 6
 
 #define DCNV4_DTYPE_F32 0
 #define DCNV4_DTYPE_F16 1
@@ -324,6 +324,19 @@ int dcnv4_gfx950_center_feature_blend_backward(const void *grad_output, const vo
  * benchmark quotes beside the nominal HBM peak, and its known traffic calibrates hardware byte counters.
  */
 int dcnv4_gfx950_stream_copy(const void *src, void *dst, size_t bytes, void *stream);
+
+/*
+ * Measurement aid without a counterpart in the reference: one 1024-lane workgroup reads 16-byte vectors from LDS at
+ * addresses cell * 1024 + slot * 16 (a new cell of 64 for every read) for `iters` rounds of eight reads per lane and
+ * writes the cycle counter's ticks per 1000 wave-level read instructions to the device word `ticks_per_1000_reads`.
+ *   pattern 0  one cell per wave, slot = lane (consecutive addresses)
+ *           1  a random cell per lane, slot = lane & 15 (16 consecutive lanes cover 16 different slots of 256 bytes)
+ *           2  a random cell per lane, slot = lane & 7
+ *           3  a random cell and a random slot per lane (a gather of rows at data-dependent cells)
+ *           4  a random cell per lane, slot 0 for all (worst case)
+ * The ratios between the patterns say which address patterns the sampling kernels' LDS reads can hope for.
+ */
+int dcnv4_gfx950_lds_read_probe(int pattern, int iters, unsigned int *ticks_per_1000_reads, void *stream);
 
 #ifdef __cplusplus
 }

@@ -235,3 +235,16 @@ def test_stream_copy_copies_and_rejects_odd_sizes():
     assert torch.equal(small, out)
     with pytest.raises(ValueError, match="multiple of 16"):
         ext.stream_copy(torch.zeros(3, device="cuda"), torch.zeros(3, device="cuda"))
+
+
+def test_lds_read_probe_orders_its_patterns():
+    """The measurement aid behind the LDS-pattern figures: all lanes on one 16-byte slot must cost several times what
+    16 lanes on 16 different slots cost, and a random gather lies in between."""
+    from dcnv4_amd import ext
+    best = min(ext.lds_read_probe(1, 2000) for _ in range(3))
+    gather = min(ext.lds_read_probe(3, 2000) for _ in range(3))
+    worst = min(ext.lds_read_probe(4, 2000) for _ in range(3))
+    print(f"LDS probe: spread {best:.2f}, gather {gather:.2f}, one slot {worst:.2f} ticks per read", flush=True)
+    assert 0 < best < gather < worst and worst > 3 * best
+    with pytest.raises(ValueError, match="pattern"):
+        ext.lds_read_probe(9)
