@@ -24,7 +24,7 @@ def test_library_exports_every_symbol_the_header_declares():
     from dcnv4_amd import _lib
     lib = ctypes.CDLL(_lib.LIB_PATH)
     declared = _declared_functions()
-    assert len(declared) == 22, sorted(declared)
+    assert len(declared) == 23, sorted(declared)
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in include/dcnv4_gfx950.h but not exported"
     assert set(declared) == set(_lib.SIGNATURES), "ctypes table and header list different functions"
