@@ -304,7 +304,7 @@ bool plan_gather_tiles(DcnLaunch *L, int s, bool backward) {
   L->gt_lpg = 1;
   L->gt_pad = 16;
   L->gt_reach = reach_setting();
-  if (!tiled_gather_enabled() || L->softmax) return false;
+  if (!tiled_gather_enabled()) return false;
   const int lane_bytes = L->D * s;
   if (lane_bytes % 16 != 0) return false;
   const int nv = lane_bytes / 16;

@@ -20,8 +20,9 @@
 //   * a sampling point whose corners leave the window is remembered in a per-lane bit mask and
 //     served afterwards from global memory (the range-checked gather of dcnv4_kernels.hip), so
 //     any offset is handled; with offsets inside the window that code never runs.
-// The softmax variant of the modulation (never requested by the reference's Python side) stays on
-// the global-memory kernels.
+// The softmax variant of the modulation (dcnv4_im2col_cuda.cuh:173-193, dcnv4_col2im_cuda.cuh:352-365; never
+// requested by the reference's Python side) runs on the instantiations for a run-time kernel shape (KP == 0) only, so
+// that the 3x3 instantiations carry nothing for it.
 #include <type_traits>
 
 #include "common.hpp"
@@ -346,11 +347,25 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_forward_tiled_kernel(cons
     for (int c = 0; c < EPV; ++c) acc[v][c] = 0.f;
   typedef typename std::conditional<(KP > 0), uint32_t, uint64_t>::type mask_t;     // one bit per sampling point
   mask_t far_mask = 0;
+  // softmax over the group's modulation logits: running maximum and reciprocal sum, the probabilities are recomputed per tap
+  float sm_max = 0.f, sm_inv = 1.f;
+  if constexpr (KP == 0) {
+    if (p.softmax) {
+      sm_max = lds_elem<Tag>(om, 2 * Kp);
+      for (int k = 1; k < Kp; ++k) sm_max = fmaxf(sm_max, lds_elem<Tag>(om, 2 * Kp + k));
+      float sum = 0.f;
+      for (int k = 0; k < Kp; ++k) sum += __expf(lds_elem<Tag>(om, 2 * Kp + k) - sm_max);
+      sm_inv = 1.f / sum;
+    }
+  }
 
   auto position = [&](int k, int i, int j, float &y, float &x, float &m) {
     x = add_rn(x_base, mul_rn(add_rn((float)(i * p.dw), lds_elem<Tag>(om, 2 * k)), p.offset_scale));
     y = add_rn(y_base, mul_rn(add_rn((float)(j * p.dh), lds_elem<Tag>(om, 2 * k + 1)), p.offset_scale));
     m = lds_elem<Tag>(om, 2 * Kp + k);
+    if constexpr (KP == 0) {
+      if (p.softmax) m = __expf(m - sm_max) * sm_inv;
+    }
   };
   // A sampling point in flight: its four modulated corner weights and its LDS reads.
   struct Flight {
@@ -537,8 +552,26 @@ __device__ __forceinline__ void dcnv4_offset_mask_grad_tiled_body(const DcnLaunc
     const bool pair = p.gt_lpg == 2;       // the two lanes of a (pixel, group) add their halves of each dot product
     typedef typename std::conditional<(KP > 0), uint32_t, uint64_t>::type mask_t;
     mask_t far_mask = 0;
+    // softmax over the group's modulation logits (KP == 0 only): statistics before the slots turn into gradients;
+    // sm_dot collects sum_k p_k * dL/dp_k in the lane that writes, for the Jacobian at the end
+    float sm_max = 0.f, sm_inv = 1.f, sm_dot = 0.f;
+    if constexpr (KP == 0) {
+      if (p.softmax) {
+        sm_max = lds_elem<Tag>(om, 2 * Kp);
+        for (int k = 1; k < Kp; ++k) sm_max = fmaxf(sm_max, lds_elem<Tag>(om, 2 * Kp + k));
+        float sum = 0.f;
+        for (int k = 0; k < Kp; ++k) sum += __expf(lds_elem<Tag>(om, 2 * Kp + k) - sm_max);
+        sm_inv = 1.f / sum;
+      }
+    }
     auto put = [&](int k, float gx, float gy, float gz, float m, bool writer) {
       if (!writer) return;
+      if constexpr (KP == 0) {
+        if (p.softmax) {      // the slot holds p_k * dL/dp_k until every tap is done (dcnv4_col2im_cuda.cuh:337-339)
+          gz *= m;
+          sm_dot += gz;
+        }
+      }
       const float f0[1] = {gx * p.offset_scale * m}, f1[1] = {gy * p.offset_scale * m}, f2[1] = {gz};
       om[2 * k] = Pack<Tag, 1>::encode(f0);
       om[2 * k + 1] = Pack<Tag, 1>::encode(f1);
@@ -554,7 +587,10 @@ __device__ __forceinline__ void dcnv4_offset_mask_grad_tiled_body(const DcnLaunc
     auto one_tap = [&](int k, int i, int j) {
       const float x = add_rn(x_base, mul_rn(add_rn((float)(i * p.dw), lds_elem<Tag>(om, 2 * k)), p.offset_scale));
       const float y = add_rn(y_base, mul_rn(add_rn((float)(j * p.dh), lds_elem<Tag>(om, 2 * k + 1)), p.offset_scale));
-      const float m = lds_elem<Tag>(om, 2 * Kp + k);
+      float m = lds_elem<Tag>(om, 2 * Kp + k);
+      if constexpr (KP == 0) {
+        if (p.softmax) m = __expf(m - sm_max) * sm_inv;
+      }
       const WinTap wt = window_tap(y, x, p.H, p.W, t, cell_stride, lane_bytes, zero_base);
       far_mask |= (mask_t)(wt.inside && !wt.ok) << k;
       // Chebyshev distance of the point from the reference point; its ceiling is how far the weighted corners of
@@ -668,7 +704,10 @@ __device__ __forceinline__ void dcnv4_offset_mask_grad_tiled_body(const DcnLaunc
     auto far_tap = [&](int k, int i, int j) {
       const float x = add_rn(x_base, mul_rn(add_rn((float)(i * p.dw), lds_elem<Tag>(om_g, 2 * k)), p.offset_scale));
       const float y = add_rn(y_base, mul_rn(add_rn((float)(j * p.dh), lds_elem<Tag>(om_g, 2 * k + 1)), p.offset_scale));
-      const float m = lds_elem<Tag>(om_g, 2 * Kp + k);
+      float m = lds_elem<Tag>(om_g, 2 * Kp + k);
+      if constexpr (KP == 0) {
+        if (p.softmax) m = __expf(m - sm_max) * sm_inv;
+      }
       const Tap tp = make_tap(y, x, p.H, p.W, img_base, pix_bytes);
       // beyond the reach cap: left out of the reach statistic above, folded per destination tile instead
       if (tp.valid != 0 && fmaxf(fabsf(x - p0xf), fabsf(y - p0yf)) > p.gv_reach_cap) dcnv4_fold_far_point(p, t.b, t.g0 + gl, tp.y0, tp.x0, p0y, p0x);
@@ -720,6 +759,15 @@ __device__ __forceinline__ void dcnv4_offset_mask_grad_tiled_body(const DcnLaunc
             else if ((far_mask >> k) & 1) far_tap(k, i, j);
             ++k;
           }
+      }
+      // softmax Jacobian: dL/dlogit_k = p_k * dL/dp_k - p_k * sum_j p_j * dL/dp_j (dcnv4_col2im_cuda.cuh:352-365); the
+      // logits are read from memory again, their slots hold the first term
+      if (p.softmax && part == 0) {
+        for (int k = 0; k < Kp; ++k) {
+          const float pk = __expf(lds_elem<Tag>(om_g, 2 * Kp + k) - sm_max) * sm_inv;
+          const float f[1] = {lds_elem<Tag>(om, 2 * Kp + k) - pk * sm_dot};
+          om[2 * Kp + k] = Pack<Tag, 1>::encode(f);
+        }
       }
     }
   }

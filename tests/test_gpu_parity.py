@@ -129,17 +129,36 @@ def test_dcnv4_every_kernel_path_matches_oracle(oracle, name, path, dtype):
     assert (gom[..., used:] == 0).all(), "padded tail of grad_offset_mask must be exactly zero"
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float16], ids=["fp32", "fp16"])
-def test_dcnv4_softmax_flag_matches_oracle(oracle, dtype):
-    v, om, go, (geom, G, D, scale, rc) = _dcn_inputs(DCN_CASES["remove_center"], dtype, seed=5)
+SOFTMAX_PATHS = {
+    "library_choice": {},                       # the LDS-tiled gathers (their run-time-shape instantiations)
+    "direct_gather": dict(gather="direct"),
+    "reach0": dict(reach=0),                    # every sampling point through the tiled gathers' global-memory path
+    "gather_tile4_reach1": dict(gather_tile=4, reach=1),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("path", list(SOFTMAX_PATHS))
+@pytest.mark.parametrize("name", ["remove_center", "cfg1_56x56_c64_g4", "stride2", "dilation2_pad2", "kernel_5x5", "g5_16x12",
+                                  "far_offsets_mostly_outside", "d64_g4_20x18", "stage_7x7_c512_g32"])
+def test_dcnv4_softmax_flag_matches_oracle(oracle, name, path, dtype):
+    """The reference's latent softmax over a group's modulation scalars (dcnv4_im2col_cuda.cuh:173-193,
+    dcnv4_col2im_cuda.cuh:352-365), through both gather families."""
+    from dcnv4_amd import ext
+    v, om, go, (geom, G, D, scale, rc) = _dcn_inputs(DCN_CASES[name], dtype, seed=5)
+    print(f"softmax case {name} path {path} dtype {dtype}", flush=True)
     args = _oracle_args(geom, G, D, scale, rc)
     want = oracle.dcnv4_forward(cabi.f64(v), cabi.f64(om), *args, softmax=True, coord_f32=True)
     wgv, wgom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *args, softmax=True, coord_f32=True)
-    out = cabi.dcnv4_forward(v.cuda(), om.cuda(), geom, G, D, scale, rc, softmax=1)
-    gv, gom = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), geom, G, D, scale, rc, softmax=1)
+    with ext.launch_options(**SOFTMAX_PATHS[path]):
+        out = cabi.dcnv4_forward(v.cuda(), om.cuda(), geom, G, D, scale, rc, softmax=1)
+        gv, gom = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), geom, G, D, scale, rc, softmax=1)
+    torch.cuda.synchronize()
     cabi.assert_close(out, want, *FWD_TOL[dtype], what="output")
     cabi.assert_close(gv, wgv, *GRAD_TOL[dtype], what="grad_value")
     cabi.assert_close(gom, wgom, *GRAD_TOL[dtype], what="grad_offset_mask")
+    used = G * 3 * (geom[0] * geom[1] - rc)
+    assert (gom[..., used:] == 0).all(), "padded tail of grad_offset_mask must be exactly zero"
 
 
 def test_dcnv4_unpadded_offset_mask_rows(oracle):

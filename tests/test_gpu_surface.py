@@ -430,18 +430,25 @@ def test_dcnv4_module_under_autocast_runs_the_half_kernels_and_returns_fp32_para
 
 @pytest.mark.parametrize("options", [dict(gather="direct"), dict(tile=16), dict(gather="direct", tile=8),
                                      dict(gather="tiled", reach=2)])
-def test_launch_options_change_the_kernels_not_the_results(options):
-    """Thread-local launch options (what a tuned table entry applies around a call) against the library's own choice."""
+def test_launch_options_change_the_kernels_not_the_results(oracle, options):
+    """Thread-local launch options (what a tuned table entry applies around a call): every result against the oracle,
+    and against the library's own choice."""
     import dcnv4_amd
     from dcnv4_amd import ext
     v, om, go = make_dcnv4_inputs(2, 20, 18, 4, 16, offset_range=3.0, seed=7, dtype=torch.float16)
-    v, om, go = v.cuda(), om.cuda(), go.cuda()
     geom = (3, 3, 1, 1, 1, 1, 1, 1)
+    oracle_out = oracle.dcnv4_forward(cabi.f64(v), cabi.f64(om), *geom, 4, 16, 1.0, 0, coord_f32=True)
+    oracle_gv, oracle_gom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *geom, 4, 16, 1.0, 0, coord_f32=True)
+    v, om, go = v.cuda(), om.cuda(), go.cuda()
     want = ext.dcnv4_forward(v, om, *geom, 4, 16, 1.0, 64, 0, 0, 0, False)
     wgv, wgom = ext.dcnv4_backward(v, om, *geom, 4, 16, 1.0, 64, go, 0, 0, 0, False)
     with ext.launch_options(**options):
         out = ext.dcnv4_forward(v, om, *geom, 4, 16, 1.0, 64, 0, 8, 128, False)
         gv, gom = ext.dcnv4_backward(v, om, *geom, 4, 16, 1.0, 64, go, 0, 0, 0, False)
+    for got_out, got_gv, got_gom in ((want, wgv, wgom), (out, gv, gom)):
+        cabi.assert_close(got_out, oracle_out, 1e-2, 1e-3, what=f"output, {options}")
+        cabi.assert_close(got_gv, oracle_gv, 1e-2, 1e-2, what=f"grad_value, {options}")
+        cabi.assert_close(got_gom, oracle_gom, 1e-2, 1e-2, what=f"grad_offset_mask, {options}")
     assert _rel_err(out.float().cpu(), want.float().cpu()) < 2e-3
     assert _rel_err(gv.float().cpu(), wgv.float().cpu()) < 1e-2
     assert _rel_err(gom.float().cpu(), wgom.float().cpu()) < 2e-3
@@ -551,14 +558,17 @@ def test_depthwise_batches_beyond_the_32_bit_addressing_span_are_chunked_consist
     assert _rel_err(gw.double(), gw_sum) < 1e-5 and _rel_err(gb.double(), gb_sum) < 1e-5
 
 
-def test_autograd_function_applies_a_tuned_table_entry(monkeypatch):
+def test_autograd_function_applies_a_tuned_table_entry(oracle, monkeypatch):
     """DCNv4Function looks shapes up as (B, H, W, group, channels per group), the reference's key convention; an
     entry with a kernel family must reach the library as a launch option around the call, and only around it."""
     import dcnv4_amd
     from dcnv4_amd import _lib, ext
     from dcnv4_amd.functions import launch_spec as ls
     B, H, W, G, D = 2, 12, 10, 2, 16
-    v, om, go = (t.cuda() for t in make_dcnv4_inputs(B, H, W, G, D, seed=14, dtype=torch.float16))
+    v, om, go = make_dcnv4_inputs(B, H, W, G, D, seed=14, dtype=torch.float16)
+    oracle_out = oracle.dcnv4_forward(cabi.f64(v), cabi.f64(om), *GEOM, G, D, 1.0, 0, coord_f32=True)
+    oracle_gv, oracle_gom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *GEOM, G, D, 1.0, 0, coord_f32=True)
+    v, om, go = v.cuda(), om.cuda(), go.cuda()
     want = dcnv4_amd.DCNv4Function.apply(v, om, *GEOM, G, D, 1.0, 256, 0)
     monkeypatch.setitem(ls.GFX950_TABLE, ls.table_key(B, H, W, G, D, 2, "fwd"), {"d_stride": 8, "n_thread": 128, "gather": "direct"})
     monkeypatch.setitem(ls.GFX950_TABLE, ls.table_key(B, H, W, G, D, 2, "bwd"), {"d_stride": 1, "n_thread": 64, "tile": 16})
@@ -580,7 +590,10 @@ def test_autograd_function_applies_a_tuned_table_entry(monkeypatch):
         ls._lookup.cache_clear()
     assert (b"gather", 2) in seen and (b"tile", 16) in seen
     assert seen[-1] == (b"tile", 0) and (b"gather", 0) in seen          # back at the library's choice
-    assert _rel_err(out.float().cpu(), want.float().cpu()) < 2e-3 and vg.grad is not None and omg.grad is not None
+    assert _rel_err(out.float().cpu(), want.float().cpu()) < 2e-3
+    cabi.assert_close(out.detach(), oracle_out, 1e-2, 1e-3, what="output through the table entry")
+    cabi.assert_close(vg.grad, oracle_gv, 1e-2, 1e-2, what="grad_value through the table entry")
+    cabi.assert_close(omg.grad, oracle_gom, 1e-2, 1e-2, what="grad_offset_mask through the table entry")
 
 
 def test_block_tail_at_the_model_stage_one_size_normalises_every_row():
