@@ -76,6 +76,7 @@ bool dcnv4_backward_dual_fits(const DcnLaunch &p, int elem_bytes) {
   if (p.gt_h * p.gt_w * p.gt_ng * p.gt_lpg > kDualThreads) return false;
   const int nv = p.D * elem_bytes / 16 / p.gt_lpg;
   if (p.D * elem_bytes % (16 * p.gt_lpg) != 0 || !(nv == 1 || nv == 2 || nv == 4)) return false;
+  if (nv == 1 && p.gt_lpg != 1) return false;      // the one-vector instantiation is built for one lane per (pixel, group)
   return std::max(dcnv4_tiled_gather_lds_bytes(p, elem_bytes), dcnv4_grad_value_lds_bytes(p)) <= kMaxLdsPerWorkgroup / 2 - 512;
 }
 

@@ -12,7 +12,9 @@ __global__ void __launch_bounds__(kTiledThreads) dcnv4_offset_mask_grad_tiled_ke
 
 template <typename Tag, int NV, bool BWD, bool PAIR>
 hipError_t launch_nv(const DcnLaunch &p, hipStream_t stream, dim3 grid, dim3 block, size_t lds) {
-  const bool k3 = p.kh == 3 && p.kw == 3 && !p.softmax;      // the softmax variant lives in the run-time-shape instantiations
+  // the 3x3 instantiations know their lanes per (pixel, group) at compile time; the softmax variant lives in the
+  // run-time-shape ones
+  const bool k3 = p.kh == 3 && p.kw == 3 && !p.softmax && (PAIR || p.gt_lpg == 1);
   auto go = [&](auto kernel) -> hipError_t {
     // leaves room for the kernels' static LDS
     if (hipError_t e = ensure_dynamic_lds_limit(reinterpret_cast<const void *>(kernel), kMaxLdsPerWorkgroup - 1024)) return e;

@@ -309,7 +309,7 @@ __device__ __forceinline__ WinTap window_tap(float y, float x, int H, int W, con
   r.w[0] = hy * hx; r.w[1] = hy * r.lx; r.w[2] = r.ly * hx; r.w[3] = r.ly * r.lx;
   const bool near = (unsigned)ry < (unsigned)max(t.wh - 1, 0) && (unsigned)rx < (unsigned)max(t.ww - 1, 0);
   r.ok = r.inside && near;
-  r.addr = r.ok ? __mul24(__mul24(ry, t.ww) + rx, cell_stride) + lane_bytes : zero_base;
+  r.addr = r.ok ? __mul24(ry, __mul24(t.ww, cell_stride)) + __mul24(rx, cell_stride) + lane_bytes : zero_base;      // two full-rate 24-bit multiply-adds
   return r;
 }
 
@@ -536,7 +536,7 @@ __device__ __forceinline__ void dcnv4_offset_mask_grad_tiled_body(const DcnLaunc
   __syncthreads();
 
   uint32_t reach_needed = 0;
-  float reach_f = 0.f;
+  uint32_t reach_bits = 0;      // bit pattern of the largest distance so far: non-negative floats order like their bits
   if (active) {
     float go[NV][EPV];
 #pragma unroll
@@ -549,7 +549,8 @@ __device__ __forceinline__ void dcnv4_offset_mask_grad_tiled_body(const DcnLaunc
     elem_t *om = s_om + unit * 3 * Kp;
     const int zero_base = t.wh * t.ww * cell_stride, row_bytes = t.ww * cell_stride;
     const int lane_bytes = gl * p.D * Tag::kBytes + part * NV * 16;
-    const bool pair = p.gt_lpg == 2;       // the two lanes of a (pixel, group) add their halves of each dot product
+    // the two lanes of a (pixel, group) add their halves of each dot product (known at compile time for the 3x3 instantiations)
+    const bool pair = KP > 0 ? PAIR : p.gt_lpg == 2;
     typedef typename std::conditional<(KP > 0), uint32_t, uint64_t>::type mask_t;
     mask_t far_mask = 0;
     // softmax over the group's modulation logits (KP == 0 only): statistics before the slots turn into gradients;
@@ -597,7 +598,7 @@ __device__ __forceinline__ void dcnv4_offset_mask_grad_tiled_body(const DcnLaunc
       // the 2x2 block lie from it at most (a point at an integer distance k has its far corners at weight 0)
       // (points beyond the cap are not `ok` - the cap exceeds what any window covers - and are folded where they are served)
       const float dist = fmaxf(fabsf(x - p0xf), fabsf(y - p0yf));
-      if (wt.inside && dist <= p.gv_reach_cap) reach_f = fmaxf(reach_f, dist);
+      reach_bits = max(reach_bits, (wt.inside && dist <= p.gv_reach_cap) ? __builtin_bit_cast(uint32_t, dist) : 0u);
       u32x4 raw[4][NV];
 #pragma unroll
       for (int cn = 0; cn < 4; ++cn) {
@@ -685,7 +686,7 @@ __device__ __forceinline__ void dcnv4_offset_mask_grad_tiled_body(const DcnLaunc
       const WinTap wt = window_tap(y, x, p.H, p.W, t, cell_stride, lane_bytes - part_bytes, zero_base);
       const int far_own = wt.inside && !wt.ok;
       const float dist = fmaxf(fabsf(x - p0xf), fabsf(y - p0yf));
-      if (wt.inside && dist <= p.gv_reach_cap) reach_f = fmaxf(reach_f, dist);
+      reach_bits = max(reach_bits, (wt.inside && dist <= p.gv_reach_cap) ? __builtin_bit_cast(uint32_t, dist) : 0u);
       far_mask |= ((mask_t)pair_pick<0>(far_own) << k0) | ((mask_t)pair_pick<1>(far_own) << (k0 + 1));
       float d0[4], d1[4], d[4];
       window_dots(pair_pick<0>(wt.addr) + part_bytes, d0);
@@ -774,7 +775,7 @@ __device__ __forceinline__ void dcnv4_offset_mask_grad_tiled_body(const DcnLaunc
 
   // the reach the grad_value kernel has to cover: fold in LDS, then touch the global word only when it would grow
   // (same-address global atomics retire slowly)
-  reach_needed = wave_max_u32((uint32_t)min(ceilf(reach_f), 1048576.f));
+  reach_needed = wave_max_u32((uint32_t)min(ceilf(__builtin_bit_cast(float, reach_bits)), 1048576.f));
   if ((threadIdx.x & (kWave - 1)) == 0 && reach_needed != 0) atomicMax(&s_reach, reach_needed);
   __syncthreads();
   if (threadIdx.x == 0) {
