@@ -71,15 +71,15 @@ MEASURED_TRAFFIC_BYTES = {
     "dcnv4_fwd:T-stage2:float16": 47.5e6,      # algorithmic 47.4e6
     "dcnv4_bwd:T-stage2:float16": 116.8e6,     # algorithmic 81.9e6
     "dcnv4_fwd:T-stage3:float16": 23.8e6,      # algorithmic 23.7e6
-    "dcnv4_bwd:T-stage3:float16": 51.3e6,      # algorithmic 40.9e6
+    "dcnv4_bwd:T-stage3:float16": 51.5e6,      # algorithmic 40.9e6
     "dcnv4_fwd:T-stage4:float16": 12.0e6,      # algorithmic 11.8e6
     "dcnv4_bwd:T-stage4:float16": 23.0e6,      # algorithmic 20.5e6
     "dcnv4_fwd:T-stage1:float32": 192.8e6,     # algorithmic 192.7e6
-    "dcnv4_bwd:T-stage1:float32": 551.1e6,     # algorithmic 334.0e6
+    "dcnv4_bwd:T-stage1:float32": 550.1e6,     # algorithmic 334.0e6
     "dcnv4_fwd:T-stage2:float32": 94.9e6,      # algorithmic 94.7e6
-    "dcnv4_bwd:T-stage2:float32": 262.8e6,     # algorithmic 163.8e6
+    "dcnv4_bwd:T-stage2:float32": 262.7e6,     # algorithmic 163.8e6
     "dcnv4_fwd:T-stage3:float32": 47.5e6,      # algorithmic 47.4e6
-    "dcnv4_bwd:T-stage3:float32": 121.0e6,     # algorithmic 81.9e6
+    "dcnv4_bwd:T-stage3:float32": 121.4e6,     # algorithmic 81.9e6
     "dcnv4_fwd:T-stage4:float32": 23.9e6,      # algorithmic 23.7e6
     "dcnv4_bwd:T-stage4:float32": 45.1e6,      # algorithmic 40.9e6
 }
