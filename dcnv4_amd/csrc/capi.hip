@@ -509,14 +509,12 @@ void fda_choose_order(FdaLaunch *F, const FdaProblem &pr, int N, int G, int D, i
   // The workgroups of a launch - one per CU, 1024 lanes and most of the LDS each - should pass over the chip in two
   // even rounds: measured on 128x128.. and 100x151.. pyramids (4 images, 8 heads of 32 fp16 channels), two rounds
   // take 0.158 / 0.135 ms against 0.180 / 0.165 ms without staging, while counts that leave a partial last round
-  // or more rounds (every workgroup stages the levels again) lose the gain.  With few sampling points per workgroup
-  // (under 16 K: 1024 queries of 4 levels x 4 points, or 512 of 4 x 8 - 100x152.. pyramid, 2 images, 8 points:
-  // 0.159 -> 0.142 ms staged), or heads wider than 64 bytes (half as many pixels fit), staging costs more than the
-  // LDS reads save.
+  // or more rounds (every workgroup stages the levels again) lose the gain.  With few queries per workgroup, or
+  // heads wider than 64 bytes (half as many pixels fit), staging costs more than the LDS reads save.
   const int pairs = (int)(F->n_row / F->Q) * G;
   const int sub_q = kFdaStagedThreads / width;
   const int blocks = std::max(1, 2 * kCusPerDevice / std::max(1, pairs));
-  const bool pays = head_bytes <= 64 && (long long)F->Q * L * K >= (long long)blocks * 1024 * 16;
+  const bool pays = head_bytes <= 64 && (long long)F->Q >= (long long)blocks * 1024;
   if (g_opt.fda_stage != kOptTiled && !(pyramid_fits && pays)) return;
   F->stage_budget = (int)(budget & ~size_t(15));
   F->stage_blocks = std::max(1, std::min(blocks, (F->Q + sub_q - 1) / sub_q));
