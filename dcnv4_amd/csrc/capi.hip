@@ -482,40 +482,57 @@ int fda_prepare(FdaProblem *pr, bool backward, bool scatter, int dtype, int batc
   return DCNV4_OK;
 }
 
-// One head per workgroup, workgroups ordered [image][head][block of queries], when a head's slice of a value image
-// fits an XCD's L2 and the whole image does not: the gathers then hit L2.  A workgroup takes as many queries as fill
-// it with one head's lanes (and fit the LDS).
+// One head per workgroup, workgroups ordered [image][head][block of queries], when the whole value image does not fit
+// an XCD's L2 with room to spare: an XCD then gathers from one head's slice of it at a time.  In the forward also when
+// that slice alone exceeds the L2 - it is still an n-th of what the query-row order gathers from (4 images of
+// 128x128.., 8 heads of 64 fp32 channels: 0.895 -> 0.453 ms; 100x152.., 2 images: 0.401 -> 0.218 ms).  A workgroup
+// takes as many queries as fill it with one head's lanes (and fit the LDS).
 void fda_choose_order(FdaLaunch *F, const FdaProblem &pr, int N, int G, int D, int L, int K, bool backward) {
   const size_t line = 128, head_bytes = (size_t)D * pr.s;
   const size_t lines_per_pixel = (std::max(head_bytes, line) + line - 1) / line;      // cache lines a head touches per pixel
   const size_t head_footprint = (size_t)N * lines_per_pixel * line;
   F->head_major = 0;
   if (g_opt.fda_order == 1 || G <= 1) return;
-  if (g_opt.fda_order != 2 && (pr.img_elems * pr.s <= kL2BytesPerXcd / 2 || head_footprint > kL2BytesPerXcd)) return;
+  if (g_opt.fda_order != 2 && (pr.img_elems * pr.s <= kL2BytesPerXcd / 2 || (backward && head_footprint > kL2BytesPerXcd))) return;
   F->head_major = 1;
   const int width = 1 << F->lanes.tpgp_log2;
   const size_t lds_per_row = (size_t)3 * L * K * sizeof(float) * (backward ? 2 : 1);
   F->nq_block = std::max(1, std::min((backward ? kFdaBackwardThreads : kFdaForwardThreads) / width, (int)(kMaxDynamicLds / lds_per_row)));
   // Forward: the smallest levels of the head's value slice in LDS.  The level shapes live in device memory, so the
-  // choice goes by what a pyramid with a factor of two between levels would need: its last two levels hold about
-  // 5.9 % of the pixels (6.5 % asked for).  The kernel stages whatever really fits; with nothing staged it only runs
-  // at lower occupancy.
+  // choice goes by what a pyramid with a factor of two between levels would need: its last level holds about 1.2 %
+  // of the pixels (1.5 % asked for).  The kernel stages whatever really fits; with nothing staged it only runs at
+  // lower occupancy.
   F->stage_budget = 0;
   if (backward || g_opt.fda_stage == kOptPlain || (head_bytes % 16) != 0 || width > 64) return;
   const size_t rows_bytes = (size_t)(kFdaStagedThreads / width) * lds_per_row;
   if (rows_bytes + 4096 > kMaxLdsPerWorkgroup - 2048) return;
   const size_t budget = std::min<size_t>(kMaxLdsPerWorkgroup - 2048 - rows_bytes, 112 * 1024);
-  const bool pyramid_fits = L >= 3 && (size_t)N * head_bytes * 13 / 200 + fda_staged_zero_bytes((int)head_bytes) <= budget;
-  // The workgroups of a launch - one per CU, 1024 lanes and most of the LDS each - should pass over the chip in two
-  // even rounds: measured on 128x128.. and 100x151.. pyramids (4 images, 8 heads of 32 fp16 channels), two rounds
-  // take 0.158 / 0.135 ms against 0.180 / 0.165 ms without staging, while counts that leave a partial last round
-  // or more rounds (every workgroup stages the levels again) lose the gain.  With few queries per workgroup, or
-  // heads wider than 64 bytes (half as many pixels fit), staging costs more than the LDS reads save.
+  const bool level_fits = L >= 2 && (size_t)N * head_bytes * 3 / 200 + fda_staged_zero_bytes((int)head_bytes) <= budget;
+  // The workgroups of a launch - one per CU, 1024 lanes and most of the LDS each - pass over the chip in two even
+  // rounds (other counts leave a partial last round, or stage the levels more often).  Measured forward times,
+  // staged against one head per workgroup without staging, 8 heads of 32 channels, fp16 / fp32:
+  //   128x128.. 4 levels x 4 points, 4 images  0.142 / 0.294 against 0.172 / 0.215 ms
+  //   128x128.. 4 x 8, 4 images                0.309 / 0.519 against 0.327 / 0.393
+  //   100x152.. 4 x 8, 2 images                0.141 / 0.169 against 0.158 / 0.185;  8 images 0.678 / 1.09 against 0.573 / 0.694
+  //   64x64.. 4 x 8, 8 images                  0.124 / 0.158 against 0.139 / 0.193;  80x80.. 3 x 8, 4 images 0.095 / 0.119 against 0.105 / 0.127
+  //   one image (64 workgroups per head, 1.2 rounds of queries each): 2-5 % slower staged
+  //   heads of 128 bytes and more with 4 x 4 points: 3-27 % slower staged (100x152.., 2 images, 64 fp16 channels: 0.110
+  //   against 0.099 ms); heads of 16 fp32 channels: 15-27 % faster staged on four shapes, 9 % slower on 128x128.. 4 x 8
+  // What decides is the L2: the 32 workgroups that an XCD runs at a time belong to 32 / (workgroups per head)
+  // consecutive heads, whose slices of the value image (heads of one pixel share 128-byte lines) must stay in its
+  // 4 MB together - and every workgroup needs at least two rounds of queries, or the rounds do not divide evenly.
+  // Wide heads gain only with long rows (24 points and more per query and head: 80x80.. 3 x 8, 32 fp32 channels
+  // 0.119 against 0.128 ms).
   const int pairs = (int)(F->n_row / F->Q) * G;
   const int sub_q = kFdaStagedThreads / width;
   const int blocks = std::max(1, 2 * kCusPerDevice / std::max(1, pairs));
-  const bool pays = head_bytes <= 64 && (long long)F->Q >= (long long)blocks * 1024;
-  if (g_opt.fda_stage != kOptTiled && !(pyramid_fits && pays)) return;
+  const int cus_per_xcd = kCusPerDevice / 8;
+  const size_t heads_at_once = (size_t)std::max(1, (cus_per_xcd + blocks - 1) / blocks);
+  const size_t lines_at_once = (heads_at_once * head_bytes + line - 1) / line;
+  const bool l2_holds = (size_t)N * lines_at_once * line <= kL2BytesPerXcd * 3 / 4;
+  const bool rounds_even = (long long)(F->Q + sub_q - 1) / sub_q >= 2LL * blocks;
+  const bool width_pays = head_bytes <= 64 || L * K >= 24;
+  if (g_opt.fda_stage != kOptTiled && !(level_fits && l2_holds && rounds_even && width_pays)) return;
   F->stage_budget = (int)(budget & ~size_t(15));
   F->stage_blocks = std::max(1, std::min(blocks, (F->Q + sub_q - 1) / sub_q));
 }
