@@ -212,10 +212,12 @@ constexpr int kDefaultReach = 5;
 
 int reach_setting() { return g_opt.reach < 0 ? kDefaultReach : std::min(g_opt.reach, 64); }
 
-// Flash attention backward: head widths the tiled grad_value kernel handles (8 lanes x up to 4 channels,
-// whole 8-channel blocks), with point counts that fit its 32-bit point ids.
+// Flash attention backward: head widths the tiled grad_value kernel handles (whole 8-channel blocks; a launch
+// accumulates up to 32 channels - 8 lanes x 4 - and wider heads take a launch per window of 32 over the same point
+// records and lists), with point counts that fit its 32-bit point ids.
+constexpr int kFdaWindowChannels = 32;
 bool fda_tiled_shape(int D, int L, int Q, int K) {
-  return D % 8 == 0 && D <= 32 && L >= 1 && K >= 1 && (long long)Q * K < (1ll << 31);
+  return D % 8 == 0 && D <= 4 * kFdaWindowChannels && L >= 1 && K >= 1 && (long long)Q * K < (1ll << 31);
 }
 
 constexpr size_t kL2BytesPerXcd = 4u << 20;
@@ -458,7 +460,13 @@ int fda_prepare(FdaProblem *pr, bool backward, bool scatter, int dtype, int batc
 
   FdaLaunch &F = pr->launch;
   F = FdaLaunch{};
-  if (int rc = choose_lanes(D, s, d_stride, scatter, &F.lanes)) return rc;
+  // The gather kernels (forward, and the backward in front of the tiled grad_value kernel) take 16-byte lanes whatever
+  // the hint: a reference-style d_stride of 1 or 2 would cost them 25-180 % (cfg 4, fp16: forward 0.146 -> 0.233 / 0.407
+  // ms, backward 0.584 -> 0.728 / 1.039 ms).  The hint is still checked, and narrows the lanes of the atomic scatter.
+  LaneMap hinted;
+  if (int rc = choose_lanes(D, s, d_stride, scatter, &hinted)) return rc;
+  if (scatter) F.lanes = hinted;
+  else if (int rc = choose_lanes(D, s, 0, false, &F.lanes)) return rc;
   const int width = 1 << F.lanes.tpgp_log2;
   if (backward && width > kWave)
     return fail(DCNV4_ERR_INVALID_ARGUMENT, "backward needs head_channels/%d <= 64 lanes per head, got %d",
@@ -1026,12 +1034,17 @@ static int fda_backward_impl(const void *value, const int64_t *spatial_shapes, c
         if (pass == 0) fda_choose_order(&F, pr, spatial_size, num_heads, head_channels, num_levels, num_points, true);
         F.clear_state = (pass == 0 && b0 == 0) ? 1 : 0;
         if (pass == 0) e = launch_fda_backward(dtype, F, kFdaNoScatter, st);
-        else if (pass == 1) e = launch_fda_grad_value(dtype, F, st);
-        else {
+        else if (pass == 1) {
+          for (int c0 = 0; c0 < head_channels && e == hipSuccess; c0 += kFdaWindowChannels) {
+            F.gv_c0 = c0;
+            F.gv_dc = std::min(kFdaWindowChannels, head_channels - c0);
+            e = launch_fda_grad_value(dtype, F, st);
+          }
+        } else {
           // The fallback sums with fp32 atomics: straight into grad_value for fp32 tensors (the tiled kernel has left
           // it zeroed), for 16-bit tensors into an fp32 image that takes the place of the - by now dead - keys and
           // records, is cleared first and narrowed afterwards; all three launches return at once without the flag.
-          const size_t n = (size_t)nb * pr.img_elems;      // a multiple of 8: heads of 8, 16, 24 or 32 channels
+          const size_t n = (size_t)nb * pr.img_elems;      // a multiple of 8: heads of whole 8-channel blocks
           float *acc = pr.s == 2 ? reinterpret_cast<float *>(ws + kStateBytes) + (size_t)b0 * pr.img_elems : static_cast<float *>(F.grad_value);
           F.grad_value_acc = acc;
           const dim3 grid((unsigned)std::min<size_t>((n / 8 + 255) / 256, 4096)), block(256);

@@ -239,7 +239,9 @@ __global__ void __launch_bounds__(kTileCells * LPC * SUBS) fda_grad_value_kernel
   constexpr int DP = CW * kCellLanes;
   constexpr int kParkBytes = Tag::kBytes;
   constexpr int kGoStride = (((DP * kParkBytes + 15) / 16) | 1) * 16;     // an odd number of 16-byte units per parked row
-  const int D = p.D, QK = p.Q * p.K;
+  // D: the head's channels in memory; this launch accumulates the window [c0, c0 + Dc) of them (heads wider than 32
+  // channels take several launches over the same records and lists)
+  const int D = p.D, c0 = p.gv_c0, Dc = p.gv_dc, QK = p.Q * p.K;
   uint32_t *s_count = lds32;                                  // [kTileCells] entries per cell in this batch
   uint32_t *s_offs = s_count + kTileCells;                    // [kTileCells + 4] first entry of every cell, then the total
   uint32_t *s_list = s_offs + kTileCells + 4;                 // [kListCap] listed point ids
@@ -267,8 +269,8 @@ __global__ void __launch_bounds__(kTileCells * LPC * SUBS) fda_grad_value_kernel
   const int BG = p.n_img * p.G;
 
   // value rows that no level covers (spatial_size beyond the levels, gaps between them) get zeros, like the
-  // reference's zeros_like(value) (flash_deform_attn_cuda.cu:118)
-  {
+  // reference's zeros_like(value) (flash_deform_attn_cuda.cu:118); whole rows, by the launch of the first window
+  if (c0 == 0) {
     const long long rows = (long long)p.n_img * p.N;
     const int row_elems = p.G * p.D;
     for (long long r = (long long)blockIdx.x * kApplyThreads + tid; r < rows; r += (long long)gridDim.x * kApplyThreads) {
@@ -350,9 +352,9 @@ __global__ void __launch_bounds__(kTileCells * LPC * SUBS) fda_grad_value_kernel
 #pragma unroll
       for (int u = 0; u < kRowsPerLane; ++u) {
         const int h = my_slot + u * kRowStep;
-        const bool live = h < nb && my_part * CW < D;
+        const bool live = h < nb && my_part * CW < Dc;
         const uint32_t q = s_list[min((int)b0 + min(h, max(nb - 1, 0)), kListCap - 1)] / (uint32_t)p.K;
-        a.go[u] = buffer_load<CW * Tag::kBytes>(go_rs, live ? (q * (uint32_t)D + (uint32_t)(my_part * CW)) * Tag::kBytes : kDropOffset);
+        a.go[u] = buffer_load<CW * Tag::kBytes>(go_rs, live ? (q * (uint32_t)D + (uint32_t)(c0 + my_part * CW)) * Tag::kBytes : kDropOffset);
       }
       return a;
     };
@@ -516,13 +518,13 @@ __global__ void __launch_bounds__(kTileCells * LPC * SUBS) fda_grad_value_kernel
       const int cy = my_cell / tw, cx = my_cell - cy * tw;
       const long long n = (long long)lp.start + (long long)(ty0 + cy) * lp.W + tx0 + cx;      // level tables are not validated
       if (n >= 0 && n < p.N) {
-        elem_t *dst = reinterpret_cast<elem_t *>(p.grad_value) + (((size_t)b * p.N + (size_t)n) * p.G + g) * D + my_part * CW;
-        if ((D % CW) == 0 && (CW * Tag::kBytes) % 4 == 0) {
-          if (my_part * CW < D) __builtin_nontemporal_store(Pack<Tag, CW>::encode(acc), reinterpret_cast<goN_t *>(dst));
+        elem_t *dst = reinterpret_cast<elem_t *>(p.grad_value) + (((size_t)b * p.N + (size_t)n) * p.G + g) * D + c0 + my_part * CW;
+        if ((D % CW) == 0 && (Dc % CW) == 0 && (CW * Tag::kBytes) % 4 == 0) {
+          if (my_part * CW < Dc) __builtin_nontemporal_store(Pack<Tag, CW>::encode(acc), reinterpret_cast<goN_t *>(dst));
         } else {
 #pragma unroll
           for (int c = 0; c < CW; ++c)
-            if (my_part * CW + c < D) { const float f[1] = {acc[c]}; dst[c] = Pack<Tag, 1>::encode(f); }
+            if (my_part * CW + c < Dc) { const float f[1] = {acc[c]}; dst[c] = Pack<Tag, 1>::encode(f); }
         }
       }
     }
@@ -535,9 +537,11 @@ int fda_sub_lists_for(int) { return kSubLists; }
 
 template <typename Tag>
 hipError_t launch_t(const FdaLaunch &p, hipStream_t stream) {
-  // binning: one workgroup per chunk of every (image, head, level)
-  hipLaunchKernelGGL(fda_bin_points_kernel<Tag>, dim3((unsigned)(p.n_img * p.G * p.L * p.n_chunks)), dim3(kBinThreads), 0, stream, p);
-  if (hipError_t e = hipGetLastError()) return e;
+  // binning: one workgroup per chunk of every (image, head, level); once, in front of the first channel window
+  if (p.gv_c0 == 0) {
+    hipLaunchKernelGGL(fda_bin_points_kernel<Tag>, dim3((unsigned)(p.n_img * p.G * p.L * p.n_chunks)), dim3(kBinThreads), 0, stream, p);
+    if (hipError_t e = hipGetLastError()) return e;
+  }
 
   int dev = 0, cus = 256;
   if (hipGetDevice(&dev) == hipSuccess) {
@@ -545,7 +549,7 @@ hipError_t launch_t(const FdaLaunch &p, hipStream_t stream) {
     if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
   }
   const size_t lds = fda_grad_value_lds_bytes(p, Tag::kBytes);
-  const int lpc = fda_cell_lanes(p.D, Tag::kBytes), cw = fda_padded_channels(p.D) / lpc;
+  const int lpc = fda_cell_lanes(p.gv_dc, Tag::kBytes), cw = fda_padded_channels(p.gv_dc) / lpc;
   const int subs = fda_sub_lists_for(lpc);
   const int threads = kTileCells * lpc * subs;
   // persistent workgroups: as many per CU as LDS and wave slots (32 per CU) allow
@@ -577,12 +581,12 @@ hipError_t launch_t(const FdaLaunch &p, hipStream_t stream) {
 }  // namespace
 
 size_t fda_grad_value_lds_bytes(const FdaLaunch &p, int elem_bytes) {
-  const size_t go_stride = ((((size_t)fda_padded_channels(p.D) * elem_bytes + 15) / 16) | 1) * 16;
+  const size_t go_stride = ((((size_t)fda_padded_channels(p.gv_dc) * elem_bytes + 15) / 16) | 1) * 16;
   const size_t head = ((size_t)2 * kTileCells + 4) * sizeof(uint32_t);
   const size_t batch = head + ((size_t)kListCap + 2 * kTabCap + 4) * sizeof(uint32_t) + ((size_t)4 * kBatch + 2) * sizeof(u32x2) +
                        (size_t)(kBatch + 1) * go_stride;
   // the sub-lists' partial sums meet in LDS behind the counters: a float per lane and channel it holds
-  const size_t meet = head + (size_t)kTileCells * kSubLists * fda_padded_channels(p.D) * sizeof(float);
+  const size_t meet = head + (size_t)kTileCells * kSubLists * fda_padded_channels(p.gv_dc) * sizeof(float);
   return std::max(batch, meet);
 }
 

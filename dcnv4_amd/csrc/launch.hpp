@@ -171,6 +171,7 @@ struct FdaLaunch {
   int n_chunks;             // chunks of kFdaChunkPoints points per (image, head, level)
   int tile_stride;          // table row length: an upper bound of the tiles of one level
   int n_img;
+  int gv_c0, gv_dc;         // tiled grad_value kernel: the window [gv_c0, gv_c0 + gv_dc) of a head's channels this launch accumulates (at most 32)
 };
 
 // Key of a sampling point: (y0 + 1) << 8 | (x0 + 1) for the integer position (y0, x0) of its first

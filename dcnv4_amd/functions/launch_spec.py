@@ -50,8 +50,9 @@ def _vector_channels(group_channels, elem_bytes):
 
 
 def _spec(group, group_channels, elem_bytes, scatter=False):
-    # backward scatters with one channel per lane (contiguous dwords per atomic instruction)
-    d_stride = 1 if scatter and group_channels <= 64 else _vector_channels(group_channels, elem_bytes)
+    # forward and backward gather with 16-byte lanes (grad_value is a gather too); `scatter` is kept for callers that
+    # name the direction
+    d_stride = _vector_channels(group_channels, elem_bytes)
     lanes_per_group = 1
     while lanes_per_group < group_channels // d_stride:
         lanes_per_group *= 2

@@ -154,7 +154,7 @@ int flash_deform_attn_gfx950_forward(const void *value, const int64_t *spatial_s
 
 /*
  * Bytes of device scratch flash_deform_attn_gfx950_backward needs for this problem (16-byte aligned;
- * contents need no initialisation).  Head widths that are multiples of 8 up to 32 take about 34 bytes
+ * contents need no initialisation).  Head widths that are multiples of 8 up to 128 take about 34 bytes
  * per sampling point (a key, a position-and-probability record, and list space for binning the points by
  * tile) plus grad_output once more and a tile table; other widths take an fp32 image of value for 16-bit
  * tensors.  The reference allocates its fp32 gradient buffers itself

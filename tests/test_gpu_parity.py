@@ -245,6 +245,11 @@ def test_flash_deform_attn_forward_and_backward_match_oracle(oracle, name, dtype
 FDA_PATH_CASES = {
     # head width 24 pads to 32 accumulator channels in the tiled grad_value kernel
     "d24_three_levels": (2, [(12, 20), (6, 10), (3, 5)], 3, 24, 4, 90, (-0.2, 1.2)),
+    # heads wider than 32 channels: the tiled grad_value kernel runs once per window of 32 channels over the same
+    # records and lists - two whole windows, a window of 8 behind one of 32, four windows
+    "d64_three_levels": (2, [(14, 18), (7, 9), (4, 5)], 3, 64, 4, 120, (-0.1, 1.1)),
+    "d40_two_windows": (1, [(10, 12), (5, 6)], 2, 40, 8, 70, (0.0, 1.0)),
+    "d128_four_windows": (1, [(9, 8), (5, 4)], 2, 128, 4, 60, (0.0, 1.0)),
     # 6000 queries x 8 points on a 3x3 level: every tile collects far more points than one batch, the list is flushed repeatedly
     "crowded_small_level": (1, [(3, 3), (20, 17)], 2, 16, 8, 6000, (0.0, 1.0)),
     # a level wider than the 16-bit fields of a key: the scan recomputes those positions

@@ -84,7 +84,9 @@ def test_launch_hints_are_well_formed(G, C, es):
         while lanes < C // d_stride:
             lanes *= 2
         assert n_thread % (G * lanes) == 0 and n_thread >= G * lanes
-    assert ls.find_spec_bwd(64, 56, 56, G, C, es)[0] == 1      # scatter layout: one channel per lane
+    # the backward gathers as well (grad_value is a gather): the same 16-byte lanes as the forward, never a narrowing hint
+    assert ls.find_spec_bwd(64, 56, 56, G, C, es) == ls.findspec(64, 56, 56, G, C, es)
+    assert ls.findspec_attn_bwd(4, 21760, G, C, es) == ls.findspec_attn(4, 21760, G, C, es)
 
 
 def test_dcnv4_module_keeps_the_reference_parameter_schema():
