@@ -222,6 +222,8 @@ FDA_CASES = {
     "d6_heads5": (1, [(6, 6), (3, 3)], 5, 6, 4, 11, (0.0, 1.0)),
     "d64_two_levels": (1, [(9, 9), (5, 5)], 4, 64, 4, 33, (0.0, 1.0)),
     "one_query": (1, [(4, 4)], 1, 32, 4, 1, (0.0, 1.0)),
+    # a decoder's few queries against an encoder's pyramid: with fp32 tensors the backward takes the atomic scatter by itself
+    "decoder_few_queries": (2, [(20, 30), (10, 15)], 4, 32, 4, 12, (0.0, 1.0)),
 }
 
 
