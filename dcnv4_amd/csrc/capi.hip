@@ -536,12 +536,24 @@ void fda_choose_order(FdaLaunch *F, const FdaProblem &pr, int N, int G, int D, i
   // 0.119 against 0.128 ms).
   const int pairs = (int)(F->n_row / F->Q) * G;
   const int sub_q = kFdaStagedThreads / width;
-  const int blocks = std::max(1, 2 * kCusPerDevice / std::max(1, pairs));
   const int cus_per_xcd = kCusPerDevice / 8;
-  const size_t heads_at_once = (size_t)std::max(1, (cus_per_xcd + blocks - 1) / blocks);
-  const size_t lines_at_once = (heads_at_once * head_bytes + line - 1) / line;
-  const bool l2_holds = (size_t)N * lines_at_once * line <= kL2BytesPerXcd * 3 / 4;
-  const bool rounds_even = (long long)(F->Q + sub_q - 1) / sub_q >= 2LL * blocks;
+  // Two rounds when the L2 then holds the heads an XCD works on; else twice, four or eight times as many workgroups (more
+  // rounds, each workgroup staging again, but fewer heads at a time: 8 images of 100x152.., 4 x 4 points, fp16: 0.302 ms
+  // plain, 0.306 ms staged in two rounds, 0.268 ms in four; 16 images of 128x128..: 0.644 / 0.936 / 0.605 ms in eight).
+  int blocks = 0;
+  bool l2_holds = false, rounds_even = false;
+  // (heads of 128 bytes lose 12-13 % when staged in more than two rounds; so do small pyramids, whose head slices the
+  // plain kernel's L2 holds several of anyway: 16 images of 80x80.., 0.193 ms plain against 0.232 ms staged in four rounds)
+  const int max_mul = head_bytes <= 64 && (size_t)N * line >= kL2BytesPerXcd / 2 ? 8 : 1;
+  for (int mul = 1; mul <= max_mul && !(l2_holds && rounds_even); mul *= 2) {
+    blocks = std::max(1, 2 * kCusPerDevice / std::max(1, pairs)) * mul;
+    const size_t heads_at_once = (size_t)std::max(1, (cus_per_xcd + blocks - 1) / blocks);
+    const size_t lines_at_once = (heads_at_once * head_bytes + line - 1) / line;
+    l2_holds = (size_t)N * lines_at_once * line <= kL2BytesPerXcd * 3 / 4;
+    rounds_even = (long long)(F->Q + sub_q - 1) / sub_q >= 2LL * blocks;
+    if (!rounds_even) break;      // more workgroups only shorten the rounds further
+  }
+  if (!(l2_holds && rounds_even)) blocks = std::max(1, 2 * kCusPerDevice / std::max(1, pairs));      // what a forced staging launches
   const bool width_pays = head_bytes <= 64 || L * K >= 24;
   if (g_opt.fda_stage != kOptTiled && !(level_fits && l2_holds && rounds_even && width_pays)) return;
   F->stage_budget = (int)(budget & ~size_t(15));
