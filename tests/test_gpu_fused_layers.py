@@ -140,7 +140,8 @@ def test_center_feature_function_takes_parameters_that_are_views_into_a_flat_buf
 # ---------------------------------------------------------------- attention on un-packed rows
 @pytest.mark.parametrize("loc_fp32", [True, False], ids=["loc_fp32", "loc_like_value"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
-@pytest.mark.parametrize("name", ["detr_small_4lvl_k4", "k8_one_level", "five_levels", "k3_generic_points", "d6_heads5", "one_query"])
+@pytest.mark.parametrize("name", ["detr_small_4lvl_k4", "k8_one_level", "five_levels", "k3_generic_points", "d6_heads5", "one_query",
+                                  "d64_two_levels", "decoder_few_queries"])
 def test_flash_deform_attn_split_rows_match_oracle_on_fp16_rounded_locations(oracle, name, dtype, loc_fp32):
     """The oracle sees what the reference's module would have packed: locations rounded to fp16, then the logits
     (DCNv4_op/DCNv4/modules/flash_deform_attn.py:132-133)."""
