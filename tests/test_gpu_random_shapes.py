@@ -46,6 +46,15 @@ def test_dcnv4_random_shapes_match_oracle(oracle, seed, dtype):
     cabi.assert_close(out, want, *FWD_TOL[dtype], what="output")
     cabi.assert_close(gv, wgv, *GRAD_TOL[dtype], what="grad_value")
     cabi.assert_close(gom, wgom, *GRAD_TOL[dtype], what="grad_offset_mask")
+    if seed % 2 == 0:       # every other shape also with the softmax over a group's modulation scalars
+        want = oracle.dcnv4_forward(cabi.f64(v), cabi.f64(om), *args, softmax=True, coord_f32=True)
+        wgv, wgom = oracle.dcnv4_backward(cabi.f64(v), cabi.f64(om), cabi.f64(go), *args, softmax=True, coord_f32=True)
+        out = cabi.dcnv4_forward(v.cuda(), om.cuda(), geom, G, D, scale, rc, softmax=1)
+        gv, gom = cabi.dcnv4_backward(v.cuda(), om.cuda(), go.cuda(), geom, G, D, scale, rc, softmax=1)
+        torch.cuda.synchronize()
+        cabi.assert_close(out, want, *FWD_TOL[dtype], what="output, softmax")
+        cabi.assert_close(gv, wgv, *GRAD_TOL[dtype], what="grad_value, softmax")
+        cabi.assert_close(gom, wgom, *GRAD_TOL[dtype], what="grad_offset_mask, softmax")
 
 
 def _random_fda_case(rnd):
@@ -56,7 +65,7 @@ def _random_fda_case(rnd):
         K = rnd.choice([4, 4, 8, 2, 3])
         if L * K > 32:
             continue
-        G, D = rnd.choice([1, 2, 4, 8, 8, 3]), rnd.choice([8, 16, 32, 32, 32, 64, 24])
+        G, D = rnd.choice([1, 2, 4, 8, 8, 3]), rnd.choice([8, 16, 32, 32, 32, 64, 24, 40, 96, 128])
         Q = rnd.choice([None, None, rnd.randint(1, 3000)])
         return rnd.randint(1, 3), shapes, G, D, K, Q, rnd.choice([(0.0, 1.0), (-0.2, 1.2), (0.3, 0.7)])
 
